@@ -1,0 +1,41 @@
+// Error text storage and checks shared by every entry point.
+#include "common.h"
+
+#include <stdarg.h>
+
+namespace pace_kv {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int check_pool(const pace_kv_pool_t* pool, const char* who) {
+  PACE_REQUIRE(pool != nullptr, "%s: pool is NULL", who);
+  PACE_REQUIRE(pool->k != nullptr && pool->v != nullptr, "%s: pool has a NULL K or V pointer", who);
+  PACE_REQUIRE(pool->block_size == PACE_KV_BLOCK_TOKENS, "%s: block_size %d unsupported (must be %d)", who,
+               pool->block_size, PACE_KV_BLOCK_TOKENS);
+  PACE_REQUIRE(pool->head_dim == 64 || pool->head_dim == 128, "%s: head_dim %d unsupported (64 or 128)", who,
+               pool->head_dim);
+  PACE_REQUIRE(pool->num_blocks > 0 && pool->num_kv_heads > 0, "%s: empty pool (%d blocks, %d heads)", who,
+               pool->num_blocks, pool->num_kv_heads);
+  const int64_t slab = (int64_t)pool->block_size * pool->head_dim;
+  PACE_REQUIRE(pool->k_head_stride >= slab && pool->v_head_stride >= slab, "%s: head stride smaller than a slab", who);
+  PACE_REQUIRE(pool->k_block_stride >= pool->k_head_stride && pool->v_block_stride >= pool->v_head_stride,
+               "%s: block stride smaller than head stride", who);
+  PACE_REQUIRE((pool->k_head_stride % 8) == 0 && (pool->v_head_stride % 8) == 0 && (pool->k_block_stride % 8) == 0 &&
+                   (pool->v_block_stride % 8) == 0,
+               "%s: pool strides must be multiples of 8 elements (16 bytes)", who);
+  PACE_REQUIRE(aligned16(pool->k) && aligned16(pool->v), "%s: pool pointers must be 16-byte aligned", who);
+  return PACE_KV_OK;
+}
+
+}  // namespace pace_kv
+
+extern "C" const char* pace_kv_last_error(void) { return pace_kv::g_error; }
+
+extern "C" int32_t pace_kv_abi_version(void) { return 1; }

@@ -1,0 +1,54 @@
+// Shared helpers for the gfx950 KV-cache kernels: error reporting, bf16 bit
+// helpers and the vector types the matrix-core builtins take.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "pace_kv_hip.h"
+
+namespace pace_kv {
+
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+// Returns PACE_KV_EINVAL from the enclosing entry point with a message.
+#define PACE_REQUIRE(cond, ...)           \
+  do {                                    \
+    if (!(cond)) {                        \
+      ::pace_kv::set_error(__VA_ARGS__);  \
+      return PACE_KV_EINVAL;              \
+    }                                     \
+  } while (0)
+
+#define PACE_HIP_CHECK(expr)                                                      \
+  do {                                                                            \
+    hipError_t e_ = (expr);                                                       \
+    if (e_ != hipSuccess) {                                                       \
+      ::pace_kv::set_error("%s failed: %s", #expr, hipGetErrorString(e_));        \
+      return PACE_KV_EHIP;                                                        \
+    }                                                                             \
+  } while (0)
+
+int check_pool(const pace_kv_pool_t* pool, const char* who);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// Round-to-nearest-even fp32 -> bf16 bits (NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+}  // namespace pace_kv

@@ -1,0 +1,238 @@
+// Pool data movement for gfx950: append by slot, block-table gather, block copy.
+// All three are pure byte movers bounded by HBM bandwidth; every global access
+// is a 16-byte lane access, coalesced over rows of the token-major side.
+#include "common.h"
+
+namespace pace_kv {
+
+// ---------------------------------------------------------------------------------
+// Append.  One thread moves eight dims (16 bytes) of one (token, head) row of K and
+// of V.  K keeps its row shape; V is written dim-major, so its eight values land 32
+// bytes apart (one per dim) at the token's column.
+// ---------------------------------------------------------------------------------
+// Where the tokens go: either an explicit slot id per token, or "position
+// seq_lens[b] + pos_offset + t of sequence b" resolved through the block table.
+struct AppendDest {
+  const int64_t* slots;
+  const int32_t* table;
+  const int32_t* seq_lens;
+  int32_t table_stride;
+  int32_t pos_offset;
+};
+
+template <int D, bool PAGED>
+__global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, const uint16_t* __restrict__ k_new,
+                                                        const uint16_t* __restrict__ v_new, int64_t sb, int64_t sh,
+                                                        int64_t st, int32_t n_tokens, int32_t total_rows,
+                                                        const AppendDest dest) {
+  constexpr int CHUNKS = D / 8;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int chunk = (int)(gid % CHUNKS);
+  const int64_t row = gid / CHUNKS;  // (token i, head h), head fastest
+  if (row >= total_rows) return;
+  const int H = pool.num_kv_heads;
+  const int h = (int)(row % H);
+  const int64_t i = row / H;  // b * n_tokens + t
+  const int64_t b = i / n_tokens, t = i % n_tokens;
+  int64_t blk;
+  int off;
+  if (PAGED) {
+    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + t;
+    if (pos < 0 || pos / PACE_KV_BLOCK_TOKENS >= dest.table_stride) return;
+    blk = dest.table[b * dest.table_stride + pos / PACE_KV_BLOCK_TOKENS];
+    off = (int)(pos % PACE_KV_BLOCK_TOKENS);
+  } else {
+    const int64_t slot = dest.slots[i];
+    if (slot < 0) return;
+    blk = slot / PACE_KV_BLOCK_TOKENS;
+    off = (int)(slot % PACE_KV_BLOCK_TOKENS);
+  }
+  if (blk < 0 || blk >= pool.num_blocks) return;  // never write outside the pool
+  const int64_t src = b * sb + h * sh + t * st + chunk * 8;
+  const u32x4 kv = *reinterpret_cast<const u32x4*>(k_new + src);
+  const u32x4 vv = *reinterpret_cast<const u32x4*>(v_new + src);
+  uint16_t* kdst = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride +
+                   (int64_t)off * D + chunk * 8;
+  *reinterpret_cast<u32x4*>(kdst) = kv;
+  uint16_t* vdst = reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride +
+                   (int64_t)(chunk * 8) * PACE_KV_BLOCK_TOKENS + off;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    vdst[(2 * j) * PACE_KV_BLOCK_TOKENS] = (uint16_t)(vv[j] & 0xffffu);
+    vdst[(2 * j + 1) * PACE_KV_BLOCK_TOKENS] = (uint16_t)(vv[j] >> 16);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Gather.  One 256-thread workgroup rebuilds one logical block (16 tokens) of one KV
+// head of one sequence in the dense [B][H*n_rep][L][D] layout.  K slabs are copied
+// as they are; V slabs are staged in LDS and read back transposed.
+// ---------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
+                                                        int32_t table_stride, const int32_t* __restrict__ seq_lens,
+                                                        int32_t n_rep, uint16_t* __restrict__ k_out,
+                                                        uint16_t* __restrict__ v_out, int64_t osb, int64_t osh,
+                                                        int32_t out_len) {
+  constexpr int CHUNKS = D / 8;                             // 16-byte chunks per row
+  constexpr int SLAB_CHUNKS = PACE_KV_BLOCK_TOKENS * CHUNKS;  // per (block, head)
+  __shared__ uint16_t vt[D * PACE_KV_BLOCK_TOKENS + 8];
+  const int j = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int len = seq_lens[b];
+  const int t0 = j * PACE_KV_BLOCK_TOKENS;
+  const bool live = t0 < len;  // uniform per workgroup
+  int64_t blk = 0;
+  if (live) blk = table[(int64_t)b * table_stride + j];
+  blk = blk < 0 ? 0 : (blk >= pool.num_blocks ? pool.num_blocks - 1 : blk);  // never read outside the pool
+  const uint16_t* ksrc = reinterpret_cast<const uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
+  const uint16_t* vsrc = reinterpret_cast<const uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
+  if (live) {
+    for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x)
+      *reinterpret_cast<u32x4*>(&vt[c * 8]) = *reinterpret_cast<const u32x4*>(vsrc + c * 8);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x) {
+    const int tok = c / CHUNKS, chunk = c % CHUNKS;
+    const int t = t0 + tok;
+    if (t >= out_len) continue;
+    u32x4 kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
+    if (t < len) {
+      kv = *reinterpret_cast<const u32x4*>(ksrc + c * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t lo = vt[(chunk * 8 + 2 * e) * PACE_KV_BLOCK_TOKENS + tok];
+        const uint32_t hi = vt[(chunk * 8 + 2 * e + 1) * PACE_KV_BLOCK_TOKENS + tok];
+        vv[e] = lo | (hi << 16);
+      }
+    }
+    for (int r = 0; r < n_rep; ++r) {
+      const int64_t o = (int64_t)b * osb + (int64_t)(h * n_rep + r) * osh + (int64_t)t * D + chunk * 8;
+      *reinterpret_cast<u32x4*>(k_out + o) = kv;
+      *reinterpret_cast<u32x4*>(v_out + o) = vv;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Block copy.  One workgroup per (pair, head): both slabs of that head, 16 bytes per
+// lane access.  Layout-agnostic (a slab is copied verbatim).
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void kv_copy_blocks_kernel(pace_kv_pool_t src, pace_kv_pool_t dst,
+                                                             const int32_t* __restrict__ pairs) {
+  const int pair = blockIdx.x, h = blockIdx.y;
+  const int64_t s = pairs[2 * pair], d = pairs[2 * pair + 1];
+  if (s < 0 || s >= src.num_blocks || d < 0 || d >= dst.num_blocks) return;  // uniform per workgroup
+  const int slab_chunks = PACE_KV_BLOCK_TOKENS * src.head_dim / 8;
+  const u32x4* ks = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(src.k) + s * src.k_block_stride +
+                                                   h * src.k_head_stride);
+  const u32x4* vs = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(src.v) + s * src.v_block_stride +
+                                                   h * src.v_head_stride);
+  u32x4* kd = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dst.k) + d * dst.k_block_stride + h * dst.k_head_stride);
+  u32x4* vd = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dst.v) + d * dst.v_block_stride + h * dst.v_head_stride);
+  for (int c = threadIdx.x; c < slab_chunks; c += blockDim.x) {
+    const u32x4 a = ks[c];
+    const u32x4 bq = vs[c];
+    kd[c] = a;
+    vd[c] = bq;
+  }
+}
+
+}  // namespace pace_kv
+
+using namespace pace_kv;
+
+static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
+                      int64_t stride_b, int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
+                      const AppendDest& dest, bool paged, void* stream) {
+  if (int rc = check_pool(pool, who)) return rc;
+  PACE_REQUIRE(batch >= 0 && n_tokens >= 0, "%s: negative batch (%d) or n_tokens (%d)", who, batch, n_tokens);
+  if (batch == 0 || n_tokens == 0) return PACE_KV_OK;
+  PACE_REQUIRE(k_new && v_new, "%s: NULL input pointer", who);
+  PACE_REQUIRE(aligned16(k_new) && aligned16(v_new), "%s: k_new / v_new must be 16-byte aligned", who);
+  PACE_REQUIRE(stride_b % 8 == 0 && stride_h % 8 == 0 && stride_t % 8 == 0,
+               "%s: input strides must be multiples of 8 elements", who);
+  const int64_t rows = (int64_t)batch * n_tokens * pool->num_kv_heads;
+  PACE_REQUIRE(rows < (int64_t)1 << 31, "%s: too many rows (%lld)", who, (long long)rows);
+  const int chunks = pool->head_dim / 8;
+  const int64_t threads = rows * chunks;
+  PACE_REQUIRE((threads + 255) / 256 < (int64_t)1 << 31, "%s: grid too large", who);
+  const unsigned grid = (unsigned)((threads + 255) / 256);
+  const uint16_t* k = static_cast<const uint16_t*>(k_new);
+  const uint16_t* v = static_cast<const uint16_t*>(v_new);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define PACE_LAUNCH_APPEND(DIM, PG)                                                                                  \
+  hipLaunchKernelGGL((kv_append_kernel<DIM, PG>), dim3(grid), dim3(256), 0, s, *pool, k, v, stride_b, stride_h, stride_t, \
+                     n_tokens, (int32_t)rows, dest)
+  if (pool->head_dim == 128) {
+    if (paged) PACE_LAUNCH_APPEND(128, true); else PACE_LAUNCH_APPEND(128, false);
+  } else {
+    if (paged) PACE_LAUNCH_APPEND(64, true); else PACE_LAUNCH_APPEND(64, false);
+  }
+#undef PACE_LAUNCH_APPEND
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
+}
+
+extern "C" int pace_kv_append(const pace_kv_pool_t* pool, const void* k_new, const void* v_new, int64_t stride_b,
+                              int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
+                              const int64_t* slot_mapping, void* stream) {
+  if (batch > 0 && n_tokens > 0) PACE_REQUIRE(slot_mapping != nullptr, "pace_kv_append: slot_mapping is NULL");
+  AppendDest dest = {slot_mapping, nullptr, nullptr, 0, 0};
+  return run_append("pace_kv_append", pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest, false,
+                    stream);
+}
+
+extern "C" int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_new, const void* v_new, int64_t stride_b,
+                                    int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
+                                    const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens,
+                                    int32_t pos_offset, void* stream) {
+  if (batch > 0 && n_tokens > 0)
+    PACE_REQUIRE(block_table != nullptr && seq_lens != nullptr && table_stride >= 1,
+                 "pace_kv_append_paged: NULL block_table / seq_lens or bad table_stride");
+  AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset};
+  return run_append("pace_kv_append_paged", pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest, true,
+                    stream);
+}
+
+extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                              const int32_t* seq_lens, int32_t batch, int32_t n_rep, void* k_out, void* v_out,
+                              int64_t out_stride_b, int64_t out_stride_h, int32_t out_len, void* stream) {
+  if (int rc = check_pool(pool, "pace_kv_gather")) return rc;
+  PACE_REQUIRE(batch >= 0 && out_len >= 0 && n_rep >= 1, "pace_kv_gather: bad batch (%d), out_len (%d) or n_rep (%d)",
+               batch, out_len, n_rep);
+  if (batch == 0 || out_len == 0) return PACE_KV_OK;
+  PACE_REQUIRE(block_table && seq_lens && k_out && v_out, "pace_kv_gather: NULL pointer");
+  PACE_REQUIRE(aligned16(k_out) && aligned16(v_out), "pace_kv_gather: outputs must be 16-byte aligned");
+  PACE_REQUIRE(out_stride_b % 8 == 0 && out_stride_h % 8 == 0, "pace_kv_gather: output strides must be multiples of 8");
+  const int n_blocks = (out_len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
+  PACE_REQUIRE(table_stride >= 1, "pace_kv_gather: table_stride %d", table_stride);
+  PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "pace_kv_gather: batch/heads exceed grid limits");
+  dim3 grid(n_blocks, pool->num_kv_heads, batch);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint16_t* ko = static_cast<uint16_t*>(k_out);
+  uint16_t* vo = static_cast<uint16_t*>(v_out);
+  if (pool->head_dim == 128)
+    hipLaunchKernelGGL(kv_gather_kernel<128>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, n_rep,
+                       ko, vo, out_stride_b, out_stride_h, out_len);
+  else
+    hipLaunchKernelGGL(kv_gather_kernel<64>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, n_rep, ko,
+                       vo, out_stride_b, out_stride_h, out_len);
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
+}
+
+extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst, const int32_t* pairs,
+                                   int32_t n_pairs, void* stream) {
+  if (int rc = check_pool(src, "pace_kv_copy_blocks(src)")) return rc;
+  if (int rc = check_pool(dst, "pace_kv_copy_blocks(dst)")) return rc;
+  PACE_REQUIRE(src->head_dim == dst->head_dim && src->num_kv_heads == dst->num_kv_heads,
+               "pace_kv_copy_blocks: src and dst pools differ in head_dim or num_kv_heads");
+  PACE_REQUIRE(n_pairs >= 0, "pace_kv_copy_blocks: negative n_pairs");
+  if (n_pairs == 0) return PACE_KV_OK;
+  PACE_REQUIRE(pairs != nullptr, "pace_kv_copy_blocks: pairs is NULL");
+  PACE_REQUIRE(src->num_kv_heads <= 65535, "pace_kv_copy_blocks: too many heads");
+  hipLaunchKernelGGL(kv_copy_blocks_kernel, dim3(n_pairs, src->num_kv_heads), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), *src, *dst, pairs);
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
+}

@@ -1,0 +1,479 @@
+// Paged scaled-dot-product attention for gfx950 (decode and multi-token verify).
+//
+// Work decomposition: one 64-lane wavefront per (sequence, KV head, context
+// partition, group of query rows).  The query rows of one KV head are the
+// q_len * n_rep (token, GQA replica) pairs; up to 16*NQT of them ride along in
+// registers, so K and V are read from HBM once per KV head, not once per query
+// head.  A second small kernel merges the partitions of a sequence.
+//
+// Inner step ("unit") = 32 tokens = two pool blocks.  With lane = (n, g),
+// n = lane % 16, g = lane / 16:
+//   S^T tile  = K[16 tokens x 32 dims] * Q^T[32 dims x 16 rows]   (v_mfma_f32_16x16x32_bf16)
+//       A operand: lane (n, g) holds 16 bytes of K row tok(n): dims 32*kk + 8g .. +8
+//       C layout : lane (n, g) holds rows 4g..4g+3 of the tile, column n = query row
+//   Token rows of the two tiles are interleaved so that lane (n, g) ends up with
+//   the scores of tokens 8g..8g+7 of the unit for query row n -- exactly the B
+//   operand slot of the second product:
+//   O^T tile  = V^T[16 dims x 32 tokens] * P^T[32 tokens x 16 rows]
+//       A operand: lane (n, g) holds 16 bytes of the dim-major V slab: dim 16j+n,
+//                  tokens 8g..8g+7 of the unit  (one coalesced 16-byte load)
+//   so probabilities never leave their lane between the two products, and the
+//   softmax state (running max, sum, output accumulators) of query row n lives
+//   in the four lanes (n, 0..3).
+#include "common.h"
+
+namespace pace_kv {
+
+struct PagedAttnParams {
+  const uint16_t* q;
+  int64_t q_sb, q_sh, q_ss;
+  uint16_t* out;
+  int64_t o_sb, o_sh, o_ss;
+  const uint16_t* kpool;
+  const uint16_t* vpool;
+  int64_t k_bs, k_hs, v_bs, v_hs;
+  int32_t num_blocks;
+  const int32_t* table;
+  int32_t table_stride;
+  const int32_t* seq_lens;
+  const int32_t* kv_start;
+  const void* mask;
+  int32_t mask_is_f32;
+  int32_t mask_len;
+  int64_t m_sb, m_ss;
+  int32_t n_rep, q_len, num_q_heads;
+  int32_t causal;
+  int32_t n_qgroups;
+  int32_t part_tokens;
+  int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
+  float scale_log2;   // softmax scale * log2(e)
+  float* part_o;      // [B][Hq][S][max_parts][D]
+  float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
+};
+
+constexpr float kNegInf = -__builtin_inff();
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+template <int D>
+struct UnitRegs {
+  u32x4 k[2][D / 32];  // [tile][contraction step]
+  u32x4 v[D / 16];     // [dim tile]
+};
+
+// Issue the 16-byte loads of one 32-token unit.  ids: pool block ids of the
+// unit's two blocks (wave-uniform).
+template <int D>
+__device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n,
+                                          int g) {
+  // K: lane (n, g) reads token 8*(n/4) + 4*tile + n%4 of the unit.
+  const int tok0 = 8 * (n >> 2) + (n & 3);  // tile 0; tile 1 is +4
+  const int64_t kblk = (n >= 8) ? idB : idA;
+  const uint16_t* kp = p.kpool + kblk * p.k_bs + (int64_t)kvh * p.k_hs + (tok0 & 15) * D + 8 * g;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + t * 4 * D + kk * 32);
+  // V: lane (n, g) reads dim 16j + n, tokens 8g..8g+7 of the unit.
+  const int64_t vblk = (g >= 2) ? idB : idA;
+  const uint16_t* vp = p.vpool + vblk * p.v_bs + (int64_t)kvh * p.v_hs + n * PACE_KV_BLOCK_TOKENS + 8 * (g & 1);
+#pragma unroll
+  for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 16 * PACE_KV_BLOCK_TOKENS);
+}
+
+template <int D, int NQT>
+struct RowState {
+  f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
+  float m[NQT];          // running max (log2 units)
+  float l[NQT];          // this lane's share of the running sum
+  int limit[NQT];        // last readable token of the row (-1: row is padding)
+  int64_t mask_off[NQT]; // element offset of the row's mask line
+};
+
+template <int D, int NQT, bool HAS_MASK>
+__device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
+                                             RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
+                                             int start, bool full, int g) {
+  constexpr int KK = D / 32;
+  constexpr int MT = D / 16;
+  // Zero V columns past the end of the sequence so that stale pool contents
+  // (possibly non-finite bit patterns) cannot reach the accumulators.
+  u32x4 vreg[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) vreg[j] = r.v[j];
+  if (!full) {
+    const int nvalid = tok_end - (t0 + 8 * g);  // tokens of this lane's 8 that exist
+    if (nvalid < 8) {
+      u32x4 keep;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int c = nvalid - 2 * e;  // tokens 2e, 2e+1 live in dword e
+        keep[e] = c >= 2 ? 0xffffffffu : (c == 1 ? 0x0000ffffu : 0u);
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j) vreg[j] &= keep;
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[t][kk]),
+                                                      __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
+      s[t] = acc * p.scale_log2;
+    }
+    // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
+    if (HAS_MASK) {
+      const int mbase = t0 + 8 * g;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = mbase + 4 * t + i;
+          float add = kNegInf;
+          if (tok < p.mask_len && st.limit[qt] >= 0) {
+            if (p.mask_is_f32)
+              add = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok] * kLog2e;
+            else
+              add = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]) * kLog2e;
+          }
+          s[t][i] += add;
+        }
+    }
+    if (!full || HAS_MASK) {
+      const int hi = min(st.limit[qt], tok_end - 1);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = t0 + 8 * g + 4 * t + i;
+          if (tok > hi || tok < start) s[t][i] = kNegInf;
+          // a NaN score can only come from a stale K row; it is replaced above
+          // when out of range, and propagates (like the reference) when in range.
+        }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    mx = fmaxf(mx, xor_lanes(mx, 16));
+    mx = fmaxf(mx, xor_lanes(mx, 32));
+    const float m_old = st.m[qt];
+    const float m_new = fmaxf(m_old, mx);
+    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_old - m_use);  // m_old = -inf -> 0
+    float psum = 0.f;
+    f32x4 pr[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pr[t][i] = __builtin_amdgcn_exp2f(s[t][i] - m_use);
+        psum += pr[t][i];
+      }
+    st.m[qt] = m_new;
+    st.l[qt] = st.l[qt] * alpha + psum;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j) st.o[qt][j] *= alpha;
+    }
+    u32x4 pb;
+    pb[0] = pack_bf16x2(pr[0][0], pr[0][1]);
+    pb[1] = pack_bf16x2(pr[0][2], pr[0][3]);
+    pb[2] = pack_bf16x2(pr[1][0], pr[1][1]);
+    pb[3] = pack_bf16x2(pr[1][2], pr[1][3]);
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+      st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
+                                                           __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
+  }
+}
+
+template <int D, int NQT, bool HAS_MASK>
+__global__ __launch_bounds__(64) void paged_attn_kernel(const PagedAttnParams p) {
+  constexpr int KK = D / 32;
+  constexpr int MT = D / 16;
+  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+  const int part = blockIdx.x, kvh = blockIdx.y;
+  const int b = blockIdx.z / p.n_qgroups, qg = blockIdx.z % p.n_qgroups;
+  const int len = p.seq_lens[b];
+  const int P = p.part_tokens;
+  const int n_parts = len > 0 ? (len + P - 1) / P : 1;
+  if (part >= n_parts) return;
+  const int start = p.kv_start ? p.kv_start[b] : 0;
+  const int tok_begin = part * P;
+  const int tok_end = min(len, tok_begin + P);
+  const int S = p.q_len, R = S * p.n_rep;
+
+  // Query rows of this wave (B operand of the first product) and per-row limits.
+  u32x4 qreg[NQT][KK];
+  RowState<D, NQT> st;
+  int row_s[NQT], row_h[NQT];
+  int min_limit = 0x7fffffff;
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int r = (qg * NQT + qt) * 16 + n;
+    const bool valid = r < R;
+    const int s = valid ? r / p.n_rep : 0;
+    const int hq = kvh * p.n_rep + (valid ? r % p.n_rep : 0);
+    row_s[qt] = s;
+    row_h[qt] = hq;
+    st.limit[qt] = valid ? (p.causal ? len - S + s : len - 1) : -1;
+    if (valid) min_limit = min(min_limit, st.limit[qt]);
+    st.mask_off[qt] = HAS_MASK ? (int64_t)b * p.m_sb + (int64_t)s * p.m_ss : 0;
+    st.m[qt] = kNegInf;
+    st.l[qt] = 0.f;
+    const uint16_t* qp = p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)s * p.q_ss + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  // Rows of padding lanes must not relax the "whole unit readable" test.
+  min_limit = min(min_limit, __shfl_xor(min_limit, 1, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 2, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 4, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 8, 64));
+
+  // Pool block ids of this partition, one per lane (partition <= 64 blocks).
+  const int first_blk = tok_begin / PACE_KV_BLOCK_TOKENS;
+  const int live_blks = (len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
+  int my_id = 0;
+  if (first_blk + lane < live_blks) my_id = p.table[(int64_t)b * p.table_stride + first_blk + lane];
+  my_id = my_id < 0 ? 0 : (my_id >= p.num_blocks ? p.num_blocks - 1 : my_id);  // never read outside the pool
+
+  const int n_units = (tok_end - tok_begin + 31) / 32;
+  UnitRegs<D> bufA, bufB;
+  if (n_units > 0) load_unit<D>(bufA, p, kvh, __builtin_amdgcn_readlane(my_id, 0), __builtin_amdgcn_readlane(my_id, 1), n, g);
+  for (int u = 0; u < n_units; u += 2) {
+    const int t0 = tok_begin + 32 * u;
+    if (u + 1 < n_units)
+      load_unit<D>(bufB, p, kvh, __builtin_amdgcn_readlane(my_id, 2 * u + 2), __builtin_amdgcn_readlane(my_id, 2 * u + 3), n,
+                   g);
+    {
+      const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
+      compute_unit<D, NQT, HAS_MASK>(bufA, qreg, st, p, t0, tok_end, start, full, g);
+    }
+    if (u + 1 < n_units) {
+      if (u + 2 < n_units)
+        load_unit<D>(bufA, p, kvh, __builtin_amdgcn_readlane(my_id, 2 * u + 4), __builtin_amdgcn_readlane(my_id, 2 * u + 5),
+                     n, g);
+      const int t1 = t0 + 32;
+      const bool full = (t1 + 32 <= tok_end) && (t1 + 31 <= min_limit) && (t1 >= start);
+      compute_unit<D, NQT, HAS_MASK>(bufB, qreg, st, p, t1, tok_end, start, full, g);
+    }
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int r = (qg * NQT + qt) * 16 + n;
+    float l = st.l[qt];
+    l += xor_lanes(l, 16);
+    l += xor_lanes(l, 32);
+    if (r >= R) continue;
+    if (p.max_parts == 1) {
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)row_h[qt] * p.o_sh + (int64_t)row_s[qt] * p.o_ss + 4 * g;
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        u32x2 w;
+        w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
+        w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
+        *reinterpret_cast<u32x2*>(op + 16 * j) = w;
+      }
+    } else {
+      const int64_t row = ((int64_t)b * p.num_q_heads + row_h[qt]) * S + row_s[qt];
+      float* po = p.part_o + (row * p.max_parts + part) * D + 4 * g;
+#pragma unroll
+      for (int j = 0; j < MT; ++j) *reinterpret_cast<f32x4*>(po + 16 * j) = st.o[qt][j];
+      if (g == 0) {
+        float* ml = p.part_ml + (row * p.max_parts + part) * 2;
+        ml[0] = st.m[qt];
+        ml[1] = l;
+      }
+    }
+  }
+}
+
+// Merge the partitions of one query row: out = sum_p 2^(m_p - M) o_p / sum_p 2^(m_p - M) l_p.
+template <int D>
+__global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnParams p) {
+  const int64_t row = blockIdx.x;  // (b, hq, s)
+  const int S = p.q_len;
+  const int s = (int)(row % S);
+  const int hq = (int)((row / S) % p.num_q_heads);
+  const int b = (int)(row / ((int64_t)S * p.num_q_heads));
+  const int len = p.seq_lens[b];
+  const int n_parts = len > 0 ? (len + p.part_tokens - 1) / p.part_tokens : 1;
+  const float* ml = p.part_ml + row * p.max_parts * 2;
+  const float* po = p.part_o + row * p.max_parts * D;
+  float M = kNegInf;
+  for (int i = 0; i < n_parts; ++i) M = fmaxf(M, ml[2 * i]);
+  const float m_use = (M == kNegInf) ? 0.f : M;
+  constexpr int PER = D / 64;  // dims per lane
+  float acc[PER];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+  float L = 0.f;
+  for (int i = 0; i < n_parts; ++i) {
+    const float w = __builtin_amdgcn_exp2f(ml[2 * i] - m_use);
+    L += w * ml[2 * i + 1];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) acc[e] += w * po[(int64_t)i * D + threadIdx.x * PER + e];
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + threadIdx.x * PER;
+  if (PER == 2) {
+    *reinterpret_cast<uint32_t*>(op) = pack_bf16x2(acc[0] * inv, acc[PER - 1] * inv);
+  } else {
+    op[0] = (uint16_t)f32_to_bf16_bits(acc[0] * inv);
+  }
+}
+
+static int auto_partition(int32_t max_seq_len, int64_t waves_per_partition_row) {
+  // Aim for about eight resident waves per compute unit (256 CUs); never split
+  // finer than 128 tokens, never coarser than 1024 (64 pool blocks, one id per lane).
+  const int64_t target_waves = 2048;
+  int64_t per = ((int64_t)max_seq_len * waves_per_partition_row + target_waves - 1) / target_waves;
+  per = (per + 31) / 32 * 32;
+  if (per < 128) per = 128;
+  if (per > 1024) per = 1024;
+  return (int)per;
+}
+
+static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
+  if (requested > 0) return requested;
+  const int nqt_rows = 64;
+  const int64_t groups = (rows + nqt_rows - 1) / nqt_rows;
+  return auto_partition(max_seq_len, (int64_t)batch * num_kv_heads * groups);
+}
+
+template <int D, int NQT>
+static void launch(const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
+  if (has_mask)
+    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, true>), grid, dim3(64), 0, s, p);
+  else
+    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, false>), grid, dim3(64), 0, s, p);
+}
+
+static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, void* stream, const char* who) {
+  if (int rc = check_pool(pool, who)) return rc;
+  PACE_REQUIRE(a != nullptr, "%s: args is NULL", who);
+  PACE_REQUIRE(a->batch >= 0 && a->q_len >= 1 && a->num_q_heads >= 1, "%s: bad batch (%d), q_len (%d) or num_q_heads (%d)",
+               who, a->batch, a->q_len, a->num_q_heads);
+  if (a->batch == 0) return PACE_KV_OK;
+  PACE_REQUIRE(a->q && a->out && a->block_table && a->seq_lens, "%s: NULL q / out / block_table / seq_lens", who);
+  PACE_REQUIRE(a->num_q_heads % pool->num_kv_heads == 0, "%s: num_q_heads %d not a multiple of num_kv_heads %d", who,
+               a->num_q_heads, pool->num_kv_heads);
+  PACE_REQUIRE(aligned16(a->q) && (a->q_stride_b % 8) == 0 && (a->q_stride_h % 8) == 0 && (a->q_stride_s % 8) == 0,
+               "%s: q must be 16-byte aligned with strides that are multiples of 8 elements", who);
+  PACE_REQUIRE((reinterpret_cast<uintptr_t>(a->out) & 7u) == 0 && (a->o_stride_b % 4) == 0 && (a->o_stride_h % 4) == 0 &&
+                   (a->o_stride_s % 4) == 0,
+               "%s: out must be 8-byte aligned with strides that are multiples of 4 elements", who);
+  PACE_REQUIRE(a->max_seq_len >= 0 && a->table_stride >= 1, "%s: bad max_seq_len (%d) or table_stride (%d)", who,
+               a->max_seq_len, a->table_stride);
+  PACE_REQUIRE((int64_t)a->table_stride * PACE_KV_BLOCK_TOKENS >= a->max_seq_len,
+               "%s: block table row (%d blocks) cannot hold max_seq_len %d", who, a->table_stride, a->max_seq_len);
+  if (a->mask) {
+    PACE_REQUIRE(a->mask_dtype == PACE_DTYPE_F32 || a->mask_dtype == PACE_DTYPE_BF16, "%s: bad mask dtype %d", who,
+                 a->mask_dtype);
+    PACE_REQUIRE(a->mask_len >= 0, "%s: negative mask_len", who);
+  }
+  const int n_rep = a->num_q_heads / pool->num_kv_heads;
+  const int rows = a->q_len * n_rep;
+  const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
+  PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= 1024, "%s: partition_tokens %d must be a multiple of 32 in [32, 1024]",
+               who, part);
+  const int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
+
+  PagedAttnParams p;
+  p.q = static_cast<const uint16_t*>(a->q);
+  p.q_sb = a->q_stride_b, p.q_sh = a->q_stride_h, p.q_ss = a->q_stride_s;
+  p.out = static_cast<uint16_t*>(a->out);
+  p.o_sb = a->o_stride_b, p.o_sh = a->o_stride_h, p.o_ss = a->o_stride_s;
+  p.kpool = static_cast<const uint16_t*>(pool->k);
+  p.vpool = static_cast<const uint16_t*>(pool->v);
+  p.k_bs = pool->k_block_stride, p.k_hs = pool->k_head_stride;
+  p.v_bs = pool->v_block_stride, p.v_hs = pool->v_head_stride;
+  p.num_blocks = pool->num_blocks;
+  p.table = a->block_table, p.table_stride = a->table_stride;
+  p.seq_lens = a->seq_lens, p.kv_start = a->kv_start;
+  p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
+  p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
+  p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;
+  p.causal = a->causal;
+  p.part_tokens = part, p.max_parts = max_parts;
+  p.scale_log2 = a->scale * kLog2e;
+  p.part_o = nullptr, p.part_ml = nullptr;
+
+  // Query-row tiles per wave: 1 for plain decode with n_rep <= 16, up to 4.
+  const int tiles = (rows + 15) / 16;
+  const int nqt = tiles >= 4 ? 4 : (tiles == 3 ? 4 : tiles);
+  p.n_qgroups = (tiles + nqt - 1) / nqt;
+
+  if (max_parts > 1) {
+    const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
+    const size_t need = rows_total * max_parts * (pool->head_dim + 2) * sizeof(float);
+    PACE_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need,
+                 "%s: workspace too small (%zu bytes given, %zu needed)", who, a->workspace_bytes, need);
+    PACE_REQUIRE(aligned16(a->workspace), "%s: workspace must be 16-byte aligned", who);
+    p.part_o = static_cast<float*>(a->workspace);
+    p.part_ml = p.part_o + rows_total * max_parts * pool->head_dim;
+  }
+  PACE_REQUIRE((int64_t)a->batch * p.n_qgroups <= 65535 && pool->num_kv_heads <= 65535, "%s: grid too large", who);
+  dim3 grid(max_parts, pool->num_kv_heads, a->batch * p.n_qgroups);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool has_mask = a->mask != nullptr;
+  if (pool->head_dim == 128) {
+    if (nqt == 1) launch<128, 1>(p, grid, has_mask, s);
+    else if (nqt == 2) launch<128, 2>(p, grid, has_mask, s);
+    else launch<128, 4>(p, grid, has_mask, s);
+  } else {
+    if (nqt == 1) launch<64, 1>(p, grid, has_mask, s);
+    else if (nqt == 2) launch<64, 2>(p, grid, has_mask, s);
+    else launch<64, 4>(p, grid, has_mask, s);
+  }
+  PACE_HIP_CHECK(hipGetLastError());
+  if (max_parts > 1) {
+    const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
+    PACE_REQUIRE(rows_total < ((size_t)1 << 31), "%s: too many query rows", who);
+    if (pool->head_dim == 128)
+      hipLaunchKernelGGL(paged_attn_merge_kernel<128>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+    else
+      hipLaunchKernelGGL(paged_attn_merge_kernel<64>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+    PACE_HIP_CHECK(hipGetLastError());
+  }
+  return PACE_KV_OK;
+}
+
+}  // namespace pace_kv
+
+using namespace pace_kv;
+
+extern "C" size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
+                                                  int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {
+  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
+  const int rows = q_len * (num_q_heads / num_kv_heads);
+  const int part = resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, rows);
+  const int max_parts = (max_seq_len + part - 1) / part;
+  if (max_parts <= 1) return 0;
+  return (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float);
+}
+
+extern "C" int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {
+  if (args && args->q_len != 1) {
+    set_error("pace_paged_attn_decode: q_len must be 1 (got %d); use pace_paged_attn_verify", args->q_len);
+    return PACE_KV_EINVAL;
+  }
+  return run_paged_attn(pool, args, stream, "pace_paged_attn_decode");
+}
+
+extern "C" int pace_paged_attn_verify(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {
+  return run_paged_attn(pool, args, stream, "pace_paged_attn_verify");
+}

@@ -1,0 +1,153 @@
+"""ctypes binding of ``libpace_kv_hip.so`` (declared in ``include/pace_kv_hip.h``).
+
+The library is the only implementation of the hot path: if it is missing or a
+symbol cannot be resolved this module raises, it never substitutes another path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
+from typing import Optional
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libpace_kv_hip.so")
+
+BLOCK_TOKENS = 16
+DTYPE_F32, DTYPE_BF16 = 0, 1
+ABI_VERSION = 1
+
+EXPORTED_SYMBOLS = (
+    "pace_kv_last_error",
+    "pace_kv_abi_version",
+    "pace_kv_append",
+    "pace_kv_append_paged",
+    "pace_kv_gather",
+    "pace_kv_copy_blocks",
+    "pace_paged_attn_workspace_bytes",
+    "pace_paged_attn_decode",
+    "pace_paged_attn_verify",
+    "pace_attn_dense",
+)
+
+
+class PoolDesc(Structure):
+    """``pace_kv_pool_t``."""
+
+    _fields_ = [
+        ("k", c_void_p),
+        ("v", c_void_p),
+        ("k_block_stride", c_int64),
+        ("k_head_stride", c_int64),
+        ("v_block_stride", c_int64),
+        ("v_head_stride", c_int64),
+        ("num_blocks", c_int32),
+        ("num_kv_heads", c_int32),
+        ("head_dim", c_int32),
+        ("block_size", c_int32),
+    ]
+
+
+class PagedAttnArgs(Structure):
+    """``pace_paged_attn_args_t``."""
+
+    _fields_ = [
+        ("q", c_void_p),
+        ("q_stride_b", c_int64),
+        ("q_stride_h", c_int64),
+        ("q_stride_s", c_int64),
+        ("out", c_void_p),
+        ("o_stride_b", c_int64),
+        ("o_stride_h", c_int64),
+        ("o_stride_s", c_int64),
+        ("block_table", c_void_p),
+        ("table_stride", c_int32),
+        ("seq_lens", c_void_p),
+        ("kv_start", c_void_p),
+        ("mask", c_void_p),
+        ("mask_dtype", c_int32),
+        ("mask_len", c_int32),
+        ("mask_stride_b", c_int64),
+        ("mask_stride_s", c_int64),
+        ("batch", c_int32),
+        ("num_q_heads", c_int32),
+        ("q_len", c_int32),
+        ("causal", c_int32),
+        ("max_seq_len", c_int32),
+        ("partition_tokens", c_int32),
+        ("scale", c_float),
+        ("workspace", c_void_p),
+        ("workspace_bytes", c_size_t),
+    ]
+
+
+class NativeError(RuntimeError):
+    """A C-ABI entry point returned a failure code."""
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and declare every prototype."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            f"{_LIB_PATH} is missing: build it with `python amd-pace_amd/build.py` "
+            "(hipcc, gfx950). There is no other implementation of this path."
+        )
+    lib = ctypes.CDLL(_LIB_PATH)
+    P = POINTER(PoolDesc)
+    lib.pace_kv_last_error.restype = c_char_p
+    lib.pace_kv_last_error.argtypes = []
+    lib.pace_kv_abi_version.restype = c_int32
+    lib.pace_kv_abi_version.argtypes = []
+    lib.pace_kv_append.restype = ctypes.c_int
+    lib.pace_kv_append.argtypes = [P, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p]
+    lib.pace_kv_append_paged.restype = ctypes.c_int
+    lib.pace_kv_append_paged.argtypes = [
+        P, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
+        c_void_p, c_int32, c_void_p, c_int32, c_void_p,
+    ]
+    lib.pace_kv_gather.restype = ctypes.c_int
+    lib.pace_kv_gather.argtypes = [
+        P, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p,
+    ]
+    lib.pace_kv_copy_blocks.restype = ctypes.c_int
+    lib.pace_kv_copy_blocks.argtypes = [P, P, c_void_p, c_int32, c_void_p]
+    lib.pace_paged_attn_workspace_bytes.restype = c_size_t
+    lib.pace_paged_attn_workspace_bytes.argtypes = [c_int32] * 7
+    A = POINTER(PagedAttnArgs)
+    lib.pace_paged_attn_decode.restype = ctypes.c_int
+    lib.pace_paged_attn_decode.argtypes = [P, A, c_void_p]
+    lib.pace_paged_attn_verify.restype = ctypes.c_int
+    lib.pace_paged_attn_verify.argtypes = [P, A, c_void_p]
+    lib.pace_attn_dense.restype = ctypes.c_int
+    lib.pace_attn_dense.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+        c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
+    ]
+    got = int(lib.pace_kv_abi_version())
+    if got != ABI_VERSION:
+        raise ImportError(f"{_LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    """Raise ``NativeError`` carrying the library's message when ``rc`` is a failure."""
+    if rc != 0:
+        msg = load().pace_kv_last_error().decode("utf-8", "replace")
+        raise NativeError(f"[{rc}] {msg}")
+
+
+def current_stream_ptr() -> int:
+    """Raw ``hipStream_t`` of torch's current stream on the current device."""
+    import torch
+
+    return int(torch.cuda.current_stream().cuda_stream)

@@ -1,0 +1,450 @@
+"""KV-cache manager interface of the reference, backed by block-paged HBM storage.
+
+Interface kept from ``pace/llm/cache.py`` of the reference:
+
+* ``KVCacheType`` (``:18-33``) -- string-constructible enum, plus ``PAGED``.
+* ``KVCacheManager(config, max_seq_length, cache_type)`` (``:48-123``) -- one cache
+  per ``config.num_hidden_layers``; ``len()``, ``[]``, ``update_mask``,
+  ``update_cache_with_beam_indices``, ``remove_cache``.
+* ``KVCacheBase`` (``:126-167``) -- ``update_cache(key_states, value_states,
+  concat_dim) -> (key, value)``, ``remove_cache(remove_len)``, ``update_mask``,
+  ``update_cache_with_beam_indices``; attributes ``key``, ``value``, ``seq_len``,
+  ``concat_dim``.
+
+Error behaviour kept: changed ``concat_dim`` -> ``AssertionError``
+(``:286-289``); over-long removal -> ``ValueError("Cannot remove more tokens
+than available in cache.")`` (``:237-238``); unknown type -> ``ValueError``.
+
+``PagedKVCache`` stores ``num_kv_heads`` heads (a GQA-expanded input, which is
+what the reference's models pass after ``repeat_kv``, ``pace/llm/models/llama.py:151-158``,
+is de-duplicated by stride) and returns *views* instead of dense tensors;
+``MultiHeadAttention`` accepts those views, and ``view.dense()`` materialises the
+reference-shaped ``[B, Hq, L, D]`` tensor.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from abc import ABC, abstractmethod
+from enum import Enum
+from typing import List, Optional, Sequence, Tuple, Union
+
+import numpy as np
+import torch
+
+from .. import _native as nat
+from ..utils.logging import PACE_LLM_ASSERT, PACE_LLM_DEBUG
+from .paged import BLOCK, PagedState, blocks_for
+
+
+class KVCacheType(Enum):
+    DYNAMIC = "dynamic"
+    BMC = "bmc"
+    PAGED = "paged"
+
+    @staticmethod
+    def get_kv_cache_type(cache_type: Union[str, "KVCacheType"]) -> "KVCacheType":
+        return KVCacheType(cache_type) if isinstance(cache_type, str) else cache_type
+
+
+def get_kv_cache_class(cache_type: Union[str, KVCacheType]):
+    cache_type = KVCacheType.get_kv_cache_type(cache_type)
+    if cache_type is KVCacheType.PAGED:
+        return PagedKVCache
+    if cache_type in (KVCacheType.DYNAMIC, KVCacheType.BMC):
+        from .contiguous import BMCKVCache, DynamicKVCache
+
+        return DynamicKVCache if cache_type is KVCacheType.DYNAMIC else BMCKVCache
+    raise ValueError(f"Invalid cache type: {cache_type}")
+
+
+class KVCacheBase(ABC):
+    """Per-layer cache contract (reference ``cache.py:126-167``)."""
+
+    key = None
+    value = None
+    seq_len = 0
+    concat_dim: Optional[int] = None
+
+    @abstractmethod
+    def update_cache(self, key_states, value_states, concat_dim: int):
+        ...
+
+    @abstractmethod
+    def remove_cache(self, remove_len: int) -> None:
+        ...
+
+    def update_mask(self, attn_mask: torch.Tensor, input_size: int) -> torch.Tensor:
+        return attn_mask
+
+    def update_cache_with_beam_indices(self, beam_idx: torch.Tensor) -> None:
+        if self.key is not None and self.value is not None:
+            self.key = self.key.index_select(0, beam_idx.to(self.key.device))
+            self.value = self.value.index_select(0, beam_idx.to(self.value.device))
+
+    def _pin_concat_dim(self, concat_dim: int) -> None:
+        if self.concat_dim is None:
+            self.concat_dim = concat_dim
+        else:
+            PACE_LLM_ASSERT(self.concat_dim == concat_dim, "concat_dim should be the same for all updates")
+
+
+class PagedKVView:
+    """What ``PagedKVCache.update_cache`` returns in place of a dense tensor."""
+
+    def __init__(self, cache: "PagedKVCache", which: str):
+        self.cache = cache
+        self.which = which
+
+    @property
+    def shape(self) -> Tuple[int, int, int, int]:
+        c = self.cache
+        return (c.batch, c.num_kv_heads * c.n_rep, int(c.lens.max(initial=0)), c.head_dim)
+
+    def size(self, dim: int) -> int:
+        return self.shape[dim]
+
+    def dense(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None) -> torch.Tensor:
+        k, v = self.cache.gather(n_rep=n_rep, pad_to=pad_to)
+        return k if self.which == "key" else v
+
+
+class PagedKVCache(KVCacheBase):
+    """One layer of block-paged K/V in HBM.
+
+    ``shared`` lets the layers of a ``KVCacheManager`` use one block table.
+    ``num_kv_heads`` (or ``n_rep``) tells the cache how a GQA-expanded input maps
+    to stored heads; with neither, every input head is stored.
+    """
+
+    def __init__(
+        self,
+        max_seq_length: int,
+        *,
+        shared: Optional[dict] = None,
+        num_kv_heads: Optional[int] = None,
+        n_rep: Optional[int] = None,
+        num_blocks: Optional[int] = None,
+    ):
+        self.max_seq_length = int(max_seq_length)
+        self._shared = shared if shared is not None else {}
+        self._cfg_kv_heads = num_kv_heads
+        self._cfg_n_rep = n_rep
+        self._cfg_num_blocks = num_blocks
+        self.state: Optional[PagedState] = None
+        self.pool: Optional[torch.Tensor] = None
+        self._desc: Optional[nat.PoolDesc] = None
+        self.lens: np.ndarray = np.zeros(0, dtype=np.int64)
+        self.seq_len = 0
+        self.concat_dim = None
+        self.key: Optional[PagedKVView] = None
+        self.value: Optional[PagedKVView] = None
+        self.batch = 0
+        self.num_kv_heads = 0
+        self.n_rep = 1
+        self.head_dim = 0
+        self.partition_tokens = 0  # 0: let the library choose
+        PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
+
+    # -- set-up -----------------------------------------------------------------
+    def _lazy_init(self, key_states: torch.Tensor) -> None:
+        if self.pool is not None:
+            return
+        if not key_states.is_cuda:
+            raise RuntimeError("PagedKVCache stores its blocks in GPU memory; key/value states must be device tensors")
+        if key_states.dtype != torch.bfloat16:
+            raise RuntimeError(f"PagedKVCache stores bf16; got {key_states.dtype}")
+        nat.load()
+        B, h_in, _, D = key_states.shape
+        if self._cfg_kv_heads is not None:
+            hkv = int(self._cfg_kv_heads)
+        elif self._cfg_n_rep is not None:
+            hkv = h_in // int(self._cfg_n_rep)
+        else:
+            hkv = h_in
+        if h_in % hkv:
+            raise RuntimeError(f"{h_in} input heads cannot be reduced to {hkv} KV heads")
+        self.batch, self.num_kv_heads, self.head_dim = int(B), hkv, int(D)
+        self.n_rep = int(self._cfg_n_rep) if self._cfg_n_rep is not None else h_in // hkv
+        if "state" not in self._shared:
+            self._shared["state"] = PagedState(B, self.max_seq_length, self._cfg_num_blocks, key_states.device)
+        self.state = self._shared["state"]
+        if self.state.batch != B:
+            raise RuntimeError(f"batch changed from {self.state.batch} to {B}")
+        nb = self.state.allocator.num_blocks
+        # [block][K|V][head][16*D]: one block of one layer is contiguous.
+        self.pool = torch.zeros((nb, 2, hkv, BLOCK * D), dtype=torch.bfloat16, device=key_states.device)
+        self.state.pools.append(self.pool)
+        self._desc = self._describe(self.pool)
+        self.lens = np.zeros(B, dtype=np.int64)
+
+    def _describe(self, pool: torch.Tensor) -> nat.PoolDesc:
+        nb, _, hkv, slab = pool.shape
+        return nat.PoolDesc(
+            k=pool[:, 0].data_ptr(),
+            v=pool[:, 1].data_ptr(),
+            k_block_stride=pool.stride(0),
+            k_head_stride=pool.stride(2),
+            v_block_stride=pool.stride(0),
+            v_head_stride=pool.stride(2),
+            num_blocks=nb,
+            num_kv_heads=hkv,
+            head_dim=slab // BLOCK,
+            block_size=BLOCK,
+        )
+
+    # -- reference interface ----------------------------------------------------
+    def update_cache(self, key_states: torch.Tensor, value_states: torch.Tensor, concat_dim: int):
+        """Append ``T`` tokens to every sequence (reference ``cache.py:268-326``)."""
+        self._pin_concat_dim(concat_dim)
+        PACE_LLM_ASSERT(key_states.dim() == 4 and concat_dim == 2, "PagedKVCache expects [B, H, T, D] with concat_dim=2")
+        self._lazy_init(key_states)
+        self._append(key_states, value_states, None)
+        return self.key, self.value
+
+    def remove_cache(self, remove_len: int) -> None:
+        """Drop the last ``remove_len`` tokens of every sequence (reference ``cache.py:224-240``)."""
+        if self.pool is None:
+            return
+        if remove_len > self.seq_len or (self.lens < remove_len).any():
+            raise ValueError("Cannot remove more tokens than available in cache.")
+        self.truncate(np.full(self.batch, int(remove_len), dtype=np.int64))
+
+    def update_cache_with_beam_indices(self, beam_idx: torch.Tensor) -> None:
+        """Batch-row gather (reference ``cache.py:161-167``): sequence ``i`` becomes a
+        copy of old sequence ``beam_idx[i]``; blocks are copied on the device."""
+        if self.pool is None:
+            return
+        self.reorder([int(i) for i in beam_idx.tolist()])
+
+    # -- paged-only surface -----------------------------------------------------
+    def append_ragged(self, key_states: torch.Tensor, value_states: torch.Tensor, counts: Sequence[int]):
+        """Append ``counts[b]`` of the ``T`` given tokens to sequence ``b``."""
+        self._pin_concat_dim(2)
+        self._lazy_init(key_states)
+        self._append(key_states, value_states, np.asarray(counts, dtype=np.int64))
+        return self.key, self.value
+
+    def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray]) -> None:
+        B, h_in, T, D = k.shape
+        if B != self.batch or D != self.head_dim or h_in % self.num_kv_heads:
+            raise RuntimeError(f"update of shape {tuple(k.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={D}]")
+        if v.shape != k.shape:
+            raise RuntimeError("key_states and value_states differ in shape")
+        if k.stride(3) != 1 or v.stride(3) != 1 or k.stride() != v.stride() or any(s % 8 for s in k.stride()[:3]):
+            k, v = k.contiguous(), v.contiguous()
+        head_step = h_in // self.num_kv_heads  # de-duplicate a repeat_kv-expanded input
+        st = self.state
+        lib = nat.load()
+        stream = nat.current_stream_ptr()
+        if counts is None:
+            new_lens = self.lens + T
+            st.ensure_capacity(new_lens)
+            lens_dev = st.device_lens(new_lens)
+            table = st.device_table()
+            nat.check(
+                lib.pace_kv_append_paged(
+                    ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
+                    B, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -T, stream,
+                )
+            )
+        else:
+            if (counts < 0).any() or (counts > T).any():
+                raise ValueError("counts must lie in [0, T]")
+            new_lens = self.lens + counts
+            st.ensure_capacity(new_lens)
+            slots = torch.from_numpy(st.slots(self.lens, counts, T)).pin_memory().to(k.device, non_blocking=True)
+            nat.check(
+                lib.pace_kv_append(
+                    ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
+                    B, T, slots.data_ptr(), stream,
+                )
+            )
+        self.lens = new_lens
+        self.seq_len = int(new_lens.max(initial=0))
+        if self.key is None:
+            self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
+
+    def truncate(self, remove: Sequence[int]) -> None:
+        """Per-sequence rollback: forget the last ``remove[b]`` tokens of sequence ``b``
+        and return emptied blocks to the free list."""
+        remove = np.asarray(remove, dtype=np.int64)
+        if (remove > self.lens).any() or (remove < 0).any():
+            raise ValueError("Cannot remove more tokens than available in cache.")
+        self.lens = self.lens - remove
+        self.seq_len = int(self.lens.max(initial=0))
+        self._release()
+
+    def _release(self) -> None:
+        # Blocks are shared by every layer: only the longest view of a sequence frees.
+        peers = self._shared.get("layers")
+        lens = self.lens if not peers else np.max([p.lens for p in peers if p.pool is not None], axis=0)
+        self.state.release_beyond(lens)
+
+    def evict_blocks(self, b: int, logical_blocks: Sequence[int]) -> None:
+        """Remove whole logical blocks from the middle of sequence ``b``; the
+        surviving tokens keep their order and become the sequence."""
+        peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
+        new_lens = self.state.evict(b, logical_blocks, self.lens)
+        for p in peers:
+            p.lens = new_lens.copy()
+            p.seq_len = int(new_lens.max(initial=0))
+
+    def compact(self) -> int:
+        """Pack live blocks into the lowest pool ids (every layer's pool); returns blocks moved."""
+        moves = self.state.plan_compaction()
+        if len(moves):
+            pairs = torch.from_numpy(moves).pin_memory().to(self.pool.device, non_blocking=True)
+            lib = nat.load()
+            for pool in self.state.pools:
+                desc = self._describe(pool)
+                nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), pairs.data_ptr(), len(moves), nat.current_stream_ptr()))
+            self.state.apply_moves(moves)
+        return len(moves)
+
+    def reorder(self, beam_idx: Sequence[int]) -> None:
+        st = self.state
+        peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
+        old_table, old_n, old_lens = st.table.copy(), st.n_blocks.copy(), self.lens.copy()
+        pairs: List[Tuple[int, int]] = []
+        new_rows = []
+        for src in beam_idx:
+            n = int(old_n[src])
+            fresh = st.allocator.allocate(n)
+            pairs += list(zip(old_table[src, :n].tolist(), fresh))
+            new_rows.append(fresh)
+        if pairs:
+            dev = torch.tensor(pairs, dtype=torch.int32).pin_memory().to(self.pool.device, non_blocking=True)
+            lib = nat.load()
+            for pool in st.pools:
+                desc = self._describe(pool)
+                nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), dev.data_ptr(), len(pairs), nat.current_stream_ptr()))
+        for b in range(st.batch):
+            st.allocator.free(old_table[b, : int(old_n[b])].tolist())
+        st.table[:] = 0
+        for i, row in enumerate(new_rows):
+            st.table[i, : len(row)] = row
+            st.n_blocks[i] = len(row)
+        st._table_dirty = True
+        new_lens = old_lens[list(beam_idx)]
+        for p in peers:
+            p.lens = new_lens.copy()
+            p.seq_len = int(new_lens.max(initial=0))
+
+    def gather(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Dense ``[B, Hkv*n_rep, L, D]`` copies of K and V (zeros past each length)."""
+        n_rep = self.n_rep if n_rep is None else int(n_rep)
+        L = int(self.lens.max(initial=0)) if pad_to is None else int(pad_to)
+        shape = (self.batch, self.num_kv_heads * n_rep, L, self.head_dim)
+        k = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
+        v = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
+        if L:
+            st = self.state
+            table, lens_dev = st.device_table(), st.device_lens(self.lens)
+            nat.check(
+                nat.load().pace_kv_gather(
+                    ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), self.batch, n_rep,
+                    k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, nat.current_stream_ptr(),
+                )
+            )
+        return k, v
+
+    def attend(self, query: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+               kv_start: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``softmax(q K^T / sqrt(D) + mask) V`` of ``query [B, Hq, S, D]`` over this cache.
+
+        Without a mask, row ``s`` of sequence ``b`` reads tokens ``<= len_b - S + s``
+        (the causal mask ``pace/llm/models/llama.py:292-299`` builds); with an additive
+        mask ``[B|1, 1, S|1, Lm]`` the mask alone decides, as in the reference.
+        """
+        if query.dim() != 4 or query.dtype != torch.bfloat16 or not query.is_cuda:
+            raise RuntimeError("paged attention expects a bf16 device tensor [B, Hq, S, D]")
+        B, hq, S, D = query.shape
+        if B != self.batch or D != self.head_dim or hq % self.num_kv_heads:
+            raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.head_dim}]")
+        if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
+            query = query.contiguous()
+        out = torch.empty((B, hq, S, D), dtype=torch.bfloat16, device=query.device)
+        st = self.state
+        max_len = int(self.lens.max(initial=0))
+        lib = nat.load()
+        ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, self.partition_tokens, self.num_kv_heads))
+        ws = st.workspace(ws_bytes)
+        table, lens_dev = st.device_table(), st.device_lens(self.lens)
+        a = nat.PagedAttnArgs()
+        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = query.data_ptr(), query.stride(0), query.stride(1), query.stride(2)
+        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+        a.block_table, a.table_stride = table.data_ptr(), table.stride(0)
+        a.seq_lens = lens_dev.data_ptr()
+        a.kv_start = None if kv_start is None else kv_start.data_ptr()
+        if attention_mask is not None:
+            m = attention_mask
+            if m.dim() != 4 or m.size(1) != 1 or m.size(0) not in (1, B) or m.size(2) not in (1, S):
+                raise RuntimeError(f"paged attention takes a mask [B|1, 1, S|1, L]; got {tuple(m.shape)}")
+            if m.dtype not in (torch.float32, torch.bfloat16):
+                raise RuntimeError("pace::SDPA attention only support the dtypes Float and BF16 types for input Attention mask")
+            if m.stride(3) != 1:
+                m = m.contiguous()
+            a.mask = m.data_ptr()
+            a.mask_dtype = nat.DTYPE_F32 if m.dtype == torch.float32 else nat.DTYPE_BF16
+            a.mask_len = m.size(3)
+            a.mask_stride_b = 0 if m.size(0) == 1 else m.stride(0)
+            a.mask_stride_s = 0 if m.size(2) == 1 else m.stride(2)
+            a.causal = 0
+        else:
+            a.mask, a.causal = None, 1
+        a.batch, a.num_q_heads, a.q_len = B, hq, S
+        a.max_seq_len, a.partition_tokens = max_len, self.partition_tokens
+        a.scale = 1.0 / math.sqrt(D)
+        a.workspace = None if ws is None else ws.data_ptr()
+        a.workspace_bytes = ws_bytes
+        fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
+        nat.check(fn(ctypes.byref(self._desc), ctypes.byref(a), nat.current_stream_ptr()))
+        return out
+
+
+class KVCacheManager:
+    """One cache per layer, one shared length (reference ``cache.py:48-123``).
+
+    For ``KVCacheType.PAGED`` the layers share one block table; ``num_kv_heads``
+    is taken from ``config.num_key_value_heads`` when the config has it, so the
+    GQA-expanded K/V the reference's models pass in are stored once per KV head.
+    """
+
+    def __init__(self, config, max_seq_length: int, cache_type: Union[str, KVCacheType], **paged_options):
+        self.num_layers = config.num_hidden_layers
+        self.cache_type = cache_type
+        self.kv_cache_class = get_kv_cache_class(cache_type)
+        if self.kv_cache_class is PagedKVCache:
+            shared: dict = {}
+            opts = dict(paged_options)
+            opts.setdefault("num_kv_heads", getattr(config, "num_key_value_heads", None))
+            heads = getattr(config, "num_attention_heads", None)
+            if heads and opts["num_kv_heads"]:
+                opts.setdefault("n_rep", heads // opts["num_kv_heads"])
+            self.cache_objects: List[KVCacheBase] = [
+                PagedKVCache(max_seq_length, shared=shared, **opts) for _ in range(self.num_layers)
+            ]
+            shared["layers"] = self.cache_objects
+        else:
+            self.cache_objects = [self.kv_cache_class(max_seq_length) for _ in range(self.num_layers)]
+
+    def __len__(self) -> int:
+        return int(self.cache_objects[0].seq_len)
+
+    def __getitem__(self, idx: int) -> KVCacheBase:
+        return self.cache_objects[idx]
+
+    def update_mask(self, attn_mask: torch.Tensor, input_size: int) -> torch.Tensor:
+        return self.cache_objects[0].update_mask(attn_mask, input_size)
+
+    def update_cache_with_beam_indices(self, beam_idx: torch.Tensor) -> None:
+        if self.kv_cache_class is PagedKVCache:
+            self.cache_objects[0].update_cache_with_beam_indices(beam_idx)  # moves every layer's blocks
+            return
+        for cache_object in self.cache_objects:
+            cache_object.update_cache_with_beam_indices(beam_idx)
+
+    def remove_cache(self, remove_len: int) -> None:
+        for cache_object in self.cache_objects:
+            cache_object.remove_cache(remove_len)

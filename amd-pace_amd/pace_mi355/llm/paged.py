@@ -1,0 +1,219 @@
+"""Host-side bookkeeping of the block-paged KV store: free list, block tables,
+per-sequence lengths, device mirrors, and the plans for eviction / compaction.
+
+The reference has no paged storage (its caches are contiguous tensors,
+``pace/llm/cache.py:170-400``); this module is the new surface behind the
+reference's ``KVCacheBase`` interface.  All arithmetic here is integer
+bookkeeping on the host; every byte of K/V moves in the HIP kernels.
+"""
+from __future__ import annotations
+
+from typing import Iterable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import _native as nat
+
+BLOCK = nat.BLOCK_TOKENS
+
+
+def blocks_for(n_tokens: int) -> int:
+    return (int(n_tokens) + BLOCK - 1) // BLOCK
+
+
+class BlockAllocator:
+    """LIFO free list over pool block ids ``0 .. num_blocks-1`` (lowest ids first)."""
+
+    def __init__(self, num_blocks: int):
+        self.num_blocks = int(num_blocks)
+        self._free: List[int] = list(range(self.num_blocks - 1, -1, -1))
+        self._is_free = np.ones(self.num_blocks, dtype=bool)
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self, n: int) -> List[int]:
+        if n > len(self._free):
+            raise MemoryError(f"KV block pool exhausted: need {n} blocks, {len(self._free)} free of {self.num_blocks}")
+        out = [self._free.pop() for _ in range(n)]
+        self._is_free[out] = False
+        return out
+
+    def free(self, ids: Iterable[int]) -> None:
+        for i in ids:
+            i = int(i)
+            if self._is_free[i]:
+                raise ValueError(f"block {i} freed twice")
+            self._is_free[i] = True
+            self._free.append(i)
+
+    def take(self, ids: Iterable[int]) -> None:
+        """Mark specific ids as used (compaction destinations)."""
+        want = set(int(i) for i in ids)
+        for i in want:
+            if not self._is_free[i]:
+                raise ValueError(f"block {i} is not free")
+            self._is_free[i] = False
+        self._free = [i for i in self._free if i not in want]
+
+    def free_ids(self) -> np.ndarray:
+        return np.nonzero(self._is_free)[0]
+
+
+class PagedState:
+    """Block tables and lengths of one batch, shared by every layer's pool.
+
+    All layers append the same tokens at the same positions, so one block table
+    serves them all (block ``i`` of every layer's pool belongs to the same
+    sequence range).  Lengths are tracked per call site: a layer passes the
+    lengths it is at, and the device mirror is refreshed only when they differ
+    from what the device already holds.
+    """
+
+    def __init__(self, batch: int, max_seq_length: int, num_blocks: Optional[int], device: torch.device):
+        self.batch = int(batch)
+        self.device = device
+        self.max_blocks_per_seq = max(1, blocks_for(max_seq_length))
+        if num_blocks is None:
+            num_blocks = self.batch * self.max_blocks_per_seq
+        self.allocator = BlockAllocator(num_blocks)
+        self.table = np.zeros((self.batch, self.max_blocks_per_seq), dtype=np.int32)
+        self.n_blocks = np.zeros(self.batch, dtype=np.int64)  # table entries in use per sequence
+        self.pools: List["torch.Tensor"] = []  # one [num_blocks][2][Hkv][16*D] tensor per layer
+        self._table_dev: Optional[torch.Tensor] = None
+        self._table_dirty = True
+        self._lens_dev: Optional[torch.Tensor] = None
+        self._lens_host: Optional[np.ndarray] = None
+        self._workspace: Optional[torch.Tensor] = None
+
+    # -- capacity ---------------------------------------------------------------
+    def _grow_table(self, need_cols: int) -> None:
+        if need_cols <= self.table.shape[1]:
+            return
+        cols = max(need_cols, 2 * self.table.shape[1])
+        grown = np.zeros((self.batch, cols), dtype=np.int32)
+        grown[:, : self.table.shape[1]] = self.table
+        self.table = grown
+        self._table_dirty = True
+        self._table_dev = None
+
+    def ensure_capacity(self, lens: np.ndarray) -> None:
+        """Give every sequence enough blocks to hold ``lens[b]`` tokens."""
+        need = (lens + BLOCK - 1) // BLOCK
+        self._grow_table(int(need.max(initial=0)))
+        for b in np.nonzero(need > self.n_blocks)[0]:
+            have, want = int(self.n_blocks[b]), int(need[b])
+            self.table[b, have:want] = self.allocator.allocate(want - have)
+            self.n_blocks[b] = want
+            self._table_dirty = True
+
+    def release_beyond(self, lens: np.ndarray) -> int:
+        """Free the blocks no token of ``lens`` touches any more; returns how many."""
+        need = (lens + BLOCK - 1) // BLOCK
+        freed = 0
+        for b in np.nonzero(need < self.n_blocks)[0]:
+            have, want = int(self.n_blocks[b]), int(need[b])
+            self.allocator.free(self.table[b, want:have].tolist())
+            self.table[b, want:have] = 0
+            self.n_blocks[b] = want
+            freed += have - want
+            self._table_dirty = True
+        return freed
+
+    # -- device mirrors ---------------------------------------------------------
+    def device_table(self) -> torch.Tensor:
+        if self._table_dev is None or self._table_dirty:
+            host = torch.from_numpy(self.table)
+            if self._table_dev is None or self._table_dev.shape != host.shape:
+                self._table_dev = torch.empty(host.shape, dtype=torch.int32, device=self.device)
+            self._table_dev.copy_(host.pin_memory(), non_blocking=True)
+            self._table_dirty = False
+        return self._table_dev
+
+    def device_lens(self, lens: np.ndarray) -> torch.Tensor:
+        """int32 device tensor holding ``lens``; reuses / advances the cached one."""
+        if self._lens_dev is not None and self._lens_host is not None:
+            delta = lens - self._lens_host
+            if not delta.any():
+                return self._lens_dev
+            if (delta == delta[0]).all():
+                self._lens_dev.add_(int(delta[0]))
+                self._lens_host = lens.copy()
+                return self._lens_dev
+        host = torch.from_numpy(lens.astype(np.int32))
+        if self._lens_dev is None:
+            self._lens_dev = torch.empty(self.batch, dtype=torch.int32, device=self.device)
+        self._lens_dev.copy_(host.pin_memory(), non_blocking=True)
+        self._lens_host = lens.copy()
+        return self._lens_dev
+
+    def workspace(self, nbytes: int) -> Optional[torch.Tensor]:
+        if nbytes == 0:
+            return None
+        if self._workspace is None or self._workspace.numel() < nbytes:
+            self._workspace = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        return self._workspace
+
+    # -- slot arithmetic --------------------------------------------------------
+    def slots(self, starts: np.ndarray, counts: np.ndarray, width: int) -> np.ndarray:
+        """``[B, width]`` int64 slot ids of tokens ``starts[b] .. starts[b]+counts[b]-1``; -1 pads."""
+        out = np.full((self.batch, width), -1, dtype=np.int64)
+        for b in range(self.batch):
+            n = int(counts[b])
+            if n:
+                pos = np.arange(int(starts[b]), int(starts[b]) + n)
+                out[b, :n] = self.table[b, pos // BLOCK].astype(np.int64) * BLOCK + pos % BLOCK
+        return out
+
+    # -- block-level plans ------------------------------------------------------
+    def evict(self, b: int, logical_blocks: Sequence[int], lens: np.ndarray) -> np.ndarray:
+        """Drop the given logical blocks of sequence ``b``: their pool blocks go
+        back to the free list, later table entries shift left, and the length
+        shrinks by the tokens those blocks held.  Returns the new lengths."""
+        n = int(self.n_blocks[b])
+        drop = sorted(set(int(j) for j in logical_blocks))
+        if drop and (drop[0] < 0 or drop[-1] >= n):
+            raise IndexError(f"sequence {b} has {n} blocks; cannot evict {drop}")
+        removed_tokens = sum(min(BLOCK, int(lens[b]) - j * BLOCK) for j in drop)
+        keep = [j for j in range(n) if j not in set(drop)]
+        self.allocator.free(self.table[b, drop].tolist())
+        row = self.table[b, keep].copy()
+        self.table[b, :] = 0
+        self.table[b, : len(keep)] = row
+        self.n_blocks[b] = len(keep)
+        self._table_dirty = True
+        out = lens.copy()
+        out[b] -= removed_tokens
+        return out
+
+    def plan_compaction(self) -> np.ndarray:
+        """Moves that pack all live blocks into ids ``0 .. n_live-1`` with the
+        fewest copies: every live block at or above ``n_live`` moves into a free
+        id below it.  Returns ``[n_moves, 2]`` int32 ``(src, dst)``; the two id
+        sets are disjoint."""
+        live = np.concatenate([self.table[b, : int(self.n_blocks[b])] for b in range(self.batch)] or [np.zeros(0, np.int32)])
+        n_live = live.size
+        src = np.sort(live[live >= n_live])
+        is_live = np.zeros(self.allocator.num_blocks, dtype=bool)
+        is_live[live] = True
+        dst = np.nonzero(~is_live[:n_live])[0]
+        assert src.size == dst.size
+        return np.stack([src, dst], axis=1).astype(np.int32) if src.size else np.zeros((0, 2), np.int32)
+
+    def apply_moves(self, moves: np.ndarray) -> None:
+        """Rewrite the tables and the free list after the data of ``moves`` was copied."""
+        if not len(moves):
+            return
+        remap = np.arange(self.allocator.num_blocks, dtype=np.int32)
+        remap[moves[:, 0]] = moves[:, 1]
+        self.allocator.take(moves[:, 1].tolist())
+        for b in range(self.batch):
+            n = int(self.n_blocks[b])
+            self.table[b, :n] = remap[self.table[b, :n]]
+        self.allocator.free(moves[:, 0].tolist())
+        self._table_dirty = True
+
+    def live_block_count(self) -> int:
+        return int(self.n_blocks.sum())

@@ -1,0 +1,178 @@
+/*
+ * pace_kv_hip.h -- C ABI of the MI355X (gfx950) KV-cache hot path.
+ *
+ * Everything that crosses this boundary is a raw device pointer, an explicit
+ * size/stride, or a plain-old-data struct.  No torch types, no C++ types.
+ * Every entry point enqueues on the HIP stream it is given and returns without
+ * synchronising; it returns 0 on success and a negative code on failure, with
+ * the text of the failure available from pace_kv_last_error() (thread-local).
+ *
+ * Reference interfaces these entry points stand behind (reference repository
+ * paths, file:line):
+ *   - pace::attention torch op          csrc/ops/attention.cpp:18-108
+ *   - kernels::attention_kernel         csrc/ops/kernels/attention_kernels.h:26-32
+ *   - KVCacheBase.update_cache          pace/llm/cache.py:134-143, 268-326, 370-400
+ *   - KVCacheBase.remove_cache          pace/llm/cache.py:224-240, 352-368 (host metadata only)
+ *   - update_cache_with_beam_indices    pace/llm/cache.py:161-167
+ *   - repeat_kv (folded into the kernels) pace/llm/models/llama.py:50-61
+ *
+ * Storage: a block pool.  Block size is 16 tokens.  Per block and KV head the
+ * K slab is token-major  K[token 0..15][dim 0..D-1]  and the V slab is
+ * dim-major  V[dim 0..D-1][token 0..15]  (so that 16 bytes of either slab are
+ * the eight values one matrix-core lane contracts over).  Slabs are addressed
+ * as  base + block * block_stride + head * head_stride  (strides in elements),
+ * which covers both two separate K / V allocations and one interleaved
+ * [block][2][head][...] allocation.  Unwritten slots must hold finite bit
+ * patterns (allocate the pool zero-filled).
+ */
+#ifndef PACE_KV_HIP_H
+#define PACE_KV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PACE_KV_BLOCK_TOKENS 16
+
+enum {
+  PACE_KV_OK = 0,
+  PACE_KV_EINVAL = -1, /* an argument violates the documented contract          */
+  PACE_KV_EHIP = -2,   /* a HIP runtime call failed (launch, attribute query...) */
+};
+
+enum { PACE_DTYPE_F32 = 0, PACE_DTYPE_BF16 = 1 };
+
+typedef struct pace_kv_pool {
+  void* k;                /* bf16, K slabs                                   */
+  void* v;                /* bf16, V slabs (dim-major)                       */
+  int64_t k_block_stride; /* elements between consecutive blocks of K        */
+  int64_t k_head_stride;  /* elements between consecutive KV heads of K      */
+  int64_t v_block_stride;
+  int64_t v_head_stride;
+  int32_t num_blocks;
+  int32_t num_kv_heads;
+  int32_t head_dim;       /* 64 or 128                                       */
+  int32_t block_size;     /* must be PACE_KV_BLOCK_TOKENS                    */
+} pace_kv_pool_t;
+
+/* Text of the last failure on the calling thread ("" if none). */
+const char* pace_kv_last_error(void);
+
+/* ABI version; bumped on any signature change. */
+int32_t pace_kv_abi_version(void);
+
+/*
+ * Append: scatter new tokens into the pool by slot id.
+ * Stands behind KVCacheBase.update_cache (pace/llm/cache.py:268-326, 370-400):
+ * the reference concatenates / narrow-copies [B,H,T,D] onto its contiguous
+ * buffer; here token (b,t) goes to slot_mapping[b*T+t] = block*16 + offset.
+ * k_new / v_new: bf16 [batch][num_kv_heads][n_tokens][head_dim] addressed with
+ * the element strides given (innermost dim contiguous); a GQA-expanded
+ * [B,Hq,T,D] input is deduplicated by passing stride_h * n_rep.
+ * slot_mapping: device int64 [batch*n_tokens]; negative = skip the token.
+ */
+int pace_kv_append(const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
+                   int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                   int32_t batch, int32_t n_tokens, const int64_t* slot_mapping,
+                   void* stream);
+
+/*
+ * Append by position: the same scatter, with the destination of token (b,t)
+ * resolved on the device as position seq_lens[b] + pos_offset + t of sequence
+ * b through the block table, so a decode loop needs no per-step slot upload.
+ * (Pass the lengths after the append with pos_offset = -n_tokens, or the
+ * lengths before it with pos_offset = 0.)  Positions outside the table row or
+ * mapped to a block id outside the pool are skipped.
+ */
+int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
+                         int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                         int32_t batch, int32_t n_tokens,
+                         const int32_t* block_table, int32_t table_stride,
+                         const int32_t* seq_lens, int32_t pos_offset, void* stream);
+
+/*
+ * Gather: block-table walk back into the reference's dense layout.
+ * Produces what the reference cache holds (pace/llm/cache.py:391-399 after
+ * repeat_kv, pace/llm/models/llama.py:151-158): k_out / v_out are bf16
+ * [batch][num_kv_heads*n_rep][out_len][head_dim] with the element strides
+ * given (rows contiguous); rows >= seq_lens[b] are written as zeros.
+ * block_table: device int32 [batch][table_stride]; seq_lens: device int32 [batch].
+ */
+int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                   const int32_t* seq_lens, int32_t batch, int32_t n_rep,
+                   void* k_out, void* v_out, int64_t out_stride_b, int64_t out_stride_h,
+                   int32_t out_len, void* stream);
+
+/*
+ * Copy whole blocks (compaction, beam copy-on-write; the reference's only cache
+ * copy of this kind is index_select, pace/llm/cache.py:161-167).
+ * pairs: device int32 [n_pairs][2] = (src block, dst block).  When src and dst
+ * are the same pool the set of src ids and the set of dst ids must be disjoint.
+ */
+int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst,
+                        const int32_t* pairs, int32_t n_pairs, void* stream);
+
+typedef struct pace_paged_attn_args {
+  const void* q;          /* bf16 [batch][num_q_heads][q_len][head_dim]               */
+  int64_t q_stride_b, q_stride_h, q_stride_s; /* elements; innermost contiguous      */
+  void* out;              /* bf16, same logical shape as q                            */
+  int64_t o_stride_b, o_stride_h, o_stride_s;
+  const int32_t* block_table; /* device int32 [batch][table_stride]                  */
+  int32_t table_stride;
+  const int32_t* seq_lens;    /* device int32 [batch]: tokens in cache incl. the q_len new ones */
+  const int32_t* kv_start;    /* optional device int32 [batch]: first readable token (left padding) */
+  const void* mask;           /* optional additive mask [batch|1][1][q_len|1][mask_len]  */
+  int32_t mask_dtype;         /* PACE_DTYPE_F32 / PACE_DTYPE_BF16                      */
+  int32_t mask_len;           /* columns in the mask; tokens >= mask_len are masked    */
+  int64_t mask_stride_b, mask_stride_s; /* elements; 0 for a broadcast dim            */
+  int32_t batch, num_q_heads, q_len;
+  int32_t causal;             /* 1: query row s reads tokens <= seq_len - q_len + s    */
+  int32_t max_seq_len;        /* host-side upper bound of seq_lens (sizes the grid)    */
+  int32_t partition_tokens;   /* context split size, multiple of 32, <= 1024; 0 = auto */
+  float scale;                /* softmax scale, reference uses 1/sqrt(head_dim)        */
+  void* workspace;            /* device scratch, >= pace_paged_attn_workspace_bytes()  */
+  size_t workspace_bytes;
+} pace_paged_attn_args_t;
+
+/* Scratch bytes the two entry points below need for these sizes (0 = none). */
+size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len,
+                                       int32_t head_dim, int32_t max_seq_len,
+                                       int32_t partition_tokens, int32_t num_kv_heads);
+
+/*
+ * Decode attention over the paged cache, q_len == 1.
+ * Stands behind MultiHeadAttention.forward -> backend.execute
+ * (pace/ops/attention.py:29-38, pace/ops/backends/native.py:44-47,
+ * pace/ops/backends/jit.py:43-47) for one new token per sequence.
+ */
+int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream);
+
+/*
+ * Multi-token (speculative verify / chunked prefill) attention over the paged
+ * cache: q_len >= 1 new tokens per sequence already appended; causal among
+ * themselves (the mask pace/llm/models/llama.py:292-299 builds for q_len > 1).
+ */
+int pace_paged_attn_verify(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream);
+
+/*
+ * Dense attention: body of the torch op
+ *   pace::attention(Tensor input_Q, Tensor input_K, Tensor input_V,
+ *                   Tensor? input_mask, Scalar? use_KQ) -> Tensor
+ * (csrc/ops/attention.cpp:18-108; kernel csrc/ops/kernels/attention_kernels.cpp:162-257).
+ * q [B][N][S][H], k/v [B][N][L][H] and out [B][N][S][H] are dense row-major as
+ * the reference requires (csrc/pace_tensor/pace_aten_interface.cpp:151-179);
+ * mask is an additive [mB][mN][mS][L] tensor, each of mB/mN/mS either 1 or the
+ * full extent.  qkv_dtype / mask_dtype: PACE_DTYPE_*.  out has qkv_dtype.
+ */
+int pace_attn_dense(const void* q, const void* k, const void* v, void* out,
+                    int32_t qkv_dtype, int32_t B, int32_t N, int32_t S, int32_t L, int32_t H,
+                    const void* mask, int32_t mask_dtype, int32_t mB, int32_t mN, int32_t mS,
+                    void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PACE_KV_HIP_H */

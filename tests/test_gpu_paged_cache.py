@@ -1,0 +1,139 @@
+"""GPU parity: paged append / gather / truncate / evict / compact / beam reorder,
+bit-exact against the contiguous-semantics oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bits_equal, seeded_kv
+from oracle.cache_ref import DynamicKVCacheRef, repeat_kv, valid_prefix
+from oracle.paged_ref import RaggedCacheModel
+
+pytestmark = pytest.mark.gpu
+
+
+def _paged(max_len, **kw):
+    from pace_mi355.llm import PagedKVCache
+
+    return PagedKVCache(max_len, **kw)
+
+
+@pytest.mark.parametrize("hkv,n_rep,dim", [(8, 4, 128), (2, 1, 64), (4, 8, 128)])
+def test_append_matches_reference_dynamic_cache(device, hkv, n_rep, dim):
+    """Feed the same GQA-expanded stream to the reference's DynamicKVCache restatement
+    and to the paged cache; gather(expand) must equal the reference tensors bit for bit."""
+    B = 3
+    ref = DynamicKVCacheRef(256)
+    cache = _paged(256, num_kv_heads=hkv, n_rep=n_rep)
+    for step, T in enumerate([37, 1, 1, 16, 5, 1]):
+        k, v = seeded_kv(100 + step, B, hkv, T, dim)
+        k_exp, v_exp = repeat_kv(k, n_rep), repeat_kv(v, n_rep)
+        rk, rv = ref.update_cache(k_exp, v_exp, concat_dim=2)
+        pk, pv = cache.update_cache(k_exp.to(device), v_exp.to(device), concat_dim=2)
+        assert cache.seq_len == ref.seq_len
+        assert_bits_equal(pk.dense(), rk, f"K after step {step}")
+        assert_bits_equal(pv.dense(), rv, f"V after step {step}")
+    ref.remove_cache(7)
+    cache.remove_cache(7)
+    rk, rv = valid_prefix(ref)
+    assert_bits_equal(cache.key.dense(), rk, "K after remove_cache")
+    assert_bits_equal(cache.value.dense(), rv, "V after remove_cache")
+    with pytest.raises(ValueError, match="Cannot remove more tokens than available in cache."):
+        cache.remove_cache(10_000)
+    with pytest.raises(AssertionError, match="concat_dim should be the same"):
+        cache.update_cache(k_exp.to(device), v_exp.to(device), concat_dim=1)
+
+
+def test_append_from_transposed_views(device):
+    """The models hand in [B,T,H,D] storage viewed as [B,H,T,D] (llama.py:125-138)."""
+    B, H, T, D = 2, 4, 9, 128
+    g = torch.Generator().manual_seed(7)
+    base_k = torch.randn(B, T, H, D, generator=g).to(torch.bfloat16)
+    base_v = torch.randn(B, T, H, D, generator=g).to(torch.bfloat16)
+    cache = _paged(64)
+    pk, pv = cache.update_cache(base_k.to(device).transpose(1, 2), base_v.to(device).transpose(1, 2), concat_dim=2)
+    assert_bits_equal(pk.dense(), base_k.transpose(1, 2).contiguous(), "K")
+    assert_bits_equal(pv.dense(), base_v.transpose(1, 2).contiguous(), "V")
+
+
+def test_ragged_append_truncate_evict_compact(device):
+    B, H, D = 5, 2, 128
+    rng = np.random.default_rng(11)
+    cache = _paged(400, num_blocks=160)
+    model = RaggedCacheModel(B, H, D)
+    for step in range(6):
+        T = int(rng.integers(1, 40))
+        counts = rng.integers(0, T + 1, size=B)
+        k, v = seeded_kv(200 + step, B, H, T, D)
+        cache.append_ragged(k.to(device), v.to(device), counts)
+        model.append(k, v, counts)
+        assert cache.lens.tolist() == model.seq_lens()
+    def check(tag):
+        K, V = model.dense()
+        gk, gv = cache.gather()
+        assert_bits_equal(gk, K, f"K {tag}")
+        assert_bits_equal(gv, V, f"V {tag}")
+    check("after ragged appends")
+    rem = [int(rng.integers(0, min(9, n + 1))) for n in model.seq_lens()]
+    cache.truncate(rem)
+    model.truncate(rem)
+    check("after truncate")
+    for b in range(B):
+        nb = (model.seq_lens()[b] + 15) // 16
+        drop = sorted(rng.choice(nb, size=nb * 2 // 5, replace=False).tolist()) if nb else []
+        cache.evict_blocks(b, drop)
+        model.evict_blocks(b, drop, 16)
+    assert cache.lens.tolist() == model.seq_lens()
+    check("after evict")
+    moved = cache.compact()
+    live = cache.state.live_block_count()
+    used = np.concatenate([cache.state.table[b, : cache.state.n_blocks[b]] for b in range(B)])
+    assert sorted(used.tolist()) == list(range(live)), "live blocks must occupy ids 0..n_live-1"
+    assert moved <= live
+    check("after compact")
+    # appending after compaction reuses freed ids correctly
+    k, v = seeded_kv(300, B, H, 20, D)
+    cache.append_ragged(k.to(device), v.to(device), [20] * B)
+    model.append(k, v)
+    check("after post-compaction append")
+
+
+def test_beam_reorder(device):
+    B, H, D = 4, 2, 64
+    cache = _paged(128, num_blocks=80)
+    model = RaggedCacheModel(B, H, D)
+    k, v = seeded_kv(5, B, H, 45, D)
+    cache.update_cache(k.to(device), v.to(device), 2)
+    model.append(k, v)
+    idx = [2, 2, 0, 3]
+    cache.update_cache_with_beam_indices(torch.tensor(idx))
+    model.reorder(idx)
+    K, V = model.dense()
+    gk, gv = cache.gather()
+    assert_bits_equal(gk, K, "K after beam reorder")
+    assert_bits_equal(gv, V, "V after beam reorder")
+
+
+def test_manager_layers_share_block_table(device):
+    from pace_mi355.llm import KVCacheManager, KVCacheType
+
+    class Cfg:
+        num_hidden_layers = 2
+        num_attention_heads = 8
+        num_key_value_heads = 2
+
+    mgr = KVCacheManager(Cfg(), 96, KVCacheType.PAGED)
+    refs = [DynamicKVCacheRef(96) for _ in range(2)]
+    for step, T in enumerate([30, 1, 1]):
+        for layer in range(2):
+            k, v = seeded_kv(400 + 10 * step + layer, 2, 2, T, 128)
+            ke, ve = repeat_kv(k, 4), repeat_kv(v, 4)
+            refs[layer].update_cache(ke, ve, 2)
+            mgr[layer].update_cache(ke.to(device), ve.to(device), 2)
+        assert len(mgr) == refs[0].seq_len
+    mgr.remove_cache(3)
+    for layer in range(2):
+        refs[layer].remove_cache(3)
+        rk, rv = valid_prefix(refs[layer])
+        assert_bits_equal(mgr[layer].key.dense(), rk, f"layer {layer} K")
+        assert_bits_equal(mgr[layer].value.dense(), rv, f"layer {layer} V")
+    assert mgr[0].state is mgr[1].state
