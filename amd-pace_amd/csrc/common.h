@@ -38,6 +38,23 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
+// Element offsets inside one (block, head) slab of 16 tokens x D dims.
+// K slab  [tile 2][dim chunk D/8][token slot 8][dim 8]   with token -> (tile, slot):
+//         tile = (tok >> 2) & 1,  slot = ((tok >> 3) << 2) | (tok & 3)
+// V slab  [dim tile D/16][token half 2][dim 16][token 8]
+// Both make every 16-lane quarter of a wavefront-wide 16-byte load read one
+// contiguous run (128 B per block for K, 256 B for V) in the operand order of
+// the 16x16x32 matrix-core instruction.
+template <int D>
+__host__ __device__ __forceinline__ int k_slab_offset(int tok, int dim) {
+  const int tile = (tok >> 2) & 1, slot = ((tok >> 3) << 2) | (tok & 3);
+  return tile * (D * 8) + (dim >> 3) * 64 + slot * 8 + (dim & 7);
+}
+template <int D>
+__host__ __device__ __forceinline__ int v_slab_offset(int tok, int dim) {
+  return (((dim >> 4) * 2 + (tok >> 3)) * 16 + (dim & 15)) * 8 + (tok & 7);
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
 // Round-to-nearest-even fp32 -> bf16 bits (NaN stays NaN).

@@ -7,8 +7,8 @@ namespace pace_kv {
 
 // ---------------------------------------------------------------------------------
 // Append.  One thread moves eight dims (16 bytes) of one (token, head) row of K and
-// of V.  K keeps its row shape; V is written dim-major, so its eight values land 32
-// bytes apart (one per dim) at the token's column.
+// of V.  The K chunk stays one 16-byte store; the V chunk is written token-minor, so
+// its eight values land 16 bytes apart (one per dim) at the token's column.
 // ---------------------------------------------------------------------------------
 // Where the tokens go: either an explicit slot id per token, or "position
 // seq_lens[b] + pos_offset + t of sequence b" resolved through the block table.
@@ -52,21 +52,22 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
   const u32x4 kv = *reinterpret_cast<const u32x4*>(k_new + src);
   const u32x4 vv = *reinterpret_cast<const u32x4*>(v_new + src);
   uint16_t* kdst = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride +
-                   (int64_t)off * D + chunk * 8;
+                   k_slab_offset<D>(off, chunk * 8);
   *reinterpret_cast<u32x4*>(kdst) = kv;
+  // The eight dims of this chunk sit 8 elements apart in the V slab (same dim tile).
   uint16_t* vdst = reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride +
-                   (int64_t)(chunk * 8) * PACE_KV_BLOCK_TOKENS + off;
+                   v_slab_offset<D>(off, chunk * 8);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    vdst[(2 * j) * PACE_KV_BLOCK_TOKENS] = (uint16_t)(vv[j] & 0xffffu);
-    vdst[(2 * j + 1) * PACE_KV_BLOCK_TOKENS] = (uint16_t)(vv[j] >> 16);
+    vdst[(2 * j) * 8] = (uint16_t)(vv[j] & 0xffffu);
+    vdst[(2 * j + 1) * 8] = (uint16_t)(vv[j] >> 16);
   }
 }
 
 // ---------------------------------------------------------------------------------
 // Gather.  One 256-thread workgroup rebuilds one logical block (16 tokens) of one KV
-// head of one sequence in the dense [B][H*n_rep][L][D] layout.  K slabs are copied
-// as they are; V slabs are staged in LDS and read back transposed.
+// head of one sequence in the dense [B][H*n_rep][L][D] layout.  K chunks are read
+// from their slab position; V slabs are staged in LDS and read back transposed.
 // ---------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
@@ -97,11 +98,11 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
     if (t >= out_len) continue;
     u32x4 kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
     if (t < len) {
-      kv = *reinterpret_cast<const u32x4*>(ksrc + c * 8);
+      kv = *reinterpret_cast<const u32x4*>(ksrc + k_slab_offset<D>(tok, chunk * 8));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const uint32_t lo = vt[(chunk * 8 + 2 * e) * PACE_KV_BLOCK_TOKENS + tok];
-        const uint32_t hi = vt[(chunk * 8 + 2 * e + 1) * PACE_KV_BLOCK_TOKENS + tok];
+        const uint32_t lo = vt[v_slab_offset<D>(tok, chunk * 8 + 2 * e)];
+        const uint32_t hi = vt[v_slab_offset<D>(tok, chunk * 8 + 2 * e + 1)];
         vv[e] = lo | (hi << 16);
       }
     }

@@ -15,11 +15,13 @@
 //   the scores of tokens 8g..8g+7 of the unit for query row n -- exactly the B
 //   operand slot of the second product:
 //   O^T tile  = V^T[16 dims x 32 tokens] * P^T[32 tokens x 16 rows]
-//       A operand: lane (n, g) holds 16 bytes of the dim-major V slab: dim 16j+n,
+//       A operand: lane (n, g) holds 16 bytes of the token-minor V slab: dim 16j+n,
 //                  tokens 8g..8g+7 of the unit  (one coalesced 16-byte load)
 //   so probabilities never leave their lane between the two products, and the
 //   softmax state (running max, sum, output accumulators) of query row n lives
 //   in the four lanes (n, 0..3).
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace pace_kv {
@@ -67,19 +69,21 @@ struct UnitRegs {
 template <int D>
 __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n,
                                           int g) {
-  // K: lane (n, g) reads token 8*(n/4) + 4*tile + n%4 of the unit.
-  const int tok0 = 8 * (n >> 2) + (n & 3);  // tile 0; tile 1 is +4
+  // K: lane (n, g) supplies token 8*(n/4) + 4*tile + n%4 of the unit, i.e. token slot
+  // n % 8 of slab tile `tile` in block A (n < 8) or B; dims 32*kk + 8g .. +8 are dim
+  // chunk 4*kk + g.  A 16-lane quarter (fixed g) reads 128 contiguous bytes per block.
   const int64_t kblk = (n >= 8) ? idB : idA;
-  const uint16_t* kp = p.kpool + kblk * p.k_bs + (int64_t)kvh * p.k_hs + (tok0 & 15) * D + 8 * g;
+  const uint16_t* kp = p.kpool + kblk * p.k_bs + (int64_t)kvh * p.k_hs + g * 64 + (n & 7) * 8;
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + t * 4 * D + kk * 32);
-  // V: lane (n, g) reads dim 16j + n, tokens 8g..8g+7 of the unit.
+    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + t * (D * 8) + kk * 256);
+  // V: lane (n, g) supplies dim 16j + n, tokens 8g..8g+7 of the unit: token half g & 1
+  // of block A (g < 2) or B.  A 16-lane quarter reads 256 contiguous bytes.
   const int64_t vblk = (g >= 2) ? idB : idA;
-  const uint16_t* vp = p.vpool + vblk * p.v_bs + (int64_t)kvh * p.v_hs + n * PACE_KV_BLOCK_TOKENS + 8 * (g & 1);
+  const uint16_t* vp = p.vpool + vblk * p.v_bs + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
 #pragma unroll
-  for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 16 * PACE_KV_BLOCK_TOKENS);
+  for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
 }
 
 template <int D, int NQT>
@@ -97,6 +101,17 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (
                                              int start, bool full, int g) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
+#ifdef PACE_PROBE_LOADS_ONLY
+  {  // measurement aid: keep the loads, drop the arithmetic
+    u32x4 x = {0u, 0u, 0u, 0u};
+    for (int t = 0; t < 2; ++t)
+      for (int kk = 0; kk < KK; ++kk) x ^= r.k[t][kk];
+    for (int j = 0; j < MT; ++j) x ^= r.v[j];
+    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
+    st.l[0] = 1.f;
+    return;
+  }
+#endif
   // Zero V columns past the end of the sequence so that stale pool contents
   // (possibly non-finite bit patterns) cannot reach the accumulators.
   u32x4 vreg[MT];
@@ -192,21 +207,43 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (
   }
 }
 
-template <int D, int NQT, bool HAS_MASK>
-__global__ __launch_bounds__(64) void paged_attn_kernel(const PagedAttnParams p) {
+// Pool block ids of one wave's token range: up to 128 blocks (2048 tokens), one id per
+// lane in each of two registers, fetched with one coalesced load each and read back
+// with v_readlane (no memory access inside the unit loop).
+struct WaveBlockIds {
+  int lo, hi;
+  __device__ __forceinline__ int get(int idx) const {  // idx is wave-uniform
+    return idx < 64 ? __builtin_amdgcn_readlane(lo, idx) : __builtin_amdgcn_readlane(hi, idx - 64);
+  }
+};
+
+// NW waves per workgroup split the partition's units among themselves and merge their
+// softmax states through LDS; NBUF unit buffers per wave are kept in flight.
+// OCC is the number of such waves that must fit on one SIMD (caps the register budget).
+template <int D, int NQT, bool HAS_MASK, int NW, int NBUF, int OCC>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void paged_attn_kernel(
+    const PagedAttnParams p) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+  static_assert(NW * NQT <= 8, "LDS merge buffer holds 64 query rows");
+  __shared__ float merge_buf[64 * (D + 2)];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int part = blockIdx.x, kvh = blockIdx.y;
   const int b = blockIdx.z / p.n_qgroups, qg = blockIdx.z % p.n_qgroups;
   const int len = p.seq_lens[b];
   const int P = p.part_tokens;
   const int n_parts = len > 0 ? (len + P - 1) / P : 1;
-  if (part >= n_parts) return;
+  if (part >= n_parts) return;  // uniform over the workgroup
   const int start = p.kv_start ? p.kv_start[b] : 0;
-  const int tok_begin = part * P;
-  const int tok_end = min(len, tok_begin + P);
+  const int part_begin = part * P;
+  const int tok_end = min(len, part_begin + P);
   const int S = p.q_len, R = S * p.n_rep;
+  // This wave's share of the partition's 32-token units.
+  const int part_units = (tok_end - part_begin + 31) / 32;
+  const int per_wave = (part_units + NW - 1) / NW;
+  const int u_begin = min(part_units, wave * per_wave);
+  const int n_units = min(part_units, u_begin + per_wave) - u_begin;
+  const int tok_begin = part_begin + 32 * u_begin;
 
   // Query rows of this wave (B operand of the first product) and per-row limits.
   u32x4 qreg[NQT][KK];
@@ -241,41 +278,100 @@ __global__ __launch_bounds__(64) void paged_attn_kernel(const PagedAttnParams p)
   min_limit = min(min_limit, __shfl_xor(min_limit, 4, 64));
   min_limit = min(min_limit, __shfl_xor(min_limit, 8, 64));
 
-  // Pool block ids of this partition, one per lane (partition <= 64 blocks).
-  const int first_blk = tok_begin / PACE_KV_BLOCK_TOKENS;
-  const int live_blks = (len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
-  int my_id = 0;
-  if (first_blk + lane < live_blks) my_id = p.table[(int64_t)b * p.table_stride + first_blk + lane];
-  my_id = my_id < 0 ? 0 : (my_id >= p.num_blocks ? p.num_blocks - 1 : my_id);  // never read outside the pool
+  WaveBlockIds ids;
+  {
+    const int first_blk = tok_begin / PACE_KV_BLOCK_TOKENS;
+    const int live_blks = (len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
+    const int32_t* row = p.table + (int64_t)b * p.table_stride;
+    int lo = 0, hi = 0;
+    if (n_units > 0 && first_blk + lane < live_blks) lo = row[first_blk + lane];
+    if (n_units > 32 && first_blk + 64 + lane < live_blks) hi = row[first_blk + 64 + lane];
+    // never read outside the pool, whatever the table holds
+    ids.lo = lo < 0 ? 0 : (lo >= p.num_blocks ? p.num_blocks - 1 : lo);
+    ids.hi = hi < 0 ? 0 : (hi >= p.num_blocks ? p.num_blocks - 1 : hi);
+  }
 
-  const int n_units = (tok_end - tok_begin + 31) / 32;
-  UnitRegs<D> bufA, bufB;
-  if (n_units > 0) load_unit<D>(bufA, p, kvh, __builtin_amdgcn_readlane(my_id, 0), __builtin_amdgcn_readlane(my_id, 1), n, g);
-  for (int u = 0; u < n_units; u += 2) {
-    const int t0 = tok_begin + 32 * u;
-    if (u + 1 < n_units)
-      load_unit<D>(bufB, p, kvh, __builtin_amdgcn_readlane(my_id, 2 * u + 2), __builtin_amdgcn_readlane(my_id, 2 * u + 3), n,
-                   g);
-    {
-      const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
-      compute_unit<D, NQT, HAS_MASK>(bufA, qreg, st, p, t0, tok_end, start, full, g);
+  UnitRegs<D> buf[NBUF];
+#pragma unroll
+  for (int i = 0; i < NBUF - 1; ++i)
+    if (i < n_units) load_unit<D>(buf[i], p, kvh, ids.get(2 * i), ids.get(2 * i + 1), n, g);
+  for (int u = 0; u < n_units; u += NBUF) {
+#pragma unroll
+    for (int j = 0; j < NBUF; ++j) {
+      const int uu = u + j;
+      if (uu < n_units) {
+        const int un = uu + NBUF - 1;  // unit to put in flight now
+        if (un < n_units) load_unit<D>(buf[(j + NBUF - 1) % NBUF], p, kvh, ids.get(2 * un), ids.get(2 * un + 1), n, g);
+        const int t0 = tok_begin + 32 * uu;
+        const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
+        compute_unit<D, NQT, HAS_MASK>(buf[j], qreg, st, p, t0, tok_end, start, full, g);
+      }
     }
-    if (u + 1 < n_units) {
-      if (u + 2 < n_units)
-        load_unit<D>(bufA, p, kvh, __builtin_amdgcn_readlane(my_id, 2 * u + 4), __builtin_amdgcn_readlane(my_id, 2 * u + 5),
-                     n, g);
-      const int t1 = t0 + 32;
-      const bool full = (t1 + 32 <= tok_end) && (t1 + 31 <= min_limit) && (t1 >= start);
-      compute_unit<D, NQT, HAS_MASK>(bufB, qreg, st, p, t1, tok_end, start, full, g);
+  }
+
+  // Row sums were kept per lane; complete them over the four lanes of a row.
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float l = st.l[qt];
+    l += xor_lanes(l, 16);
+    l += xor_lanes(l, 32);
+    st.l[qt] = l;
+  }
+
+  // Pairwise merge of the waves' states through LDS (fixed order: deterministic).
+  if (NW > 1) {
+    constexpr int ROW_F = D + 2;
+    constexpr int SLOT_F = 16 * NQT * ROW_F;
+#pragma unroll
+    for (int stride = 1; stride < NW; stride *= 2) {
+      const int slot = wave / (2 * stride);
+      const bool sender = (wave & (2 * stride - 1)) == stride;
+      const bool receiver = (wave & (2 * stride - 1)) == 0 && wave + stride < NW;
+      if (sender) {
+#pragma unroll
+        for (int qt = 0; qt < NQT; ++qt) {
+          float* rowp = merge_buf + slot * SLOT_F + (qt * 16 + n) * ROW_F;
+#pragma unroll
+          for (int j = 0; j < MT; ++j) {
+            rowp[16 * j + 4 * g + 0] = st.o[qt][j][0];
+            rowp[16 * j + 4 * g + 1] = st.o[qt][j][1];
+            rowp[16 * j + 4 * g + 2] = st.o[qt][j][2];
+            rowp[16 * j + 4 * g + 3] = st.o[qt][j][3];
+          }
+          if (g == 0) {
+            rowp[D] = st.m[qt];
+            rowp[D + 1] = st.l[qt];
+          }
+        }
+      }
+      __syncthreads();
+      if (receiver) {
+#pragma unroll
+        for (int qt = 0; qt < NQT; ++qt) {
+          const float* rowp = merge_buf + slot * SLOT_F + (qt * 16 + n) * ROW_F;
+          const float m_b = rowp[D], l_b = rowp[D + 1];
+          const float m_new = fmaxf(st.m[qt], m_b);
+          const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+          const float wa = __builtin_amdgcn_exp2f(st.m[qt] - m_use);
+          const float wb = __builtin_amdgcn_exp2f(m_b - m_use);
+#pragma unroll
+          for (int j = 0; j < MT; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) st.o[qt][j][i] = st.o[qt][j][i] * wa + rowp[16 * j + 4 * g + i] * wb;
+          }
+          st.l[qt] = st.l[qt] * wa + l_b * wb;
+          st.m[qt] = m_new;
+        }
+      }
+      __syncthreads();
     }
+    if (wave != 0) return;
   }
 
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     const int r = (qg * NQT + qt) * 16 + n;
-    float l = st.l[qt];
-    l += xor_lanes(l, 16);
-    l += xor_lanes(l, 32);
+    const float l = st.l[qt];
     if (r >= R) continue;
     if (p.max_parts == 1) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -336,30 +432,68 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   }
 }
 
-static int auto_partition(int32_t max_seq_len, int64_t waves_per_partition_row) {
-  // Aim for about eight resident waves per compute unit (256 CUs); never split
-  // finer than 128 tokens, never coarser than 1024 (64 pool blocks, one id per lane).
-  const int64_t target_waves = 2048;
-  int64_t per = ((int64_t)max_seq_len * waves_per_partition_row + target_waves - 1) / target_waves;
-  per = (per + 31) / 32 * 32;
-  if (per < 128) per = 128;
-  if (per > 1024) per = 1024;
+// Launch shape per query-tile count: waves per workgroup and unit buffers per wave.
+struct Shape {
+  int nqt, nw, nbuf, occ;
+};
+
+static Shape shape_for(int tiles) {
+  if (tiles <= 1) {
+    Shape s = {1, 4, 1, 2};
+    // Tuning override for the single-tile (decode) kernel: "NW,NBUF,OCC".
+    if (const char* e = getenv("PACE_KV_DECODE_SHAPE")) {
+      int nw = 0, nbuf = 0, occ = 0;
+      if (sscanf(e, "%d,%d,%d", &nw, &nbuf, &occ) == 3) s.nw = nw, s.nbuf = nbuf, s.occ = occ;
+    }
+    return s;
+  }
+  if (tiles == 2) return Shape{2, 4, 1, 2};
+  return Shape{4, 2, 1, 1};
+}
+
+// Tokens one workgroup may cover: each wave holds at most 128 block ids.
+static int max_partition(int nw) { return nw * 2048; }
+
+static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
+  const int tiles = (rows + 15) / 16;
+  const Shape sh = shape_for(tiles);
+  const int granule = 32 * sh.nw;
+  if (requested > 0) return requested;
+  // Enough workgroups to give every compute unit (256) two of them; a batch that
+  // already does so is not split at all.
+  const int64_t groups = (int64_t)batch * num_kv_heads * ((tiles + sh.nqt - 1) / sh.nqt);
+  int64_t parts = (512 + groups - 1) / groups;
+  if (parts < 1) parts = 1;
+  int64_t per = ((int64_t)max_seq_len + parts - 1) / parts;
+  per = (per + granule - 1) / granule * granule;
+  if (per < granule) per = granule;
+  if (per > max_partition(sh.nw)) per = max_partition(sh.nw);
   return (int)per;
 }
 
-static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
-  if (requested > 0) return requested;
-  const int nqt_rows = 64;
-  const int64_t groups = (rows + nqt_rows - 1) / nqt_rows;
-  return auto_partition(max_seq_len, (int64_t)batch * num_kv_heads * groups);
-}
-
-template <int D, int NQT>
+template <int D, int NQT, int NW, int NBUF, int OCC>
 static void launch(const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
   if (has_mask)
-    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, true>), grid, dim3(64), 0, s, p);
+    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, true, NW, NBUF, OCC>), grid, dim3(64 * NW), 0, s, p);
   else
-    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, false>), grid, dim3(64), 0, s, p);
+    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, false, NW, NBUF, OCC>), grid, dim3(64 * NW), 0, s, p);
+}
+
+template <int D>
+static bool launch_shape(const Shape& sh, const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
+#define PACE_TRY(NQT_, NW_, NBUF_, OCC_)                                         \
+  if (sh.nqt == NQT_ && sh.nw == NW_ && sh.nbuf == NBUF_ && sh.occ == OCC_) {       \
+    launch<D, NQT_, NW_, NBUF_, OCC_>(p, grid, has_mask, s);                        \
+    return true;                                                                    \
+  }
+  PACE_TRY(1, 4, 1, 2)
+  PACE_TRY(1, 4, 1, 3)
+  PACE_TRY(1, 8, 1, 2)
+  PACE_TRY(1, 4, 2, 1)
+  PACE_TRY(2, 4, 1, 2)
+  PACE_TRY(4, 2, 1, 1)
+#undef PACE_TRY
+  return false;
 }
 
 static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, void* stream, const char* who) {
@@ -387,9 +521,11 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   }
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
+  const int tiles = (rows + 15) / 16;
+  const Shape sh = shape_for(tiles);
   const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
-  PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= 1024, "%s: partition_tokens %d must be a multiple of 32 in [32, 1024]",
-               who, part);
+  PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
+               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, max_partition(sh.nw));
   const int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
 
   PagedAttnParams p;
@@ -411,11 +547,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.part_tokens = part, p.max_parts = max_parts;
   p.scale_log2 = a->scale * kLog2e;
   p.part_o = nullptr, p.part_ml = nullptr;
-
-  // Query-row tiles per wave: 1 for plain decode with n_rep <= 16, up to 4.
-  const int tiles = (rows + 15) / 16;
-  const int nqt = tiles >= 4 ? 4 : (tiles == 3 ? 4 : tiles);
-  p.n_qgroups = (tiles + nqt - 1) / nqt;
+  p.n_qgroups = (tiles + sh.nqt - 1) / sh.nqt;
 
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
@@ -430,15 +562,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   dim3 grid(max_parts, pool->num_kv_heads, a->batch * p.n_qgroups);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
-  if (pool->head_dim == 128) {
-    if (nqt == 1) launch<128, 1>(p, grid, has_mask, s);
-    else if (nqt == 2) launch<128, 2>(p, grid, has_mask, s);
-    else launch<128, 4>(p, grid, has_mask, s);
-  } else {
-    if (nqt == 1) launch<64, 1>(p, grid, has_mask, s);
-    else if (nqt == 2) launch<64, 2>(p, grid, has_mask, s);
-    else launch<64, 4>(p, grid, has_mask, s);
-  }
+  const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, grid, has_mask, s) : launch_shape<64>(sh, p, grid, has_mask, s);
+  PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d nbuf=%d occ=%d", who, sh.nqt, sh.nw, sh.nbuf, sh.occ);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;

@@ -172,21 +172,22 @@ class PagedKVCache(KVCacheBase):
         if self.state.batch != B:
             raise RuntimeError(f"batch changed from {self.state.batch} to {B}")
         nb = self.state.allocator.num_blocks
-        # [block][K|V][head][16*D]: one block of one layer is contiguous.
-        self.pool = torch.zeros((nb, 2, hkv, BLOCK * D), dtype=torch.bfloat16, device=key_states.device)
+        # [block][head][K|V][16*D]: one block of one layer is contiguous (64 KiB at 8 heads x 128 dims)
+        # and the K and V slabs a wavefront reads together are adjacent.
+        self.pool = torch.zeros((nb, hkv, 2, BLOCK * D), dtype=torch.bfloat16, device=key_states.device)
         self.state.pools.append(self.pool)
         self._desc = self._describe(self.pool)
         self.lens = np.zeros(B, dtype=np.int64)
 
     def _describe(self, pool: torch.Tensor) -> nat.PoolDesc:
-        nb, _, hkv, slab = pool.shape
+        nb, hkv, _, slab = pool.shape
         return nat.PoolDesc(
-            k=pool[:, 0].data_ptr(),
-            v=pool[:, 1].data_ptr(),
+            k=pool[:, :, 0].data_ptr(),
+            v=pool[:, :, 1].data_ptr(),
             k_block_stride=pool.stride(0),
-            k_head_stride=pool.stride(2),
+            k_head_stride=pool.stride(1),
             v_block_stride=pool.stride(0),
-            v_head_stride=pool.stride(2),
+            v_head_stride=pool.stride(1),
             num_blocks=nb,
             num_kv_heads=hkv,
             head_dim=slab // BLOCK,

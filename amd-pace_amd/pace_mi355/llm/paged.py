@@ -81,7 +81,7 @@ class PagedState:
         self.allocator = BlockAllocator(num_blocks)
         self.table = np.zeros((self.batch, self.max_blocks_per_seq), dtype=np.int32)
         self.n_blocks = np.zeros(self.batch, dtype=np.int64)  # table entries in use per sequence
-        self.pools: List["torch.Tensor"] = []  # one [num_blocks][2][Hkv][16*D] tensor per layer
+        self.pools: List["torch.Tensor"] = []  # one [num_blocks][Hkv][2][16*D] tensor per layer
         self._table_dev: Optional[torch.Tensor] = None
         self._table_dirty = True
         self._lens_dev: Optional[torch.Tensor] = None

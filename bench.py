@@ -38,7 +38,7 @@ def algorithmic_bytes(batch, ctx_after, q_heads, kv_heads, head_dim, new_tokens=
     return decode, append
 
 
-def build_cache(torch, dev, w, seed=1):
+def build_cache(torch, dev, w, seed=1, permute=True):
     """Cache holding `context` tokens per sequence in randomly permuted physical blocks."""
     import numpy as np
     from pace_mi355.llm import PagedKVCache
@@ -58,7 +58,10 @@ def build_cache(torch, dev, w, seed=1):
             cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)
             alloc = cache.state.allocator
             ids = alloc.allocate(alloc.num_free)
-            np.random.default_rng(seed).shuffle(ids)
+            if permute:
+                np.random.default_rng(seed).shuffle(ids)
+            else:
+                ids = ids[::-1]
             alloc.free(ids)
             first = False
         cache.update_cache(k, v, 2)
@@ -124,6 +127,7 @@ def main() -> int:
                     help="direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + MultiHeadAttention")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-permute", action="store_true", help="keep physical blocks in logical order (diagnostic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by "
@@ -143,7 +147,7 @@ def main() -> int:
     torch.cuda.set_device(dev)
     w = WORKLOAD
     B, ctx, hq, hkv, D = w["batch"], w["context"], w["q_heads"], w["kv_heads"], w["head_dim"]
-    cache = build_cache(torch, dev, w)
+    cache = build_cache(torch, dev, w, permute=not args.no_permute)
     cache.partition_tokens = args.partition
     g = torch.Generator(device=dev).manual_seed(2)
     k1 = torch.randn(B, hkv, 1, D, generator=g, device=dev).to(torch.bfloat16)

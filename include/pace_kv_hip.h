@@ -16,14 +16,16 @@
  *   - update_cache_with_beam_indices    pace/llm/cache.py:161-167
  *   - repeat_kv (folded into the kernels) pace/llm/models/llama.py:50-61
  *
- * Storage: a block pool.  Block size is 16 tokens.  Per block and KV head the
- * K slab is token-major  K[token 0..15][dim 0..D-1]  and the V slab is
- * dim-major  V[dim 0..D-1][token 0..15]  (so that 16 bytes of either slab are
- * the eight values one matrix-core lane contracts over).  Slabs are addressed
- * as  base + block * block_stride + head * head_stride  (strides in elements),
+ * Storage: a block pool.  Block size is 16 tokens.  One (block, KV head) slab
+ * holds 16 tokens x head_dim values in an order private to the library (see
+ * k_slab_offset / v_slab_offset in the sources: 16-byte granules arranged so
+ * that every wavefront-wide load of the attention kernel is contiguous and
+ * already in matrix-core operand order); callers only ever move data through
+ * append / gather / copy_blocks.  Slabs are addressed as
+ *   base + block * block_stride + head * head_stride   (strides in elements),
  * which covers both two separate K / V allocations and one interleaved
- * [block][2][head][...] allocation.  Unwritten slots must hold finite bit
- * patterns (allocate the pool zero-filled).
+ * [block][2][head][16*head_dim] allocation.  Unwritten slots must hold finite
+ * bit patterns (allocate the pool zero-filled).
  */
 #ifndef PACE_KV_HIP_H
 #define PACE_KV_HIP_H
@@ -47,7 +49,7 @@ enum { PACE_DTYPE_F32 = 0, PACE_DTYPE_BF16 = 1 };
 
 typedef struct pace_kv_pool {
   void* k;                /* bf16, K slabs                                   */
-  void* v;                /* bf16, V slabs (dim-major)                       */
+  void* v;                /* bf16, V slabs                                   */
   int64_t k_block_stride; /* elements between consecutive blocks of K        */
   int64_t k_head_stride;  /* elements between consecutive KV heads of K      */
   int64_t v_block_stride;
@@ -131,7 +133,7 @@ typedef struct pace_paged_attn_args {
   int32_t batch, num_q_heads, q_len;
   int32_t causal;             /* 1: query row s reads tokens <= seq_len - q_len + s    */
   int32_t max_seq_len;        /* host-side upper bound of seq_lens (sizes the grid)    */
-  int32_t partition_tokens;   /* context split size, multiple of 32, <= 1024; 0 = auto */
+  int32_t partition_tokens;   /* context split size per workgroup, multiple of 32; 0 = auto   */
   float scale;                /* softmax scale, reference uses 1/sqrt(head_dim)        */
   void* workspace;            /* device scratch, >= pace_paged_attn_workspace_bytes()  */
   size_t workspace_bytes;

@@ -1,0 +1,102 @@
+"""The C-ABI library loads on a CPU-only machine and exports every function that
+include/pace_kv_hip.h declares (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(REPO, "include", "pace_kv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pace_[a-z_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    from pace_mi355 import _native
+
+    declared = _declared_functions()
+    assert declared, "no functions parsed from the header"
+    assert sorted(_native.EXPORTED_SYMBOLS) == declared
+
+
+def test_library_exports_every_declared_symbol():
+    from pace_mi355 import _native
+
+    assert os.path.exists(_native.library_path()), "build the library first: python amd-pace_amd/build.py"
+    lib = _native.load()
+    for name in _declared_functions():
+        assert getattr(lib, name) is not None, name
+    assert lib.pace_kv_abi_version() == _native.ABI_VERSION
+    assert lib.pace_kv_last_error() == b""
+
+
+def test_struct_layouts_match_the_header():
+    """Field order of the ctypes mirrors == field order in the header's structs."""
+    from pace_mi355 import _native
+
+    text = open(os.path.join(REPO, "include", "pace_kv_hip.h")).read()
+
+    def fields(struct_name):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s_t;" % (struct_name, struct_name), text, flags=re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        names = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            parts = decl.split(",")
+            first = parts[0].split()[-1].lstrip("*")
+            names.append(first)
+            names += [p.strip().lstrip("*") for p in parts[1:]]
+        return names
+
+    assert fields("pace_kv_pool") == [f[0] for f in _native.PoolDesc._fields_]
+    assert fields("pace_paged_attn_args") == [f[0] for f in _native.PagedAttnArgs._fields_]
+    assert ctypes.sizeof(_native.PoolDesc) == 64
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    """Contract violations are rejected on the host before anything is launched."""
+    from pace_mi355 import _native
+
+    lib = _native.load()
+    bad = _native.PoolDesc(k=16, v=32, k_block_stride=4096, k_head_stride=2048, v_block_stride=4096, v_head_stride=2048,
+                           num_blocks=4, num_kv_heads=2, head_dim=128, block_size=32)
+    rc = lib.pace_kv_append(ctypes.byref(bad), 16, 16, 8, 8, 8, 1, 1, 16, None)
+    assert rc == -1 and b"block_size 32 unsupported" in lib.pace_kv_last_error()
+    bad.block_size, bad.head_dim = 16, 96
+    assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 1, 1, 16, 16, 8, 8, 16, None) == -1
+    assert b"head_dim 96 unsupported" in lib.pace_kv_last_error()
+    with pytest.raises(_native.NativeError, match="head_dim 96"):
+        _native.check(-1)
+    assert lib.pace_attn_dense(16, 16, 16, 16, 1, 1, 1, 1, 1, 300, None, 0, 1, 1, 1, None) == -1
+    assert b"head_dim 300 unsupported" in lib.pace_kv_last_error()
+    assert lib.pace_paged_attn_workspace_bytes(0, 32, 1, 128, 4096, 0, 8) == 0
+
+
+def test_torch_op_is_defined_with_reference_schema_and_checks():
+    import torch
+
+    import pace_mi355  # noqa: F401
+
+    schema = str(torch.ops.pace.attention.default._schema)
+    assert "input_Q" in schema and "Tensor? input_mask" in schema and "Scalar? use_KQ" in schema
+    q = torch.zeros(2, 2, 3, 4)
+    k = torch.zeros(2, 2, 5, 4)
+    m = torch.zeros(2, 1, 1, 5)
+    with pytest.raises(RuntimeError, match="attention requires 4D inputs"):
+        torch.ops.pace.attention(q.view(4, 3, 4), k, k, m, 0)
+    with pytest.raises(RuntimeError, match="attention requires 4D inputs"):
+        torch.ops.pace.attention(q, k, k, m.view(2, 5), 0)
+    with pytest.raises(RuntimeError, match="requires Key and Value sizes to be of same shape"):
+        torch.ops.pace.attention(q, k, torch.zeros(2, 2, 6, 4), m, 0)
+    with pytest.raises(RuntimeError, match="only support the dtypes Float and BF16 types for input"):
+        torch.ops.pace.attention(q.to(torch.int8), k.to(torch.int8), k.to(torch.int8), m.to(torch.int8), 0)
+    with pytest.raises(RuntimeError, match="attention requires use_KQ to be 0 or 1"):
+        torch.ops.pace.attention(q, k, k, m, -3)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        torch.ops.pace.attention(q, k, k, m, False)

@@ -1,0 +1,82 @@
+"""GPU parity: torch.ops.pace.attention (dense op of the reference) against the oracle."""
+import pytest
+import torch
+
+from helpers import assert_attention_close, seeded_kv, seeded_q
+from oracle.attention_ref import sdpa_fp32, sdpa_native
+
+pytestmark = pytest.mark.gpu
+
+
+def _mask(seed, shape, dtype):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+
+# Shapes drawn from the reference's property test (tests/ops/test_sdpa.py:83-91): B in {1,32,96},
+# N in {1,16,32}, H in {1,64,128}, S in {1,128,512}, L in {1,512,2048}; sized to run in seconds.
+CASES = [
+    (1, 1, 1, 1, 1), (1, 16, 128, 64, 512), (32, 1, 1, 128, 2048), (2, 32, 512, 128, 1), (3, 2, 17, 1, 33),
+    (2, 16, 1, 64, 2048), (96, 1, 1, 64, 1), (1, 1, 128, 128, 512), (2, 3, 5, 80, 70), (1, 2, 33, 256, 40),
+]
+
+
+@pytest.mark.parametrize("B,N,S,H,L", CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_kq", [False, True])
+def test_dense_op_matches_oracle(device, B, N, S, H, L, dtype, use_kq):
+    if use_kq and (B, N, S, H, L) not in (CASES[1], CASES[4]):
+        pytest.skip("use_KQ selects an experimental path of the same function; two shapes suffice")
+    k, v = seeded_kv(1, B, N, L, H, dtype)
+    q = seeded_q(2, B, N, S, H, dtype)
+    m = _mask(3, (B, 1, 1, L), dtype)  # the reference test's mask: random additive bias of shape (B,1,1,L)
+    out = torch.ops.pace.attention(q.to(device), k.to(device), v.to(device), m.to(device), use_kq)
+    assert out.dtype == dtype and out.shape == q.shape and out.is_contiguous()
+    ref = sdpa_fp32(q, k, v, m)
+    if dtype == torch.float32:
+        assert torch.allclose(out.cpu(), ref, atol=1e-5, rtol=1e-5), (out.cpu() - ref).abs().max()
+    else:
+        assert_attention_close(out, ref, "dense bf16")
+        # and the reference's own bar: 1e-1 against torch's bf16 result (tests/ops/test_sdpa.py:113-127)
+        assert torch.allclose(out.cpu().float(), sdpa_native(q, k, v, m).float(), atol=1e-1, rtol=1e-1)
+
+
+@pytest.mark.parametrize("mshape", [(1, 1, 1, 40), (2, 1, 7, 40), (2, 3, 7, 40), (1, 3, 1, 40)])
+def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
+    q, (k, v) = seeded_q(5, 2, 3, 7, 64), seeded_kv(6, 2, 3, 40, 64)
+    m = _mask(7, mshape, torch.float32)  # fp32 mask with bf16 tensors
+    out = torch.ops.pace.attention(q.to(device), k.to(device), v.to(device), m.to(device), 0)
+    assert_attention_close(out, sdpa_fp32(q, k, v, m), f"mask {mshape}")
+
+
+def test_dense_op_with_bmc_padded_buffers_and_finfo_min_mask(device):
+    """BMC returns padded buffers and pads the mask with finfo.min (cache.py:195-222); the padded
+    columns must not contribute."""
+    from pace_mi355.llm import BMCKVCache
+    from pace_mi355.ops import MultiHeadAttention
+    from oracle.attention_ref import causal_mask_4d
+
+    B, H, D, L = 2, 4, 64, 37
+    k, v = seeded_kv(8, B, H, L, D)
+    cache = BMCKVCache(128)
+    K, V = cache.update_cache(k.to(device), v.to(device), 2)
+    assert K.shape[2] == 44 and K.is_cuda
+    q = seeded_q(9, B, H, 1, D)
+    m4 = causal_mask_4d(torch.ones(B, L, dtype=torch.long), 1, L, torch.bfloat16)
+    padded = cache.update_mask(m4.to(device), L)
+    assert padded.shape[-1] == 44
+    out = MultiHeadAttention(dtype=torch.bfloat16)(q.to(device), K, V, attention_mask=padded)
+    assert_attention_close(out, sdpa_fp32(q, k, v, m4), "BMC padded")
+
+
+def test_operator_without_mask_and_noncontiguous_inputs(device):
+    from pace_mi355.ops import MultiHeadAttention
+
+    q = seeded_q(1, 2, 8, 4, 16, torch.float32)
+    k, v = seeded_kv(2, 2, 8, 4, 16, torch.float32)
+    ones = torch.ones(2, 1, 4, 4)  # the reference's operator test passes a mask of ones (test_attention.py:27)
+    mha = MultiHeadAttention(dtype=torch.float32)
+    out = mha(q.to(device), k.to(device), v.to(device), attention_mask=ones.to(device))
+    assert torch.allclose(out.cpu(), sdpa_fp32(q, k, v, ones), atol=1e-3, rtol=1e-3)
+    qt = q.transpose(1, 2).contiguous().transpose(1, 2)  # [B,H,S,D] view over [B,S,H,D] storage
+    out2 = mha(qt.to(device), k.to(device), v.to(device))
+    assert torch.allclose(out2.cpu(), sdpa_fp32(q, k, v), atol=1e-5, rtol=1e-5)

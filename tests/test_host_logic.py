@@ -1,0 +1,240 @@
+"""CPU tests of the host side: operator registry, enums, cache-manager interface,
+contiguous caches vs the oracle, block allocator and eviction / compaction plans."""
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.cache_ref import BMCKVCacheRef, DynamicKVCacheRef, valid_prefix
+from pace_mi355.llm import (
+    BMCKVCache,
+    DynamicKVCache,
+    KVCacheManager,
+    KVCacheType,
+    LLMBackendType,
+    LLMOperatorType,
+    PagedKVCache,
+    get_kv_cache_class,
+)
+from pace_mi355.llm.paged import BlockAllocator, PagedState
+from pace_mi355.ops import BackendType, DataType, FusedOperatorType, MultiHeadAttention, OperatorType, backend_registry
+from pace_mi355.ops import enum as ops_enum
+from pace_mi355.ops.base import BackendBase
+from pace_mi355.ops.registry import BackendRegistry
+
+
+# ---- registry (semantics of the reference's tests/python_ops/test_registry.py) ----
+class _A:  # dummy implementations
+    pass
+
+
+class _B:
+    pass
+
+
+@pytest.fixture()
+def registry():
+    saved = list(ops_enum.FALLBACK_BACKEND)
+    yield BackendRegistry()
+    ops_enum.FALLBACK_BACKEND[:] = saved
+
+
+def test_register_and_get_every_combination(registry):
+    for op in OperatorType:
+        for be in BackendType:
+            cls = type("Impl", (), {})
+            registry.register(op, be, list(DataType))(cls)
+            for dt in DataType:
+                assert registry.get(op, be, dt) is cls
+
+
+def test_unregistered_operator_gives_none(registry):
+    assert registry.get(OperatorType.MHA, BackendType.JIT, DataType.BFLOAT16) is None
+    assert registry.get_available_backends(OperatorType.MHA) == []
+
+
+def test_fallback_order(registry):
+    op, dt = OperatorType.MHA, DataType.BFLOAT16
+    registry.register(op, BackendType.NATIVE, [dt])(_A)
+    registry.register(op, BackendType.JIT, [dt])(_B)
+    ops_enum.FALLBACK_BACKEND[:] = [BackendType.JIT, BackendType.NATIVE]
+    assert registry.get(op, BackendType.TPP, dt) is _B
+    ops_enum.FALLBACK_BACKEND[:] = [BackendType.NATIVE, BackendType.JIT]
+    assert registry.get(op, BackendType.TPP, dt) is _A
+    assert registry.get(op, BackendType.JIT, dt) is _B  # exact match wins over fallback
+
+
+def test_fused_operators_never_fall_back(registry):
+    registry.register(FusedOperatorType.FUSEDLINEARGELU, BackendType.TPP, [DataType.BFLOAT16])(_A)
+    assert registry.get(FusedOperatorType.FUSEDLINEARGELU, BackendType.TPP, DataType.BFLOAT16) is _A
+    assert registry.get(FusedOperatorType.FUSEDLINEARGELU, BackendType.JIT, DataType.BFLOAT16) is None
+    assert registry.get(FusedOperatorType.FUSEDLINEARGELU, BackendType.TPP, DataType.FLOAT32) is None
+
+
+def test_duplicate_and_missing_assert(registry):
+    registry.register(OperatorType.LINEAR, BackendType.JIT, [DataType.BFLOAT16])(_A)
+    with pytest.raises(AssertionError, match="Duplicate registration"):
+        registry.register(OperatorType.LINEAR, BackendType.JIT, [DataType.BFLOAT16])
+    ops_enum.FALLBACK_BACKEND[:] = [BackendType.TPP]
+    with pytest.raises(AssertionError, match="No backend found for linear with jit, float32"):
+        registry.get(OperatorType.LINEAR, BackendType.JIT, DataType.FLOAT32)
+
+
+def test_registry_repr(registry):
+    registry.register(OperatorType.LINEAR, BackendType.NATIVE, [DataType.BFLOAT16])(_A)
+    text = repr(registry)
+    for needle in ("OperatorType.LINEAR", "BackendType.NATIVE", "DataType.BFLOAT16", "_A"):
+        assert needle in text
+
+
+def test_enums_are_lowercase_strings():
+    assert OperatorType.MHA == "mha" and f"{BackendType.HIP}" == "hip" and str(DataType.BFLOAT16) == "bfloat16"
+    assert [b.name for b in BackendType][:4] == ["NATIVE", "JIT", "TPP", "IMBPS"]
+    assert DataType.from_torch(torch.bfloat16) is DataType.BFLOAT16 and DataType.FLOAT32.to_torch_dtype() is torch.float32
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        DataType.from_torch(torch.int8)
+    assert LLMBackendType is BackendType and LLMOperatorType.Attention == "attention"
+
+
+def test_mha_resolves_to_hip_backend_whatever_backend_is_asked():
+    from pace_mi355.ops.backends.hip import HIPAttention
+
+    assert set(backend_registry.get_available_backends(OperatorType.MHA)) == {
+        (BackendType.HIP, DataType.FLOAT32), (BackendType.HIP, DataType.BFLOAT16)}
+    for be in BackendType:
+        mha = MultiHeadAttention(backend_impl=be, dtype=torch.bfloat16)
+        assert isinstance(mha.backend, HIPAttention) and isinstance(mha.backend, BackendBase)
+        assert mha.operator_type is OperatorType.MHA
+        assert "HIPAttention" in repr(mha)
+
+
+# ---- cache-manager interface ----
+class _Cfg:
+    num_hidden_layers = 2
+
+
+def test_cache_type_enum_and_class_lookup():
+    assert KVCacheType("dynamic") is KVCacheType.DYNAMIC and KVCacheType("bmc") is KVCacheType.BMC
+    assert KVCacheType.get_kv_cache_type("paged") is KVCacheType.PAGED
+    assert get_kv_cache_class("dynamic") is DynamicKVCache and get_kv_cache_class(KVCacheType.BMC) is BMCKVCache
+    assert get_kv_cache_class("paged") is PagedKVCache
+    with pytest.raises(ValueError):
+        KVCacheType("nope")
+
+
+def test_manager_interface_matches_reference_expectations():
+    mgr = KVCacheManager(_Cfg(), 128, KVCacheType.DYNAMIC)
+    assert len(mgr.cache_objects) == 2 and isinstance(mgr[0], DynamicKVCache) and len(mgr) == 0
+    assert mgr.update_mask(torch.ones(2, 10), 10).shape == (2, 10)
+    bmc = BMCKVCache(128)
+    k, v = bmc.update_cache(torch.rand(2, 10, 64), torch.rand(2, 10, 64), concat_dim=1)
+    assert k.shape[1] == 11 and v.shape[1] == 11
+    assert bmc.update_mask(torch.ones(2, 10), 10).shape == (2, 11)
+    dyn = DynamicKVCache(128)
+    k, v = dyn.update_cache(torch.rand(2, 10, 64), torch.rand(2, 10, 64), concat_dim=1)
+    assert k.shape[1] == 10
+    paged = KVCacheManager(_Cfg(), 128, "paged")
+    assert isinstance(paged[1], PagedKVCache) and len(paged) == 0
+    paged.remove_cache(3)  # empty caches ignore removal, like the reference
+
+
+@pytest.mark.parametrize("prod,ref", [(DynamicKVCache, DynamicKVCacheRef), (BMCKVCache, BMCKVCacheRef)])
+def test_contiguous_caches_track_the_oracle(prod, ref):
+    g = torch.Generator().manual_seed(3)
+    a, b = prod(200), ref(200)
+    for T in (13, 1, 1, 30, 2):
+        k, v = torch.randn(2, 3, T, 4, generator=g), torch.randn(2, 3, T, 4, generator=g)
+        ka, va = a.update_cache(k, v, 2)
+        kb, vb = b.update_cache(k, v, 2)
+        assert torch.equal(ka, kb) and torch.equal(va, vb) and a.seq_len == b.seq_len
+    a.remove_cache(5), b.remove_cache(5)
+    assert torch.equal(a.key.narrow(2, 0, a.seq_len), valid_prefix(b)[0])
+    k = torch.randn(2, 3, 1, 4, generator=g)
+    assert torch.equal(a.update_cache(k, k, 2)[0], b.update_cache(k, k, 2)[0])
+    m = torch.zeros(2, 1, 1, a.seq_len, dtype=torch.bfloat16)
+    assert torch.equal(a.update_mask(m, a.seq_len), b.update_mask(m, b.seq_len))
+    with pytest.raises(ValueError, match="Cannot remove more tokens than available in cache."):
+        a.remove_cache(10_000)
+    with pytest.raises(AssertionError, match="concat_dim should be the same for all updates"):
+        a.update_cache(k, k, 1)
+    idx = torch.tensor([1, 1])
+    a.update_cache_with_beam_indices(idx), b.update_cache_with_beam_indices(idx)
+    assert torch.equal(a.key, b.key)
+
+
+def test_paged_cache_refuses_cpu_tensors():
+    with pytest.raises(RuntimeError, match="GPU memory"):
+        PagedKVCache(64).update_cache(torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16), torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16), 2)
+
+
+# ---- allocator and plans ----
+def test_allocator_lifo_and_errors():
+    al = BlockAllocator(6)
+    assert al.allocate(3) == [0, 1, 2] and al.num_free == 3
+    al.free([1])
+    assert al.allocate(1) == [1]
+    with pytest.raises(ValueError, match="freed twice"):
+        al.free([5])
+    with pytest.raises(MemoryError, match="exhausted"):
+        al.allocate(4)
+    al.take([4])
+    assert sorted(al.free_ids().tolist()) == [3, 5]
+    with pytest.raises(ValueError, match="not free"):
+        al.take([0])
+
+
+def _state(batch=3, max_len=160, blocks=40):
+    return PagedState(batch, max_len, blocks, torch.device("cpu"))
+
+
+def test_capacity_release_and_slots():
+    st = _state()
+    lens = np.array([33, 16, 0])
+    st.ensure_capacity(lens)
+    assert st.n_blocks.tolist() == [3, 1, 0] and st.allocator.num_free == 36
+    s = st.slots(np.array([30, 0, 0]), np.array([3, 2, 0]), 4)
+    assert s[0].tolist() == [st.table[0, 1] * 16 + 14, st.table[0, 1] * 16 + 15, st.table[0, 2] * 16, -1]
+    assert s[1].tolist()[:2] == [st.table[1, 0] * 16, st.table[1, 0] * 16 + 1] and (s[2] == -1).all()
+    assert st.release_beyond(np.array([16, 16, 0])) == 2 and st.n_blocks.tolist() == [1, 1, 0]
+    with pytest.raises(MemoryError, match="pool exhausted"):
+        st.ensure_capacity(np.array([16, 16, 2000]))
+
+
+def test_table_grows_on_demand():
+    st = PagedState(1, 16, 300, torch.device("cpu"))
+    st.ensure_capacity(np.array([16 * 200]))
+    assert st.n_blocks[0] == 200 and st.table.shape[1] >= 200
+    assert len(set(st.table[0, :200].tolist())) == 200
+
+
+def test_evict_and_compaction_plan_properties():
+    rng = np.random.default_rng(5)
+    st = _state(batch=4, max_len=400, blocks=120)
+    lens = np.array([400, 130, 16, 77])
+    st.ensure_capacity(lens)
+    before = {b: st.table[b, : st.n_blocks[b]].copy() for b in range(4)}
+    new_lens = st.evict(0, [1, 5, 24], lens)  # block 24 is the last (full) block of 400 tokens
+    assert new_lens[0] == 400 - 48 and st.n_blocks[0] == 22
+    assert st.table[0, :22].tolist() == [x for j, x in enumerate(before[0].tolist()) if j not in (1, 5, 24)]
+    new_lens = st.evict(1, [8], new_lens)  # partial last block holds 2 tokens
+    assert new_lens[1] == 128
+    with pytest.raises(IndexError):
+        st.evict(2, [3], new_lens)
+    for b in range(4):  # scatter a few more holes
+        n = int(st.n_blocks[b])
+        if n > 2:
+            new_lens = st.evict(b, sorted(rng.choice(n - 1, size=n // 3, replace=False).tolist()), new_lens)
+    moves = st.plan_compaction()
+    live = st.live_block_count()
+    assert not (set(moves[:, 0].tolist()) & set(moves[:, 1].tolist()))
+    assert (moves[:, 0] >= live).all() and (moves[:, 1] < live).all()
+    logical = {b: st.table[b, : st.n_blocks[b]].copy() for b in range(4)}
+    st.apply_moves(moves)
+    used = np.concatenate([st.table[b, : st.n_blocks[b]] for b in range(4)])
+    assert sorted(used.tolist()) == list(range(live))
+    remap = dict(zip(moves[:, 0].tolist(), moves[:, 1].tolist()))
+    for b in range(4):
+        assert st.table[b, : st.n_blocks[b]].tolist() == [remap.get(x, x) for x in logical[b].tolist()]
+    assert sorted(st.allocator.free_ids().tolist()) == list(range(live, 120))
+    assert len(st.plan_compaction()) == 0  # idempotent
