@@ -1,13 +1,22 @@
-"""Headline benchmark: paged decode attention + KV append, Llama-3-8B shape, one MI355X.
+"""Benchmarks of the KV-cache hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--path api|direct]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode-8b]
 
-A step is one pass of the hot path over one batch: append one new token per
-sequence into the block-paged cache, then GQA decode attention over the whole
-cache (batch 64, context 4096 -> 4097 tokens read, bf16, block 16, physical
-blocks randomly permuted).  Every step runs at the same cache state (the token
-lands at position 4096 each time), so bytes per step are constant.  All inputs
-are resident in HBM before the timed region.  Prints one JSON line.
+The default workload is the headline one: Llama-3-8B-shape single-layer decode, batch 64,
+context 4096, bf16, 32 Q / 8 KV heads, head_dim 128, KV block 16, physical blocks randomly
+permuted.  A step is one pass of the hot path over one batch: append one new token per
+sequence into the block-paged cache, then GQA decode attention over the whole cache.
+Every step runs at the same cache state (the token lands at position 4096 each time), so
+the bytes per step are constant.  All inputs are resident in HBM before the timed region.
+One JSON line is printed.
+
+Other workloads (same JSON shape, `config.workload` names them):
+  ragged    batch 256, contexts log-uniform in [128, 16384], pool 1.3x live tokens:
+            append + decode per step; gather timed beside it
+  verify    batch 32, contexts U[1024, 8192], 8 draft tokens appended + causal 8-query attention
+  compact   Llama-3-70B-shape KV, batch 8, context 32768: evict 40% of the blocks, then time the
+            compaction copy and the decode over the compacted cache
+  copy-calibration   block copy of a known byte count, used to scale the HBM byte counters
 """
 from __future__ import annotations
 
@@ -25,50 +34,318 @@ for _p in (REPO, os.path.join(REPO, "amd-pace_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+METRIC = "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 1 GPU"
 
-WORKLOAD = dict(name="llama3-8b-decode", batch=64, context=4096, q_heads=32, kv_heads=8, head_dim=128, block=16)
-
-
-def algorithmic_bytes(batch, ctx_after, q_heads, kv_heads, head_dim, new_tokens=1):
-    """Bytes one step must move: K+V read once at GQA-minimal width, Q read, O written,
-    block table and lengths read, new K/V read and written, one slot id per new token."""
-    kv_tok = 2 * kv_heads * head_dim * 2
-    decode = batch * ctx_after * kv_tok + 2 * batch * q_heads * head_dim * 2 + 4 * batch * math.ceil(ctx_after / 16) + 4 * batch
-    append = 2 * (batch * new_tokens * kv_tok) + 4 * batch * new_tokens
-    return decode, append
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, scaled by the
+# same counters on the copy-calibration workload (figures and commands: profiles/decode_8b_paged_attn_kernel.txt).
+MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_071_700_000}
 
 
-def build_cache(torch, dev, w, seed=1, permute=True):
-    """Cache holding `context` tokens per sequence in randomly permuted physical blocks."""
+def kv_token_bytes(kv_heads, head_dim):
+    return 2 * kv_heads * head_dim * 2  # K and V, bf16
+
+
+def decode_bytes(lens, q_heads, kv_heads, head_dim, q_len=1):
+    """Algorithmic bytes of one attention launch: K+V read once at GQA-minimal width, Q read,
+    O written, block table and lengths read."""
+    B = len(lens)
+    return (sum(lens) * kv_token_bytes(kv_heads, head_dim) + 2 * B * q_heads * q_len * head_dim * 2
+            + 4 * sum(math.ceil(n / 16) for n in lens) + 4 * B)
+
+
+def append_bytes(batch, new_tokens, kv_heads, head_dim):
+    """New K/V read and written, one slot id per new token."""
+    return 2 * batch * new_tokens * kv_token_bytes(kv_heads, head_dim) + 4 * batch * new_tokens
+
+
+def _randn_bf16(torch, shape, gen, dev):
+    return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+
+def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor=None, headroom=64, permute=True):
+    """Paged cache holding lens[b] tokens per sequence, physical blocks in a seeded random order."""
     import numpy as np
     from pace_mi355.llm import PagedKVCache
 
-    B, ctx, hkv, D = w["batch"], w["context"], w["kv_heads"], w["head_dim"]
-    per_seq = (ctx + 64 + 15) // 16
-    cache = PagedKVCache(ctx + 64, num_kv_heads=hkv, n_rep=w["q_heads"] // hkv, num_blocks=B * per_seq)
+    B, T = len(lens), max(lens)
+    live = sum((n + headroom + 15) // 16 for n in lens)
+    num_blocks = int(pool_factor * live) if pool_factor else live
+    cache = PagedKVCache(T + headroom, num_kv_heads=kv_heads, n_rep=q_heads // kv_heads, num_blocks=num_blocks)
     g = torch.Generator(device=dev).manual_seed(seed)
-    chunk = 512
-    first = True
-    for t0 in range(0, ctx, chunk):
-        n = min(chunk, ctx - t0)
-        k = torch.randn(B, hkv, n, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        v = torch.randn(B, hkv, n, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        if first:
-            # scramble the free list so that consecutive logical blocks are far apart in HBM
-            cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)
+    lens_np = np.asarray(lens)
+    chunk = 1024
+    for t0 in range(0, T, chunk):
+        n = min(chunk, T - t0)
+        k = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
+        v = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
+        if t0 == 0:
+            cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)  # creates the pool and the free list
             alloc = cache.state.allocator
             ids = alloc.allocate(alloc.num_free)
             if permute:
-                np.random.default_rng(seed).shuffle(ids)
+                np.random.default_rng(seed).shuffle(ids)  # consecutive logical blocks end up far apart in HBM
             else:
                 ids = ids[::-1]
             alloc.free(ids)
-            first = False
-        cache.update_cache(k, v, 2)
+        cache.append_ragged(k, v, np.clip(lens_np - t0, 0, n))
     return cache
 
 
-def cpu_baseline(torch, w, budget_s=12.0):
+class FixedStep:
+    """Direct C-ABI calls with metadata frozen at "T new tokens on top of the prefilled cache":
+    the new tokens land on the same positions every step, so each step moves the same bytes."""
+
+    def __init__(self, torch, cache, q, k_new, v_new, partition=0):
+        import numpy as np
+        from pace_mi355 import _native as nat
+
+        self.nat, self.lib = nat, nat.load()
+        dev = q.device
+        B, hq, S, D = q.shape
+        T = k_new.shape[2]
+        self.cache, self.k, self.v, self.T, self.B = cache, k_new, v_new, T, B
+        lens_after = cache.lens + T
+        cache.state.ensure_capacity(lens_after)
+        self.table = cache.state.device_table()
+        self.lens_dev = torch.from_numpy(lens_after.astype(np.int32)).to(dev)
+        self.lens_after = lens_after
+        self.out = torch.empty(B, hq, S, D, dtype=torch.bfloat16, device=dev)
+        max_len = int(lens_after.max())
+        ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, partition, cache.num_kv_heads))
+        self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        a = nat.PagedAttnArgs()
+        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = (self.out.data_ptr(), self.out.stride(0), self.out.stride(1),
+                                                           self.out.stride(2))
+        a.block_table, a.table_stride, a.seq_lens = self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr()
+        a.kv_start, a.mask, a.causal = None, None, 1
+        a.batch, a.num_q_heads, a.q_len = B, hq, S
+        a.max_seq_len, a.partition_tokens, a.scale = max_len, partition, 1.0 / math.sqrt(D)
+        a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
+        self.args, self.q = a, q
+        self.attn = self.lib.pace_paged_attn_decode if S == 1 else self.lib.pace_paged_attn_verify
+        self.stream = nat.current_stream_ptr()
+
+    def append(self):
+        k, v = self.k, self.v
+        self.nat.check(self.lib.pace_kv_append_paged(
+            ctypes.byref(self.cache._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2), self.B, self.T,
+            self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr(), -self.T, self.stream))
+
+    def attend(self):
+        self.nat.check(self.attn(ctypes.byref(self.cache._desc), ctypes.byref(self.args), self.stream))
+        return self.out
+
+    def __call__(self, ev=None):
+        self.append()
+        if ev:
+            ev[0].record()
+        self.attend()
+        if ev:
+            ev[1].record()
+
+
+def run_timed(torch, step, steps, warmup):
+    """W untimed steps, then exactly K timed steps bracketed by synchronize; the attention launch of
+    every timed step is bracketed by HIP events on the launch stream.  Returns (s per step, ms per launch)."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    return dt, sum(a.elapsed_time(b) for a, b in events) / steps
+
+
+def time_call(torch, fn, reps=20, warmup=3):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in ev) / reps
+
+
+def roofline(kernel, nbytes, ms, extra=None):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    d = {"bound": "hbm", "kernel": kernel, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": int(nbytes), "avg_launch_ms": round(ms, 5)}
+    if extra:
+        d.update(extra)
+    return d
+
+
+def result_line(args, workload, step_bytes, tokens_per_step, dt, roof, extra_cfg=None, extra=None):
+    gbs = step_bytes / dt / 1e9
+    line = {
+        "metric": METRIC,
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "tokens_per_s": round(tokens_per_step / dt, 1),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": workload, "bytes_per_step": int(step_bytes), "partition_tokens": args.partition},
+        "roofline": roof,
+    }
+    if extra_cfg:
+        line["config"].update(extra_cfg)
+    if extra:
+        line.update(extra)
+    return line
+
+
+# ---- workloads ---------------------------------------------------------------------------------
+def wl_decode_8b(torch, dev, args):
+    B, ctx, hq, hkv, D = 64, 4096, 32, 8, 128
+    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute)
+    cache.partition_tokens = args.partition
+    g = torch.Generator(device=dev).manual_seed(2)
+    k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
+    q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
+    if args.path == "api":
+        from pace_mi355.ops import MultiHeadAttention
+
+        mha = MultiHeadAttention(dtype=torch.bfloat16)
+
+        def step(ev=None):
+            pk, pv = cache.update_cache(k1, v1, 2)
+            if ev:
+                ev[0].record()
+            mha(q, pk, pv)
+            if ev:
+                ev[1].record()
+            cache.remove_cache(1)
+    else:
+        step = FixedStep(torch, cache, q, k1, v1, args.partition)
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
+    line = result_line(
+        args,
+        "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, head_dim 128, "
+        "KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
+        dec + append_bytes(B, 1, hkv, D), B, dt,
+        roofline("paged_attn_kernel<128,1,...> (decode)", dec, attn_ms, {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
+        {"path": args.path})
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
+    return line
+
+
+def wl_ragged(torch, dev, args):
+    import numpy as np
+
+    B, hq, hkv, D = 256, 32, 8, 128
+    rng = np.random.default_rng(2)
+    lens = np.round(np.exp(rng.uniform(math.log(128), math.log(16384), B))).astype(int).tolist()
+    cache = build_cache(torch, dev, lens, hq, hkv, D, seed=3, pool_factor=1.3, headroom=16)
+    cache.partition_tokens = args.partition
+    g = torch.Generator(device=dev).manual_seed(4)
+    k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
+    q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
+    step = FixedStep(torch, cache, q, k1, v1, args.partition)
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    lens1 = [n + 1 for n in lens]
+    dec = decode_bytes(lens1, hq, hkv, D)
+    gather_ms = time_call(torch, lambda: cache.gather(n_rep=1), reps=5, warmup=1)
+    gather_b = 2 * sum(lens) * kv_token_bytes(hkv, D)
+    return result_line(
+        args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x, "
+        "1-token append + GQA decode", dec + append_bytes(B, 1, hkv, D), B, dt,
+        roofline("paged_attn_kernel<128,1,...> (decode, ragged) + merge", dec, attn_ms),
+        extra={"gather": roofline("kv_gather_kernel<128> (includes output allocation)", gather_b, gather_ms)})
+
+
+def wl_verify(torch, dev, args):
+    import numpy as np
+
+    B, hq, hkv, D, S = 32, 32, 8, 128, 8
+    lens = np.random.default_rng(4).integers(1024, 8193, B).tolist()
+    cache = build_cache(torch, dev, lens, hq, hkv, D, seed=4)
+    cache.partition_tokens = args.partition
+    g = torch.Generator(device=dev).manual_seed(5)
+    kd, vd = _randn_bf16(torch, (B, hkv, S, D), g, dev), _randn_bf16(torch, (B, hkv, S, D), g, dev)
+    q = _randn_bf16(torch, (B, hq, S, D), g, dev)
+    step = FixedStep(torch, cache, q, kd, vd, args.partition)
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    lens_v = [n + S for n in lens]
+    dec = decode_bytes(lens_v, hq, hkv, D, q_len=S)
+    flops = 4.0 * sum(lens_v) * hq * S * D
+    return result_line(
+        args, "PARD speculative verify: batch 32, contexts U[1024,8192] (seed 4), 8 draft tokens appended + causal "
+        "8-query attention", dec + append_bytes(B, S, hkv, D), B * S, dt,
+        roofline("paged_attn_kernel<128,2,...> (verify)", dec, attn_ms,
+                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2)}))
+
+
+def wl_compact(torch, dev, args):
+    import numpy as np
+
+    B, hq, hkv, D, ctx = 8, 64, 8, 128, 32768
+    g = torch.Generator(device=dev).manual_seed(7)
+    q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
+    block_bytes = 16 * kv_token_bytes(hkv, D)
+    times, moved = [], 0
+    for rep in range(3):  # compaction is destructive: rebuild, evict, then time one compaction
+        cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=6, headroom=0)
+        rng = np.random.default_rng(6)
+        for b in range(B):
+            cache.evict_blocks(b, np.sort(rng.choice(ctx // 16, size=int(0.4 * ctx // 16), replace=False)).tolist())
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        moved = cache.compact()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+    compact_ms = min(times)
+    cache.partition_tokens = args.partition
+    lens = cache.lens.tolist()
+    dec = decode_bytes(lens, hq, hkv, D)
+    attn_ms = time_call(torch, lambda: cache.attend(q), reps=args.steps, warmup=args.warmup)
+    return result_line(
+        args, f"long-context compaction: 70B-shape KV (64 Q / 8 KV heads), batch 8, context 32768, 40% of blocks evicted "
+        f"(seed 6), {moved} blocks moved, then decode over {lens[0]} tokens/seq", dec, B, attn_ms * 1e-3,
+        roofline("paged_attn_kernel<128,1,...> (decode after compaction) + merge", dec, attn_ms),
+        extra={"compaction": roofline("kv_copy_blocks_kernel (plan + upload + copy)", 2 * moved * block_bytes, compact_ms,
+                                      {"blocks_moved": moved})})
+
+
+def wl_copy_calibration(torch, dev, args):
+    """Copies N whole blocks (N x 64 KiB read, N x 64 KiB written): the known-size kernel the
+    HBM byte counters are scaled by."""
+    from pace_mi355 import _native as nat
+
+    hq, hkv, D, N = 32, 8, 128, 8192
+    cache = build_cache(torch, dev, [16 * 2 * N // 64] * 64, hq, hkv, D, seed=9, headroom=0)
+    pairs = torch.stack([torch.arange(0, N, dtype=torch.int32), torch.arange(N, 2 * N, dtype=torch.int32)], 1).to(dev)
+    lib = nat.load()
+
+    def copy():
+        nat.check(lib.pace_kv_copy_blocks(ctypes.byref(cache._desc), ctypes.byref(cache._desc), pairs.data_ptr(), N,
+                                          nat.current_stream_ptr()))
+
+    ms = time_call(torch, copy, reps=args.steps, warmup=args.warmup)
+    nbytes = 2 * N * 16 * kv_token_bytes(hkv, D)
+    return result_line(args, f"block copy calibration: {N} blocks of 64 KiB, disjoint src/dst", nbytes, 0, ms * 1e-3,
+                       roofline("kv_copy_blocks_kernel", nbytes, ms, {"bytes_read": nbytes // 2, "bytes_written": nbytes // 2}))
+
+
+def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
     """The reference's CPU path, restated by the oracle, on a bounded sample of the workload:
     BMC cache (its benchmark default) holding GQA-expanded K/V + torch SDPA in bf16."""
     from oracle.attention_ref import lengths_mask_4d, sdpa_native
@@ -76,7 +353,6 @@ def cpu_baseline(torch, w, budget_s=12.0):
 
     cores = torch.get_num_threads()
     B = 8
-    ctx, hq, hkv, D = w["context"], w["q_heads"], w["kv_heads"], w["head_dim"]
     n_rep = hq // hkv
     g = torch.Generator().manual_seed(0)
     cache = BMCKVCacheRef(ctx + 128)
@@ -105,17 +381,21 @@ def cpu_baseline(torch, w, budget_s=12.0):
         step()
         n_steps += 1
     dt = (time.perf_counter() - t0) / n_steps
-    decode_b, append_b = algorithmic_bytes(B, ctx + 1, hq, hkv, D)
+    nbytes = decode_bytes([ctx + 1] * B, hq, hkv, D) + append_bytes(B, 1, hkv, D)
     return {
-        "value": round((decode_b + append_b) / dt / 1e9, 3),
+        "value": round(nbytes / dt / 1e9, 3),
         "unit": "GB/s",
         "tokens_per_s": round(B / dt, 2),
         "ms_per_step": round(dt * 1e3, 3),
         "cores": cores,
         "kind": "port",
-        "sample": f"batch {B} of {w['batch']}, context {ctx}, BMC cache with GQA-expanded K/V + torch CPU SDPA bf16; "
+        "sample": f"batch {B} of {batch}, context {ctx}, BMC cache with GQA-expanded K/V + torch CPU SDPA bf16; "
                   f"2 warm-up + {n_steps} timed steps; GB/s uses the same GQA-minimal algorithmic bytes as the GPU line",
     }
+
+
+WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify, "compact": wl_compact,
+             "copy-calibration": wl_copy_calibration}
 
 
 def main() -> int:
@@ -123,135 +403,26 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="decode-8b")
     ap.add_argument("--path", choices=("api", "direct"), default="direct",
-                    help="direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + MultiHeadAttention")
+                    help="decode-8b only. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
+                         "MultiHeadAttention")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-permute", action="store_true", help="keep physical blocks in logical order (diagnostic)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by "
-              "sequence with no exchange; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by sequence or by KV "
+              "head with no exchange). Run with --gpus 1.", file=sys.stderr)
         return 2
-
     import torch
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
-    from pace_mi355 import _native as nat
-    from pace_mi355.ops import MultiHeadAttention
-
-    lib = nat.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = WORKLOAD
-    B, ctx, hq, hkv, D = w["batch"], w["context"], w["q_heads"], w["kv_heads"], w["head_dim"]
-    cache = build_cache(torch, dev, w, permute=not args.no_permute)
-    cache.partition_tokens = args.partition
-    g = torch.Generator(device=dev).manual_seed(2)
-    k1 = torch.randn(B, hkv, 1, D, generator=g, device=dev).to(torch.bfloat16)
-    v1 = torch.randn(B, hkv, 1, D, generator=g, device=dev).to(torch.bfloat16)
-    q = torch.randn(B, hq, 1, D, generator=g, device=dev).to(torch.bfloat16)
-    mha = MultiHeadAttention(dtype=torch.bfloat16)
-
-    if args.path == "api":
-        def step(ev=None):
-            pk, pv = cache.update_cache(k1, v1, 2)
-            if ev:
-                ev[0].record()
-            out = mha(q, pk, pv)
-            if ev:
-                ev[1].record()
-            cache.remove_cache(1)
-            return out
-    else:
-        # Fixed metadata: lengths after the append, block table, workspace; the new token
-        # lands at position `ctx` of every sequence on every step.
-        import numpy as np
-
-        lens_after = cache.lens + 1
-        cache.state.ensure_capacity(lens_after)
-        table = cache.state.device_table()
-        lens_dev = torch.from_numpy(lens_after.astype(np.int32)).to(dev)
-        out = torch.empty(B, hq, 1, D, dtype=torch.bfloat16, device=dev)
-        ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, 1, D, ctx + 1, args.partition, hkv))
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-        a = nat.PagedAttnArgs()
-        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
-        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
-        a.block_table, a.table_stride, a.seq_lens = table.data_ptr(), table.stride(0), lens_dev.data_ptr()
-        a.kv_start, a.mask, a.causal = None, None, 1
-        a.batch, a.num_q_heads, a.q_len = B, hq, 1
-        a.max_seq_len, a.partition_tokens, a.scale = ctx + 1, args.partition, 1.0 / math.sqrt(D)
-        a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
-        desc = cache._desc
-        stream = nat.current_stream_ptr()
-
-        def step(ev=None):
-            nat.check(lib.pace_kv_append_paged(ctypes.byref(desc), k1.data_ptr(), v1.data_ptr(), k1.stride(0), k1.stride(1),
-                                               k1.stride(2), B, 1, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -1,
-                                               stream))
-            if ev:
-                ev[0].record()
-            nat.check(lib.pace_paged_attn_decode(ctypes.byref(desc), ctypes.byref(a), stream))
-            if ev:
-                ev[1].record()
-            return out
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(events[i])
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    attn_ms = sum(e0.elapsed_time(e1) for e0, e1 in events) / args.steps
-
-    decode_b, append_b = algorithmic_bytes(B, ctx + 1, hq, hkv, D)
-    step_bytes = decode_b + append_b
-    ms_per_step = dt * 1e3 / args.steps
-    gbs = step_bytes / (dt / args.steps) / 1e9
-    achieved = decode_b / (attn_ms * 1e-3) / 1e9
-    line = {
-        "metric": "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 1 GPU",
-        "value": round(gbs, 1),
-        "unit": "GB/s",
-        "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
-        "tokens_per_s": round(B * args.steps / dt, 1),
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, "
-                        "head_dim 128, KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
-            "bytes_per_step": step_bytes,
-            "path": args.path,
-            "partition_tokens": args.partition,
-        },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "paged_attn_kernel<128,1,false> (+ merge)",
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
-            "bytes_per_launch": decode_b,
-            "avg_launch_ms": round(attn_ms, 5),
-        },
-    }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(torch, w)
-    print(json.dumps(line))
+    print(json.dumps(WORKLOADS[args.workload](torch, dev, args)))
     return 0
 
 
