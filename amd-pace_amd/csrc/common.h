@@ -55,6 +55,19 @@ __host__ __device__ __forceinline__ int v_slab_offset(int tok, int dim) {
   return (((dim >> 4) * 2 + (tok >> 3)) * 16 + (dim & 15)) * 8 + (tok & 7);
 }
 
+// Store eight dims (chunk) of one token's K and V into the slabs of its (block, head).
+// K is one 16-byte store; the V values sit 8 elements apart (token-minor slab).
+template <int D>
+__device__ __forceinline__ void store_kv_chunk(uint16_t* kslab, uint16_t* vslab, int tok, int chunk, u32x4 kv, u32x4 vv) {
+  *reinterpret_cast<u32x4*>(kslab + k_slab_offset<D>(tok, chunk * 8)) = kv;
+  uint16_t* vdst = vslab + v_slab_offset<D>(tok, chunk * 8);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    vdst[(2 * j) * 8] = (uint16_t)(vv[j] & 0xffffu);
+    vdst[(2 * j + 1) * 8] = (uint16_t)(vv[j] >> 16);
+  }
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
 // Round-to-nearest-even fp32 -> bf16 bits (NaN stays NaN).

@@ -51,17 +51,9 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
   const int64_t src = b * sb + h * sh + t * st + chunk * 8;
   const u32x4 kv = *reinterpret_cast<const u32x4*>(k_new + src);
   const u32x4 vv = *reinterpret_cast<const u32x4*>(v_new + src);
-  uint16_t* kdst = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride +
-                   k_slab_offset<D>(off, chunk * 8);
-  *reinterpret_cast<u32x4*>(kdst) = kv;
-  // The eight dims of this chunk sit 8 elements apart in the V slab (same dim tile).
-  uint16_t* vdst = reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride +
-                   v_slab_offset<D>(off, chunk * 8);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    vdst[(2 * j) * 8] = (uint16_t)(vv[j] & 0xffffu);
-    vdst[(2 * j + 1) * 8] = (uint16_t)(vv[j] >> 16);
-  }
+  store_kv_chunk<D>(reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride,
+                    reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride, off, chunk, kv,
+                    vv);
 }
 
 // ---------------------------------------------------------------------------------

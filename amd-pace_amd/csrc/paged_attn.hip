@@ -49,6 +49,12 @@ struct PagedAttnParams {
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)
+  // Fused append: the last n_new tokens of every sequence are taken from k_new / v_new
+  // (and written to the pool by this launch) instead of being read from the pool.
+  const uint16_t* k_new;
+  const uint16_t* v_new;
+  int64_t n_sb, n_sh, n_st;
+  int32_t n_new;
   float* part_o;      // [B][Hq][S][max_parts][D]
   float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
 };
@@ -84,6 +90,52 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
   const uint16_t* vp = p.vpool + vblk * p.v_bs + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
 #pragma unroll
   for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
+}
+
+// The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
+// (token idx of the unit = new token idx; tokens >= n_new are zero and get masked).
+template <int D>
+__device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnParams& p, int b, int kvh, int n_new, int n, int g) {
+  const uint16_t* kb = p.k_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
+  const uint16_t* vb = p.v_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int idx = 8 * (n >> 2) + 4 * t + (n & 3);
+#pragma unroll
+    for (int kk = 0; kk < D / 32; ++kk)
+      r.k[t][kk] = idx < n_new ? *reinterpret_cast<const u32x4*>(kb + (int64_t)idx * p.n_st + kk * 32 + 8 * g) : zero;
+  }
+#pragma unroll
+  for (int j = 0; j < D / 16; ++j) {
+    u32x4 w = zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int tok = 8 * g + e;
+      if (tok < n_new) w[e >> 1] |= (uint32_t)vb[(int64_t)tok * p.n_st + 16 * j + n] << (16 * (e & 1));
+    }
+    r.v[j] = w;
+  }
+}
+
+// Write the step's new tokens of (b, kvh) into their pool slots (positions pool_end ..).
+template <int D>
+__device__ __forceinline__ void write_new_tokens(const PagedAttnParams& p, int b, int kvh, int pool_end, int n_new, int lane) {
+  constexpr int CH = D / 8;
+  for (int item = lane; item < n_new * CH; item += 64) {
+    const int idx = item / CH, chunk = item % CH;
+    const int pos = pool_end + idx;
+    const int jb = pos / PACE_KV_BLOCK_TOKENS;
+    if (jb >= p.table_stride) continue;
+    const int64_t blk = p.table[(int64_t)b * p.table_stride + jb];
+    if (blk < 0 || blk >= p.num_blocks) continue;  // never write outside the pool
+    const int64_t src = (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh + (int64_t)idx * p.n_st + chunk * 8;
+    const u32x4 kv = *reinterpret_cast<const u32x4*>(p.k_new + src);
+    const u32x4 vv = *reinterpret_cast<const u32x4*>(p.v_new + src);
+    store_kv_chunk<D>(const_cast<uint16_t*>(p.kpool) + blk * p.k_bs + (int64_t)kvh * p.k_hs,
+                      const_cast<uint16_t*>(p.vpool) + blk * p.v_bs + (int64_t)kvh * p.v_hs, pos % PACE_KV_BLOCK_TOKENS,
+                      chunk, kv, vv);
+  }
 }
 
 template <int D, int NQT>
@@ -218,14 +270,18 @@ struct WaveBlockIds {
 };
 
 // NW waves per workgroup split the partition's units among themselves and merge their
-// softmax states through LDS; NBUF unit buffers per wave are kept in flight.
-// OCC is the number of such waves that must fit on one SIMD (caps the register budget).
-template <int D, int NQT, bool HAS_MASK, int NW, int NBUF, int OCC>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void paged_attn_kernel(
+// softmax states through LDS.  OCC is the number of such waves that must fit on one SIMD
+// (caps the register budget); latency is hidden by the other resident waves, each wave
+// keeps one unit (16 KiB) in flight.  With FUSED, one more wave per workgroup handles the
+// step's new tokens (attends to them from the caller's buffers and stores them into the
+// pool), so that its dependent round trips overlap with the streaming waves.
+template <int D, int NQT, bool HAS_MASK, int NW, int OCC, bool FUSED>
+__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-  static_assert(NW * NQT <= 8, "LDS merge buffer holds 64 query rows");
+  constexpr int NWT = NW + (FUSED ? 1 : 0);  // waves in the workgroup
+  static_assert((NWT / 2) * 16 * NQT <= 64, "LDS merge buffer holds 64 query rows");
   __shared__ float merge_buf[64 * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int part = blockIdx.x, kvh = blockIdx.y;
@@ -236,12 +292,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
   if (part >= n_parts) return;  // uniform over the workgroup
   const int start = p.kv_start ? p.kv_start[b] : 0;
   const int part_begin = part * P;
-  const int tok_end = min(len, part_begin + P);
+  // Tokens [pool_end, len) are this step's new tokens when the append is fused in.
+  const int n_new = FUSED ? min(p.n_new, len) : 0;
+  const int pool_end = len - n_new;
+  const int tok_end = min(pool_end, part_begin + P);
   const int S = p.q_len, R = S * p.n_rep;
   // This wave's share of the partition's 32-token units.
-  const int part_units = (tok_end - part_begin + 31) / 32;
+  const int part_units = max(0, (tok_end - part_begin + 31) / 32);
   const int per_wave = (part_units + NW - 1) / NW;
-  const int u_begin = min(part_units, wave * per_wave);
+  const int u_begin = min(part_units, wave * per_wave);  // the extra wave (wave == NW) gets none
   const int n_units = min(part_units, u_begin + per_wave) - u_begin;
   const int tok_begin = part_begin + 32 * u_begin;
 
@@ -291,22 +350,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
     ids.hi = hi < 0 ? 0 : (hi >= p.num_blocks ? p.num_blocks - 1 : hi);
   }
 
-  UnitRegs<D> buf[NBUF];
-#pragma unroll
-  for (int i = 0; i < NBUF - 1; ++i)
-    if (i < n_units) load_unit<D>(buf[i], p, kvh, ids.get(2 * i), ids.get(2 * i + 1), n, g);
-  for (int u = 0; u < n_units; u += NBUF) {
-#pragma unroll
-    for (int j = 0; j < NBUF; ++j) {
-      const int uu = u + j;
-      if (uu < n_units) {
-        const int un = uu + NBUF - 1;  // unit to put in flight now
-        if (un < n_units) load_unit<D>(buf[(j + NBUF - 1) % NBUF], p, kvh, ids.get(2 * un), ids.get(2 * un + 1), n, g);
-        const int t0 = tok_begin + 32 * uu;
-        const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
-        compute_unit<D, NQT, HAS_MASK>(buf[j], qreg, st, p, t0, tok_end, start, full, g);
-      }
+  UnitRegs<D> buf;
+  if (FUSED) {
+    if (wave == NW && n_new > 0 && part == n_parts - 1) {
+      load_new_unit<D>(buf, p, b, kvh, n_new, n, g);
+      if (qg == 0) write_new_tokens<D>(p, b, kvh, pool_end, n_new, lane);
+      compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g);
     }
+  }
+  for (int uu = 0; uu < n_units; ++uu) {
+    load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
+    const int t0 = tok_begin + 32 * uu;
+    const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
+    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g);
   }
 
   // Row sums were kept per lane; complete them over the four lanes of a row.
@@ -319,14 +375,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
   }
 
   // Pairwise merge of the waves' states through LDS (fixed order: deterministic).
-  if (NW > 1) {
+  if (NWT > 1) {
     constexpr int ROW_F = D + 2;
     constexpr int SLOT_F = 16 * NQT * ROW_F;
 #pragma unroll
-    for (int stride = 1; stride < NW; stride *= 2) {
+    for (int stride = 1; stride < NWT; stride *= 2) {
       const int slot = wave / (2 * stride);
       const bool sender = (wave & (2 * stride - 1)) == stride;
-      const bool receiver = (wave & (2 * stride - 1)) == 0 && wave + stride < NW;
+      const bool receiver = (wave & (2 * stride - 1)) == 0 && wave + stride < NWT;
       if (sender) {
 #pragma unroll
         for (int qt = 0; qt < NQT; ++qt) {
@@ -434,21 +490,21 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
 
 // Launch shape per query-tile count: waves per workgroup and unit buffers per wave.
 struct Shape {
-  int nqt, nw, nbuf, occ;
+  int nqt, nw, occ;
 };
 
 static Shape shape_for(int tiles) {
   if (tiles <= 1) {
-    Shape s = {1, 4, 1, 2};
-    // Tuning override for the single-tile (decode) kernel: "NW,NBUF,OCC".
+    Shape s = {1, 4, 2};
+    // Tuning override for the single-tile (decode) kernel: "NW,OCC".
     if (const char* e = getenv("PACE_KV_DECODE_SHAPE")) {
-      int nw = 0, nbuf = 0, occ = 0;
-      if (sscanf(e, "%d,%d,%d", &nw, &nbuf, &occ) == 3) s.nw = nw, s.nbuf = nbuf, s.occ = occ;
+      int nw = 0, occ = 0;
+      if (sscanf(e, "%d,%d", &nw, &occ) == 2) s.nw = nw, s.occ = occ;
     }
     return s;
   }
-  if (tiles == 2) return Shape{2, 4, 1, 2};
-  return Shape{4, 2, 1, 1};
+  if (tiles == 2) return Shape{2, 4, 2};
+  return Shape{4, 2, 1};
 }
 
 // Tokens one workgroup may cover: each wave holds at most 128 block ids.
@@ -471,27 +527,30 @@ static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t bat
   return (int)per;
 }
 
-template <int D, int NQT, int NW, int NBUF, int OCC>
+template <int D, int NQT, int NW, int OCC>
 static void launch(const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
-  if (has_mask)
-    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, true, NW, NBUF, OCC>), grid, dim3(64 * NW), 0, s, p);
-  else
-    hipLaunchKernelGGL((paged_attn_kernel<D, NQT, false, NW, NBUF, OCC>), grid, dim3(64 * NW), 0, s, p);
+  const bool fused = p.n_new > 0;
+#define PACE_GO(M_, F_) hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, F_>), grid, dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+  if (has_mask) {
+    if (fused) PACE_GO(true, true); else PACE_GO(true, false);
+  } else {
+    if (fused) PACE_GO(false, true); else PACE_GO(false, false);
+  }
+#undef PACE_GO
 }
 
 template <int D>
 static bool launch_shape(const Shape& sh, const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
-#define PACE_TRY(NQT_, NW_, NBUF_, OCC_)                                         \
-  if (sh.nqt == NQT_ && sh.nw == NW_ && sh.nbuf == NBUF_ && sh.occ == OCC_) {       \
-    launch<D, NQT_, NW_, NBUF_, OCC_>(p, grid, has_mask, s);                        \
-    return true;                                                                    \
+#define PACE_TRY(NQT_, NW_, OCC_)                                  \
+  if (sh.nqt == NQT_ && sh.nw == NW_ && sh.occ == OCC_) {            \
+    launch<D, NQT_, NW_, OCC_>(p, grid, has_mask, s);                \
+    return true;                                                     \
   }
-  PACE_TRY(1, 4, 1, 2)
-  PACE_TRY(1, 4, 1, 3)
-  PACE_TRY(1, 8, 1, 2)
-  PACE_TRY(1, 4, 2, 1)
-  PACE_TRY(2, 4, 1, 2)
-  PACE_TRY(4, 2, 1, 1)
+  PACE_TRY(1, 4, 2)
+  PACE_TRY(1, 4, 3)
+  PACE_TRY(1, 8, 2)
+  PACE_TRY(2, 4, 2)
+  PACE_TRY(4, 2, 1)
 #undef PACE_TRY
   return false;
 }
@@ -518,6 +577,13 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     PACE_REQUIRE(a->mask_dtype == PACE_DTYPE_F32 || a->mask_dtype == PACE_DTYPE_BF16, "%s: bad mask dtype %d", who,
                  a->mask_dtype);
     PACE_REQUIRE(a->mask_len >= 0, "%s: negative mask_len", who);
+  }
+  if (a->k_new || a->v_new) {
+    PACE_REQUIRE(a->k_new && a->v_new, "%s: k_new and v_new must be given together", who);
+    PACE_REQUIRE(a->n_new >= 1 && a->n_new <= 32, "%s: fused append takes 1..32 new tokens (got %d)", who, a->n_new);
+    PACE_REQUIRE(aligned16(a->k_new) && aligned16(a->v_new) && (a->new_stride_b % 8) == 0 && (a->new_stride_h % 8) == 0 &&
+                     (a->new_stride_t % 8) == 0,
+                 "%s: k_new / v_new must be 16-byte aligned with strides that are multiples of 8 elements", who);
   }
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
@@ -547,6 +613,9 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.part_tokens = part, p.max_parts = max_parts;
   p.scale_log2 = a->scale * kLog2e;
   p.part_o = nullptr, p.part_ml = nullptr;
+  p.k_new = static_cast<const uint16_t*>(a->k_new), p.v_new = static_cast<const uint16_t*>(a->v_new);
+  p.n_sb = a->new_stride_b, p.n_sh = a->new_stride_h, p.n_st = a->new_stride_t;
+  p.n_new = a->k_new ? a->n_new : 0;
   p.n_qgroups = (tiles + sh.nqt - 1) / sh.nqt;
 
   if (max_parts > 1) {
@@ -563,7 +632,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
   const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, grid, has_mask, s) : launch_shape<64>(sh, p, grid, has_mask, s);
-  PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d nbuf=%d occ=%d", who, sh.nqt, sh.nw, sh.nbuf, sh.occ);
+  PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d", who, sh.nqt, sh.nw, sh.occ);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",
@@ -77,6 +77,12 @@ class PagedAttnArgs(Structure):
         ("scale", c_float),
         ("workspace", c_void_p),
         ("workspace_bytes", c_size_t),
+        ("k_new", c_void_p),
+        ("v_new", c_void_p),
+        ("new_stride_b", c_int64),
+        ("new_stride_h", c_int64),
+        ("new_stride_t", c_int64),
+        ("n_new", c_int32),
     ]
 
 

@@ -144,6 +144,11 @@ class PagedKVCache(KVCacheBase):
         self.n_rep = 1
         self.head_dim = 0
         self.partition_tokens = 0  # 0: let the library choose
+        # Appends of up to 32 tokens are held back until the attention call that follows, which
+        # reads them from the caller's tensors and stores them into the pool in the same launch;
+        # anything else that needs the pool or the lengths first flushes them with a plain append.
+        self.fuse_append = True
+        self._pending: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
     # -- set-up -----------------------------------------------------------------
@@ -238,17 +243,14 @@ class PagedKVCache(KVCacheBase):
         st = self.state
         lib = nat.load()
         stream = nat.current_stream_ptr()
+        self._flush()
         if counts is None:
             new_lens = self.lens + T
             st.ensure_capacity(new_lens)
-            lens_dev = st.device_lens(new_lens)
-            table = st.device_table()
-            nat.check(
-                lib.pace_kv_append_paged(
-                    ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
-                    B, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -T, stream,
-                )
-            )
+            if self.fuse_append and T <= 32:
+                self._pending = (k, v, head_step)
+            else:
+                self._launch_append(k, v, head_step, new_lens)
         else:
             if (counts < 0).any() or (counts > T).any():
                 raise ValueError("counts must lie in [0, T]")
@@ -266,9 +268,28 @@ class PagedKVCache(KVCacheBase):
         if self.key is None:
             self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
 
+    def _launch_append(self, k: torch.Tensor, v: torch.Tensor, head_step: int, lens_after: np.ndarray) -> None:
+        st = self.state
+        T = k.shape[2]
+        lens_dev, table = st.device_lens(lens_after), st.device_table()
+        nat.check(
+            nat.load().pace_kv_append_paged(
+                ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
+                self.batch, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -T, nat.current_stream_ptr(),
+            )
+        )
+
+    def _flush(self) -> None:
+        """Store a held-back append into the pool now."""
+        if self._pending is not None:
+            k, v, head_step = self._pending
+            self._pending = None
+            self._launch_append(k, v, head_step, self.lens)
+
     def truncate(self, remove: Sequence[int]) -> None:
         """Per-sequence rollback: forget the last ``remove[b]`` tokens of sequence ``b``
         and return emptied blocks to the free list."""
+        self._flush()
         remove = np.asarray(remove, dtype=np.int64)
         if (remove > self.lens).any() or (remove < 0).any():
             raise ValueError("Cannot remove more tokens than available in cache.")
@@ -286,6 +307,8 @@ class PagedKVCache(KVCacheBase):
         """Remove whole logical blocks from the middle of sequence ``b``; the
         surviving tokens keep their order and become the sequence."""
         peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
+        for p in peers:
+            p._flush()
         new_lens = self.state.evict(b, logical_blocks, self.lens)
         for p in peers:
             p.lens = new_lens.copy()
@@ -293,6 +316,9 @@ class PagedKVCache(KVCacheBase):
 
     def compact(self) -> int:
         """Pack live blocks into the lowest pool ids (every layer's pool); returns blocks moved."""
+        for p in self._shared.get("layers", [self]):
+            if p.pool is not None:
+                p._flush()
         moves = self.state.plan_compaction()
         if len(moves):
             pairs = torch.from_numpy(moves).pin_memory().to(self.pool.device, non_blocking=True)
@@ -306,6 +332,8 @@ class PagedKVCache(KVCacheBase):
     def reorder(self, beam_idx: Sequence[int]) -> None:
         st = self.state
         peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
+        for p in peers:
+            p._flush()
         old_table, old_n, old_lens = st.table.copy(), st.n_blocks.copy(), self.lens.copy()
         pairs: List[Tuple[int, int]] = []
         new_rows = []
@@ -334,6 +362,7 @@ class PagedKVCache(KVCacheBase):
 
     def gather(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
         """Dense ``[B, Hkv*n_rep, L, D]`` copies of K and V (zeros past each length)."""
+        self._flush()
         n_rep = self.n_rep if n_rep is None else int(n_rep)
         L = int(self.lens.max(initial=0)) if pad_to is None else int(pad_to)
         shape = (self.batch, self.num_kv_heads * n_rep, L, self.head_dim)
@@ -399,6 +428,11 @@ class PagedKVCache(KVCacheBase):
         a.scale = 1.0 / math.sqrt(D)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes
+        if self._pending is not None:
+            k, v, head_step = self._pending
+            self._pending = None  # this launch stores them into the pool
+            a.k_new, a.v_new, a.n_new = k.data_ptr(), v.data_ptr(), k.shape[2]
+            a.new_stride_b, a.new_stride_h, a.new_stride_t = k.stride(0), k.stride(1) * head_step, k.stride(2)
         fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
         nat.check(fn(ctypes.byref(self._desc), ctypes.byref(a), nat.current_stream_ptr()))
         return out

@@ -95,7 +95,7 @@ class FixedStep:
     """Direct C-ABI calls with metadata frozen at "T new tokens on top of the prefilled cache":
     the new tokens land on the same positions every step, so each step moves the same bytes."""
 
-    def __init__(self, torch, cache, q, k_new, v_new, partition=0):
+    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True):
         import numpy as np
         from pace_mi355 import _native as nat
 
@@ -122,6 +122,10 @@ class FixedStep:
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         a.max_seq_len, a.partition_tokens, a.scale = max_len, partition, 1.0 / math.sqrt(D)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
+        self.fused = fused
+        if fused:  # the attention launch reads the new tokens from k_new / v_new and stores them into the pool
+            a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
+            a.new_stride_b, a.new_stride_h, a.new_stride_t = k_new.stride(0), k_new.stride(1), k_new.stride(2)
         self.args, self.q = a, q
         self.attn = self.lib.pace_paged_attn_decode if S == 1 else self.lib.pace_paged_attn_verify
         self.stream = nat.current_stream_ptr()
@@ -137,7 +141,8 @@ class FixedStep:
         return self.out
 
     def __call__(self, ev=None):
-        self.append()
+        if not self.fused:
+            self.append()
         if ev:
             ev[0].record()
         self.attend()
@@ -145,19 +150,24 @@ class FixedStep:
             ev[1].record()
 
 
+EVENT_EVERY = 8  # an event record costs several microseconds of GPU timeline; bracket one launch in eight
+
+
 def run_timed(torch, step, steps, warmup):
-    """W untimed steps, then exactly K timed steps bracketed by synchronize; the attention launch of
-    every timed step is bracketed by HIP events on the launch stream.  Returns (s per step, ms per launch)."""
+    """W untimed steps, then exactly K timed steps bracketed by synchronize.  Inside the timed region
+    the attention launch of every eighth step is bracketed by HIP events on the launch stream.
+    Returns (s per step, ms per launch)."""
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range((steps + EVENT_EVERY - 1) // EVENT_EVERY)]
     t0 = time.perf_counter()
     for i in range(steps):
-        step(events[i])
+        step(events[i // EVENT_EVERY] if i % EVENT_EVERY == 0 else None)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    return dt, sum(a.elapsed_time(b) for a, b in events) / steps
+    return dt, sum(a.elapsed_time(b) for a, b in events) / len(events)
 
 
 def time_call(torch, fn, reps=20, warmup=3):
@@ -231,16 +241,19 @@ def wl_decode_8b(torch, dev, args):
                 ev[1].record()
             cache.remove_cache(1)
     else:
-        step = FixedStep(torch, cache, q, k1, v1, args.partition)
+        step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
+    fused = args.path == "direct" and not args.no_fuse or args.path == "api"
+    launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
     line = result_line(
         args,
         "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, head_dim 128, "
         "KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
         dec + append_bytes(B, 1, hkv, D), B, dt,
-        roofline("paged_attn_kernel<128,1,...> (decode)", dec, attn_ms, {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
-        {"path": args.path})
+        roofline("paged_attn_kernel<128,1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
+                 {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
+        {"path": args.path, "append_fused": fused})
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
@@ -257,7 +270,7 @@ def wl_ragged(torch, dev, args):
     g = torch.Generator(device=dev).manual_seed(4)
     k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
     q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
-    step = FixedStep(torch, cache, q, k1, v1, args.partition)
+    step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     lens1 = [n + 1 for n in lens]
     dec = decode_bytes(lens1, hq, hkv, D)
@@ -280,7 +293,7 @@ def wl_verify(torch, dev, args):
     g = torch.Generator(device=dev).manual_seed(5)
     kd, vd = _randn_bf16(torch, (B, hkv, S, D), g, dev), _randn_bf16(torch, (B, hkv, S, D), g, dev)
     q = _randn_bf16(torch, (B, hq, S, D), g, dev)
-    step = FixedStep(torch, cache, q, kd, vd, args.partition)
+    step = FixedStep(torch, cache, q, kd, vd, args.partition, fused=not args.no_fuse)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     lens_v = [n + S for n in lens]
     dec = decode_bytes(lens_v, hq, hkv, D, q_len=S)
@@ -409,6 +422,8 @@ def main() -> int:
                          "MultiHeadAttention")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="launch the append as its own kernel instead of fusing it into the attention launch")
     ap.add_argument("--no-permute", action="store_true", help="keep physical blocks in logical order (diagnostic)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -137,6 +137,16 @@ typedef struct pace_paged_attn_args {
   float scale;                /* softmax scale, reference uses 1/sqrt(head_dim)        */
   void* workspace;            /* device scratch, >= pace_paged_attn_workspace_bytes()  */
   size_t workspace_bytes;
+  /* Optional fused append (NULL = off).  The last n_new (1..32) tokens of every sequence, i.e.
+   * positions seq_len - n_new .. seq_len - 1, are read from k_new / v_new
+   * [batch][num_kv_heads][n_new][head_dim] (element strides below, innermost contiguous) instead
+   * of from the pool, and this launch also stores them into their pool slots through the block
+   * table, so no separate append launch is needed for them.  Same contract as pace_kv_append_paged
+   * with pos_offset = -n_new. */
+  const void* k_new;
+  const void* v_new;
+  int64_t new_stride_b, new_stride_h, new_stride_t;
+  int32_t n_new;
 } pace_paged_attn_args_t;
 
 /* Scratch bytes the two entry points below need for these sizes (0 = none). */

@@ -115,3 +115,53 @@ def test_decode_invariant_to_physical_block_permutation(device):
     assert not np.array_equal(cache_a.state.table[:, :5], cache_b.state.table[:, :5])
     out_b = cache_b.attend(q)
     assert torch.equal(out_a.cpu().view(torch.int16), out_b.cpu().view(torch.int16))
+
+
+@pytest.mark.parametrize("T,S,lens,partition", [(1, 1, [40, 200, 1029, 16], 0), (1, 1, [4096, 17], 512), (8, 8, [31, 700], 256),
+                                                (9, 9, [100, 64], 0), (16, 1, [5, 48], 0), (32, 32, [33, 500], 0)])
+def test_fused_append_equals_append_then_attend(device, T, S, lens, partition):
+    """update_cache holds the new tokens back and the attention launch both reads them from the
+    caller's tensors and stores them: same attention result as append-then-attend (to tolerance, the
+    summation order differs) and bit-identical cache contents."""
+    B, hkv, n_rep, D = len(lens), 2, 4, 128
+    outs, caches = [], []
+    k_new, v_new = seeded_kv(900 + T, B, hkv, T, D)
+    q = seeded_q(901, B, hkv * n_rep, S, D)
+    for fuse in (True, False):
+        cache, model = _build(device, B, hkv, n_rep, D, lens, seed=sum(lens) + T, partition=partition)
+        cache.fuse_append = fuse
+        pk, pv = cache.update_cache(repeat_kv(k_new, n_rep).to(device), repeat_kv(v_new, n_rep).to(device), 2)
+        assert (cache._pending is not None) == fuse
+        outs.append(cache.attend(q.to(device)))
+        assert cache._pending is None
+        caches.append(cache)
+    model.append(k_new, v_new)
+    ref = model.attention(q, n_rep)
+    assert_attention_close(outs[0], ref, "fused")
+    assert_attention_close(outs[1], ref, "unfused")
+    for c in caches:
+        gk, gv = c.gather()
+        K, V = model.dense(n_rep)
+        assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
+    # the step after a fused one reads the stored tokens from the pool
+    q1 = seeded_q(902, B, hkv * n_rep, 1, D)
+    k1, v1 = seeded_kv(903, B, hkv, 1, D)
+    caches[0].update_cache(k1.to(device), v1.to(device), 2)
+    model.append(k1, v1)
+    assert_attention_close(caches[0].attend(q1.to(device)), model.attention(q1, n_rep), "step after fused")
+
+
+def test_pending_append_is_flushed_by_other_operations(device):
+    cache, model = _build(device, 2, 2, 2, 128, [20, 37], seed=8)
+    k1, v1 = seeded_kv(1, 2, 2, 1, 128)
+    cache.update_cache(k1.to(device), v1.to(device), 2)
+    model.append(k1, v1)
+    assert cache._pending is not None
+    cache.update_cache(k1.to(device), v1.to(device), 2)  # a second append flushes the first
+    model.append(k1, v1)
+    cache.truncate([1, 0])  # flushes the second
+    model.truncate([1, 0])
+    assert cache._pending is None
+    K, V = model.dense(2)
+    gk, gv = cache.gather()
+    assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
