@@ -64,14 +64,14 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
 template <int D>
 __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
                                                         int32_t table_stride, const int32_t* __restrict__ seq_lens,
-                                                        int32_t n_rep, uint16_t* __restrict__ k_out,
+                                                        int32_t len_bias, int32_t n_rep, uint16_t* __restrict__ k_out,
                                                         uint16_t* __restrict__ v_out, int64_t osb, int64_t osh,
                                                         int32_t out_len) {
   constexpr int CHUNKS = D / 8;                             // 16-byte chunks per row
   constexpr int SLAB_CHUNKS = PACE_KV_BLOCK_TOKENS * CHUNKS;  // per (block, head)
   __shared__ uint16_t vt[D * PACE_KV_BLOCK_TOKENS + 8];
   const int j = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int len = seq_lens[b];
+  const int len = seq_lens[b] + len_bias;
   const int t0 = j * PACE_KV_BLOCK_TOKENS;
   const bool live = t0 < len;  // uniform per workgroup
   int64_t blk = 0;
@@ -188,7 +188,7 @@ extern "C" int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_ne
 }
 
 extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
-                              const int32_t* seq_lens, int32_t batch, int32_t n_rep, void* k_out, void* v_out,
+                              const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep, void* k_out, void* v_out,
                               int64_t out_stride_b, int64_t out_stride_h, int32_t out_len, void* stream) {
   if (int rc = check_pool(pool, "pace_kv_gather")) return rc;
   PACE_REQUIRE(batch >= 0 && out_len >= 0 && n_rep >= 1, "pace_kv_gather: bad batch (%d), out_len (%d) or n_rep (%d)",
@@ -205,11 +205,11 @@ extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_t
   uint16_t* ko = static_cast<uint16_t*>(k_out);
   uint16_t* vo = static_cast<uint16_t*>(v_out);
   if (pool->head_dim == 128)
-    hipLaunchKernelGGL(kv_gather_kernel<128>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, n_rep,
-                       ko, vo, out_stride_b, out_stride_h, out_len);
+    hipLaunchKernelGGL(kv_gather_kernel<128>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias,
+                       n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
   else
-    hipLaunchKernelGGL(kv_gather_kernel<64>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, n_rep, ko,
-                       vo, out_stride_b, out_stride_h, out_len);
+    hipLaunchKernelGGL(kv_gather_kernel<64>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias, n_rep,
+                       ko, vo, out_stride_b, out_stride_h, out_len);
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }

@@ -38,6 +38,7 @@ struct PagedAttnParams {
   const int32_t* table;
   int32_t table_stride;
   const int32_t* seq_lens;
+  int32_t len_bias;
   const int32_t* kv_start;
   const void* mask;
   int32_t mask_is_f32;
@@ -46,6 +47,7 @@ struct PagedAttnParams {
   int32_t n_rep, q_len, num_q_heads;
   int32_t causal;
   int32_t n_qgroups;
+  const int32_t* items;  // optional (sequence, partition) pairs, one per blockIdx.x
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)
@@ -259,6 +261,15 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (
   }
 }
 
+// A sequence of `len` tokens is cut into ceil(len / part_tokens) partitions of equal size
+// (rounded up to whole 32-token units), so no partition is a short remainder.
+__host__ __device__ __forceinline__ int partition_count(int len, int part_tokens) {
+  return len > 0 ? (len + part_tokens - 1) / part_tokens : 1;
+}
+__host__ __device__ __forceinline__ int partition_size(int len, int n_parts) {
+  return (((len + n_parts - 1) / n_parts) + 31) & ~31;
+}
+
 // Pool block ids of one wave's token range: up to 128 blocks (2048 tokens), one id per
 // lane in each of two registers, fetched with one coalesced load each and read back
 // with v_readlane (no memory access inside the unit loop).
@@ -270,13 +281,13 @@ struct WaveBlockIds {
 };
 
 // NW waves per workgroup split the partition's units among themselves and merge their
-// softmax states through LDS.  OCC is the number of such waves that must fit on one SIMD
+// softmax states through LDS.  OCC is the least number of waves that must fit on one SIMD
 // (caps the register budget); latency is hidden by the other resident waves, each wave
 // keeps one unit (16 KiB) in flight.  With FUSED, one more wave per workgroup handles the
 // step's new tokens (attends to them from the caller's buffers and stores them into the
 // pool), so that its dependent round trips overlap with the streaming waves.
 template <int D, int NQT, bool HAS_MASK, int NW, int OCC, bool FUSED>
-__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void paged_attn_kernel(
+__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
@@ -284,12 +295,17 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   static_assert((NWT / 2) * 16 * NQT <= 64, "LDS merge buffer holds 64 query rows");
   __shared__ float merge_buf[64 * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
-  const int part = blockIdx.x, kvh = blockIdx.y;
-  const int b = blockIdx.z / p.n_qgroups, qg = blockIdx.z % p.n_qgroups;
-  const int len = p.seq_lens[b];
-  const int P = p.part_tokens;
-  const int n_parts = len > 0 ? (len + P - 1) / P : 1;
+  const int kvh = blockIdx.y;
+  int part, b, qg;
+  if (p.items) {  // compact work list: no empty workgroups, longest partitions first
+    b = p.items[2 * blockIdx.x], part = p.items[2 * blockIdx.x + 1], qg = blockIdx.z;
+  } else {
+    part = blockIdx.x, b = blockIdx.z / p.n_qgroups, qg = blockIdx.z % p.n_qgroups;
+  }
+  const int len = p.seq_lens[b] + p.len_bias;
+  const int n_parts = partition_count(len, p.part_tokens);
   if (part >= n_parts) return;  // uniform over the workgroup
+  const int P = partition_size(len, n_parts);
   const int start = p.kv_start ? p.kv_start[b] : 0;
   const int part_begin = part * P;
   // Tokens [pool_end, len) are this step's new tokens when the append is fused in.
@@ -461,8 +477,8 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   const int s = (int)(row % S);
   const int hq = (int)((row / S) % p.num_q_heads);
   const int b = (int)(row / ((int64_t)S * p.num_q_heads));
-  const int len = p.seq_lens[b];
-  const int n_parts = len > 0 ? (len + p.part_tokens - 1) / p.part_tokens : 1;
+  const int len = p.seq_lens[b] + p.len_bias;
+  const int n_parts = partition_count(len, p.part_tokens);
   const float* ml = p.part_ml + row * p.max_parts * 2;
   const float* po = p.part_o + row * p.max_parts * D;
   float M = kNegInf;
@@ -605,7 +621,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.v_bs = pool->v_block_stride, p.v_hs = pool->v_head_stride;
   p.num_blocks = pool->num_blocks;
   p.table = a->block_table, p.table_stride = a->table_stride;
-  p.seq_lens = a->seq_lens, p.kv_start = a->kv_start;
+  p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.kv_start = a->kv_start;
   p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
   p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
   p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;
@@ -629,6 +645,12 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   }
   PACE_REQUIRE((int64_t)a->batch * p.n_qgroups <= 65535 && pool->num_kv_heads <= 65535, "%s: grid too large", who);
   dim3 grid(max_parts, pool->num_kv_heads, a->batch * p.n_qgroups);
+  p.items = nullptr;
+  if (a->work_items) {
+    PACE_REQUIRE(a->n_work_items >= 1 && p.n_qgroups <= 65535, "%s: bad n_work_items %d", who, a->n_work_items);
+    p.items = a->work_items;
+    grid = dim3(a->n_work_items, pool->num_kv_heads, p.n_qgroups);
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
   const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, grid, has_mask, s) : launch_shape<64>(sh, p, grid, has_mask, s);
@@ -649,6 +671,12 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
 }  // namespace pace_kv
 
 using namespace pace_kv;
+
+extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t max_seq_len,
+                                                    int32_t partition_tokens, int32_t num_kv_heads) {
+  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
+  return resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, q_len * (num_q_heads / num_kv_heads));
+}
 
 extern "C" size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
                                                   int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 4
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",
@@ -23,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "pace_kv_append_paged",
     "pace_kv_gather",
     "pace_kv_copy_blocks",
+    "pace_paged_attn_partition_tokens",
     "pace_paged_attn_workspace_bytes",
     "pace_paged_attn_decode",
     "pace_paged_attn_verify",
@@ -83,6 +84,9 @@ class PagedAttnArgs(Structure):
         ("new_stride_h", c_int64),
         ("new_stride_t", c_int64),
         ("n_new", c_int32),
+        ("work_items", c_void_p),
+        ("n_work_items", c_int32),
+        ("seq_len_bias", c_int32),
     ]
 
 
@@ -122,10 +126,12 @@ def load() -> ctypes.CDLL:
     ]
     lib.pace_kv_gather.restype = ctypes.c_int
     lib.pace_kv_gather.argtypes = [
-        P, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p,
+        P, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p,
     ]
     lib.pace_kv_copy_blocks.restype = ctypes.c_int
     lib.pace_kv_copy_blocks.argtypes = [P, P, c_void_p, c_int32, c_void_p]
+    lib.pace_paged_attn_partition_tokens.restype = c_int32
+    lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 6
     lib.pace_paged_attn_workspace_bytes.restype = c_size_t
     lib.pace_paged_attn_workspace_bytes.argtypes = [c_int32] * 7
     A = POINTER(PagedAttnArgs)

@@ -246,7 +246,8 @@ class PagedKVCache(KVCacheBase):
         self._flush()
         if counts is None:
             new_lens = self.lens + T
-            st.ensure_capacity(new_lens)
+            if self.seq_len + T > st.min_capacity:
+                st.ensure_capacity(new_lens)
             if self.fuse_append and T <= 32:
                 self._pending = (k, v, head_step)
             else:
@@ -264,18 +265,18 @@ class PagedKVCache(KVCacheBase):
                 )
             )
         self.lens = new_lens
-        self.seq_len = int(new_lens.max(initial=0))
+        self.seq_len = self.seq_len + T if counts is None else int(new_lens.max(initial=0))
         if self.key is None:
             self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
 
     def _launch_append(self, k: torch.Tensor, v: torch.Tensor, head_step: int, lens_after: np.ndarray) -> None:
         st = self.state
         T = k.shape[2]
-        lens_dev, table = st.device_lens(lens_after), st.device_table()
+        (lens_dev, bias), table = st.device_lens(lens_after), st.device_table()
         nat.check(
             nat.load().pace_kv_append_paged(
                 ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
-                self.batch, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -T, nat.current_stream_ptr(),
+                self.batch, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias - T, nat.current_stream_ptr(),
             )
         )
 
@@ -295,7 +296,8 @@ class PagedKVCache(KVCacheBase):
             raise ValueError("Cannot remove more tokens than available in cache.")
         self.lens = self.lens - remove
         self.seq_len = int(self.lens.max(initial=0))
-        self._release()
+        if remove.any():
+            self._release()
 
     def _release(self) -> None:
         # Blocks are shared by every layer: only the longest view of a sequence frees.
@@ -370,10 +372,10 @@ class PagedKVCache(KVCacheBase):
         v = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
         if L:
             st = self.state
-            table, lens_dev = st.device_table(), st.device_lens(self.lens)
+            table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
             nat.check(
                 nat.load().pace_kv_gather(
-                    ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), self.batch, n_rep,
+                    ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, self.batch, n_rep,
                     k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, nat.current_stream_ptr(),
                 )
             )
@@ -396,12 +398,21 @@ class PagedKVCache(KVCacheBase):
             query = query.contiguous()
         out = torch.empty((B, hq, S, D), dtype=torch.bfloat16, device=query.device)
         st = self.state
-        max_len = int(self.lens.max(initial=0))
+        max_len = self.seq_len
         lib = nat.load()
-        ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, self.partition_tokens, self.num_kv_heads))
+        want = self.partition_tokens
+        if want == 0 and B > 1:
+            # A ragged batch is cut at about its mean length: the long sequences then spread over
+            # several workgroups (scheduled longest first) instead of forming the tail of the launch.
+            mean = float(self.lens.mean())
+            if max_len > 1.5 * mean:
+                want = max(1024, (int(mean) + 127) // 128 * 128)
+        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
+        ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
         ws = st.workspace(ws_bytes)
-        table, lens_dev = st.device_table(), st.device_lens(self.lens)
+        table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
         a = nat.PagedAttnArgs()
+        a.seq_len_bias = bias
         a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = query.data_ptr(), query.stride(0), query.stride(1), query.stride(2)
         a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
         a.block_table, a.table_stride = table.data_ptr(), table.stride(0)
@@ -424,7 +435,10 @@ class PagedKVCache(KVCacheBase):
         else:
             a.mask, a.causal = None, 1
         a.batch, a.num_q_heads, a.q_len = B, hq, S
-        a.max_seq_len, a.partition_tokens = max_len, self.partition_tokens
+        a.max_seq_len, a.partition_tokens = max_len, part
+        items = st.work_items(self.lens, part) if part else None
+        if items is not None:
+            a.work_items, a.n_work_items = items.data_ptr(), items.shape[0]
         a.scale = 1.0 / math.sqrt(D)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes

@@ -37,17 +37,22 @@ class BlockAllocator:
     def allocate(self, n: int) -> List[int]:
         if n > len(self._free):
             raise MemoryError(f"KV block pool exhausted: need {n} blocks, {len(self._free)} free of {self.num_blocks}")
-        out = [self._free.pop() for _ in range(n)]
+        if n == 0:
+            return []
+        out = self._free[-n:][::-1]
+        del self._free[-n:]
         self._is_free[out] = False
         return out
 
     def free(self, ids: Iterable[int]) -> None:
-        for i in ids:
-            i = int(i)
-            if self._is_free[i]:
-                raise ValueError(f"block {i} freed twice")
-            self._is_free[i] = True
-            self._free.append(i)
+        ids = [int(i) for i in ids]
+        if not ids:
+            return
+        if self._is_free[ids].any() or len(set(ids)) != len(ids):
+            dup = [i for i in ids if self._is_free[i]] or ids
+            raise ValueError(f"block {dup[0]} freed twice")
+        self._is_free[ids] = True
+        self._free.extend(ids)
 
     def take(self, ids: Iterable[int]) -> None:
         """Mark specific ids as used (compaction destinations)."""
@@ -87,6 +92,9 @@ class PagedState:
         self._lens_dev: Optional[torch.Tensor] = None
         self._lens_host: Optional[np.ndarray] = None
         self._workspace: Optional[torch.Tensor] = None
+        self.min_capacity = 0  # tokens every sequence can hold in the blocks it already owns
+        self._items_key = None
+        self._items_dev: Optional[torch.Tensor] = None
 
     # -- capacity ---------------------------------------------------------------
     def _grow_table(self, need_cols: int) -> None:
@@ -108,6 +116,7 @@ class PagedState:
             self.table[b, have:want] = self.allocator.allocate(want - have)
             self.n_blocks[b] = want
             self._table_dirty = True
+        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
 
     def release_beyond(self, lens: np.ndarray) -> int:
         """Free the blocks no token of ``lens`` touches any more; returns how many."""
@@ -120,6 +129,8 @@ class PagedState:
             self.n_blocks[b] = want
             freed += have - want
             self._table_dirty = True
+        if freed:
+            self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
         return freed
 
     # -- device mirrors ---------------------------------------------------------
@@ -132,22 +143,39 @@ class PagedState:
             self._table_dirty = False
         return self._table_dev
 
-    def device_lens(self, lens: np.ndarray) -> torch.Tensor:
-        """int32 device tensor holding ``lens``; reuses / advances the cached one."""
-        if self._lens_dev is not None and self._lens_host is not None:
+    def device_lens(self, lens: np.ndarray) -> Tuple[torch.Tensor, int]:
+        """``(tensor, bias)`` with ``tensor[b] + bias == lens[b]``: the int32 device mirror is only
+        rewritten when the lengths stop being a uniform shift of what it holds (the kernels add
+        the bias themselves)."""
+        if self._lens_dev is not None:
             delta = lens - self._lens_host
-            if not delta.any():
-                return self._lens_dev
-            if (delta == delta[0]).all():
-                self._lens_dev.add_(int(delta[0]))
-                self._lens_host = lens.copy()
-                return self._lens_dev
+            d0 = int(delta[0]) if delta.size else 0
+            if (delta == d0).all():
+                return self._lens_dev, d0
         host = torch.from_numpy(lens.astype(np.int32))
         if self._lens_dev is None:
             self._lens_dev = torch.empty(self.batch, dtype=torch.int32, device=self.device)
         self._lens_dev.copy_(host.pin_memory(), non_blocking=True)
         self._lens_host = lens.copy()
-        return self._lens_dev
+        return self._lens_dev, 0
+
+    def work_items(self, lens: np.ndarray, part_tokens: int) -> Optional[torch.Tensor]:
+        """Device ``int32 [n][2]`` list of the (sequence, partition) pairs of a ragged batch, longest
+        partitions first; ``None`` for a batch of equal lengths (a dense grid has no empty entries)."""
+        if lens.size == 0 or (lens == lens[0]).all():
+            return None
+        n_parts = np.maximum(1, -(-lens // part_tokens))
+        key = (part_tokens, n_parts.tobytes(), np.argsort(-lens, kind="stable")[:8].tobytes())
+        if key != self._items_key:
+            seq = np.repeat(np.arange(lens.size), n_parts)
+            first = np.repeat(np.cumsum(n_parts) - n_parts, n_parts)
+            part = np.arange(seq.size) - first
+            size = np.repeat(lens / n_parts, n_parts)
+            order = np.argsort(-size, kind="stable")
+            items = np.stack([seq, part], axis=1)[order].astype(np.int32)
+            self._items_dev = torch.from_numpy(items).pin_memory().to(self.device, non_blocking=True)
+            self._items_key = key
+        return self._items_dev
 
     def workspace(self, nbytes: int) -> Optional[torch.Tensor]:
         if nbytes == 0:
@@ -184,6 +212,7 @@ class PagedState:
         self.table[b, : len(keep)] = row
         self.n_blocks[b] = len(keep)
         self._table_dirty = True
+        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
         out = lens.copy()
         out[b] -= removed_tokens
         return out

@@ -111,8 +111,6 @@ class FixedStep:
         self.lens_after = lens_after
         self.out = torch.empty(B, hq, S, D, dtype=torch.bfloat16, device=dev)
         max_len = int(lens_after.max())
-        ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, partition, cache.num_kv_heads))
-        self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         a = nat.PagedAttnArgs()
         a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
         a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = (self.out.data_ptr(), self.out.stride(0), self.out.stride(1),
@@ -120,8 +118,16 @@ class FixedStep:
         a.block_table, a.table_stride, a.seq_lens = self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr()
         a.kv_start, a.mask, a.causal = None, None, 1
         a.batch, a.num_q_heads, a.q_len = B, hq, S
-        a.max_seq_len, a.partition_tokens, a.scale = max_len, partition, 1.0 / math.sqrt(D)
+        if partition == 0 and max_len > 1.5 * float(lens_after.mean()):  # same rule as PagedKVCache.attend
+            partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
+        part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, partition, cache.num_kv_heads))
+        a.max_seq_len, a.partition_tokens, a.scale = max_len, part, 1.0 / math.sqrt(D)
+        ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, cache.num_kv_heads))
+        self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
+        self.items = cache.state.work_items(lens_after, part)  # ragged batches: compact, longest-first work list
+        if self.items is not None:
+            a.work_items, a.n_work_items = self.items.data_ptr(), self.items.shape[0]
         self.fused = fused
         if fused:  # the attention launch reads the new tokens from k_new / v_new and stores them into the pool
             a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
@@ -222,7 +228,8 @@ def result_line(args, workload, step_bytes, tokens_per_step, dt, roof, extra_cfg
 # ---- workloads ---------------------------------------------------------------------------------
 def wl_decode_8b(torch, dev, args):
     B, ctx, hq, hkv, D = 64, 4096, 32, 8, 128
-    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute)
+    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute,
+                        headroom=64 + args.steps + args.warmup)
     cache.partition_tokens = args.partition
     g = torch.Generator(device=dev).manual_seed(2)
     k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
@@ -233,16 +240,17 @@ def wl_decode_8b(torch, dev, args):
         mha = MultiHeadAttention(dtype=torch.bfloat16)
 
         def step(ev=None):
-            pk, pv = cache.update_cache(k1, v1, 2)
+            pk, pv = cache.update_cache(k1, v1, 2)  # the context grows by one token per step on this path
             if ev:
                 ev[0].record()
             mha(q, pk, pv)
             if ev:
                 ev[1].record()
-            cache.remove_cache(1)
     else:
         step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    if args.path == "api":  # average context over the timed steps
+        ctx = ctx + args.warmup + (args.steps - 1) // 2
     dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
     fused = args.path == "direct" and not args.no_fuse or args.path == "api"
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)

@@ -101,10 +101,11 @@ int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_new, const vo
  * repeat_kv, pace/llm/models/llama.py:151-158): k_out / v_out are bf16
  * [batch][num_kv_heads*n_rep][out_len][head_dim] with the element strides
  * given (rows contiguous); rows >= seq_lens[b] are written as zeros.
- * block_table: device int32 [batch][table_stride]; seq_lens: device int32 [batch].
+ * block_table: device int32 [batch][table_stride]; seq_lens: device int32 [batch]
+ * (length of sequence b = seq_lens[b] + seq_len_bias).
  */
 int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
-                   const int32_t* seq_lens, int32_t batch, int32_t n_rep,
+                   const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep,
                    void* k_out, void* v_out, int64_t out_stride_b, int64_t out_stride_h,
                    int32_t out_len, void* stream);
 
@@ -124,7 +125,8 @@ typedef struct pace_paged_attn_args {
   int64_t o_stride_b, o_stride_h, o_stride_s;
   const int32_t* block_table; /* device int32 [batch][table_stride]                  */
   int32_t table_stride;
-  const int32_t* seq_lens;    /* device int32 [batch]: tokens in cache incl. the q_len new ones */
+  const int32_t* seq_lens;    /* device int32 [batch]; length of sequence b = seq_lens[b] + seq_len_bias:
+                                 tokens in cache incl. the q_len new ones                */
   const int32_t* kv_start;    /* optional device int32 [batch]: first readable token (left padding) */
   const void* mask;           /* optional additive mask [batch|1][1][q_len|1][mask_len]  */
   int32_t mask_dtype;         /* PACE_DTYPE_F32 / PACE_DTYPE_BF16                      */
@@ -147,7 +149,21 @@ typedef struct pace_paged_attn_args {
   const void* v_new;
   int64_t new_stride_b, new_stride_h, new_stride_t;
   int32_t n_new;
+  /* Optional compact work list (NULL = a dense partition x sequence grid).  Device int32
+   * [n_work_items][2] = (sequence, partition): exactly the pairs with partition <
+   * ceil(seq_len / partition_tokens), in the order they should be scheduled (longest first
+   * shortens the tail of a ragged batch).  Needs an explicit partition_tokens. */
+  const int32_t* work_items;
+  int32_t n_work_items;
+  int32_t seq_len_bias;       /* host-side constant added to every seq_lens entry, so that uniform
+                                 appends / rollbacks need no device update of the lengths */
 } pace_paged_attn_args_t;
+
+/* The context split size (tokens per workgroup) the library uses for these sizes when
+ * partition_tokens is 0; a sequence of n tokens is cut into ceil(n / split) equal partitions. */
+int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len,
+                                         int32_t max_seq_len, int32_t partition_tokens,
+                                         int32_t num_kv_heads);
 
 /* Scratch bytes the two entry points below need for these sizes (0 = none). */
 size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len,
