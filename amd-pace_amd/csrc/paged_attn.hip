@@ -47,6 +47,8 @@ struct PagedAttnParams {
   int32_t n_rep, q_len, num_q_heads;
   int32_t causal;
   int32_t n_qgroups;
+  int32_t num_kv_heads;
+  long long total_items;  // work items of the launch: KV heads x row groups x (sequence, partition) pairs
   const int32_t* items;  // optional (sequence, partition) pairs, one per blockIdx.x
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
@@ -270,6 +272,12 @@ __host__ __device__ __forceinline__ int partition_size(int len, int n_parts) {
   return (((len + n_parts - 1) / n_parts) + 31) & ~31;
 }
 
+#ifdef PACE_PROBE_TIMING
+// Measurement aid: per-wave timestamps (100 MHz clock) of the phases of one launch.
+__device__ long long g_probe[1 << 20];
+__device__ unsigned int g_probe_n;
+#endif
+
 // Pool block ids of one wave's token range: up to 128 blocks (2048 tokens), one id per
 // lane in each of two registers, fetched with one coalesced load each and read back
 // with v_readlane (no memory access inside the unit loop).
@@ -282,29 +290,49 @@ struct WaveBlockIds {
 
 // NW waves per workgroup split the partition's units among themselves and merge their
 // softmax states through LDS.  OCC is the least number of waves that must fit on one SIMD
-// (caps the register budget); latency is hidden by the other resident waves, each wave
-// keeps one unit (16 KiB) in flight.  With FUSED, one more wave per workgroup handles the
+// (caps the register budget) and OCC_MAX the most that may share it; latency is hidden by
+// the other resident waves, each wave keeps one unit (16 KiB) in flight.  With FUSED, one more wave per workgroup handles the
 // step's new tokens (attends to them from the caller's buffers and stores them into the
 // pool), so that its dependent round trips overlap with the streaming waves.
-template <int D, int NQT, bool HAS_MASK, int NW, int OCC, bool FUSED>
-__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC))) void paged_attn_kernel(
+template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED>
+__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC_MAX))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-  constexpr int NWT = NW + (FUSED ? 1 : 0);  // waves in the workgroup
-  static_assert((NWT / 2) * 16 * NQT <= 64, "LDS merge buffer holds 64 query rows");
-  __shared__ float merge_buf[64 * (D + 2)];
+  constexpr int NWT = NW + (FUSED ? 1 : 0);  // waves per work item
+  // One slot of 16*NQT query rows per sender of the first merge round.  Kept as small as the
+  // shape allows: LDS is one of the limits on how many workgroups share a compute unit.
+  constexpr int MERGE_SLOTS = NWT / 2 > 0 ? NWT / 2 : 1;
+  static_assert(MERGE_SLOTS * 16 * NQT <= 64, "LDS merge buffer holds at most 64 query rows");
+  __shared__ float merge_buf[MERGE_SLOTS * 16 * NQT * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
-  const int kvh = blockIdx.y;
-  int part, b, qg;
-  if (p.items) {  // compact work list: no empty workgroups, longest partitions first
-    b = p.items[2 * blockIdx.x], part = p.items[2 * blockIdx.x + 1], qg = blockIdx.z;
-  } else {
-    part = blockIdx.x, b = blockIdx.z / p.n_qgroups, qg = blockIdx.z % p.n_qgroups;
+#ifdef PACE_PROBE_TIMING
+  const long long pt0 = wall_clock64();
+#endif
+  // Linear work index -> (KV head, row group, sequence, partition); KV head fastest.
+  const long long L = blockIdx.x;
+  const bool active_item = L < p.total_items;
+  int kvh = 0, part = 0, b = 0, qg = 0;
+  if (active_item) {
+    kvh = (int)(L % p.num_kv_heads);
+    const long long rest = L / p.num_kv_heads;
+    if (p.items) {  // compact work list: no empty entries, longest partitions first
+      qg = (int)(rest % p.n_qgroups);
+      const long long item = rest / p.n_qgroups;
+      b = p.items[2 * item], part = p.items[2 * item + 1];
+    } else {
+      part = (int)(rest % p.max_parts);
+      const long long bz = rest / p.max_parts;
+      b = (int)(bz / p.n_qgroups), qg = (int)(bz % p.n_qgroups);
+    }
   }
-  const int len = p.seq_lens[b] + p.len_bias;
+  const int len_b = p.seq_lens[b] + p.len_bias;
+  // An idle slot (past the end of the work, or a partition this sequence does not have) runs
+  // as an empty sequence without query rows: it loads and stores nothing but keeps the barriers.
+  const bool active = active_item && part < partition_count(len_b, p.part_tokens);
+  const int len = active ? len_b : 0;
   const int n_parts = partition_count(len, p.part_tokens);
-  if (part >= n_parts) return;  // uniform over the workgroup
+  if (!active) part = 0;
   const int P = partition_size(len, n_parts);
   const int start = p.kv_start ? p.kv_start[b] : 0;
   const int part_begin = part * P;
@@ -312,7 +340,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   const int n_new = FUSED ? min(p.n_new, len) : 0;
   const int pool_end = len - n_new;
   const int tok_end = min(pool_end, part_begin + P);
-  const int S = p.q_len, R = S * p.n_rep;
+  const int S = p.q_len, R = active ? S * p.n_rep : 0;
   // This wave's share of the partition's 32-token units.
   const int part_units = max(0, (tok_end - part_begin + 31) / 32);
   const int per_wave = (part_units + NW - 1) / NW;
@@ -374,6 +402,9 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g);
     }
   }
+#ifdef PACE_PROBE_TIMING
+  const long long pt1 = wall_clock64();
+#endif
   for (int uu = 0; uu < n_units; ++uu) {
     load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const int t0 = tok_begin + 32 * uu;
@@ -381,6 +412,9 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g);
   }
 
+#ifdef PACE_PROBE_TIMING
+  const long long pt2 = wall_clock64();
+#endif
   // Row sums were kept per lane; complete them over the four lanes of a row.
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
@@ -437,6 +471,16 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       }
       __syncthreads();
     }
+#ifdef PACE_PROBE_TIMING
+    if (wave != 0 && lane == 0) {
+      const long long pt3 = wall_clock64();
+      const unsigned int slot = atomicAdd(&g_probe_n, 1u);
+      if (slot < (1u << 20) / 8) {
+        long long* o = g_probe + 8ull * slot;
+        o[0] = pt0, o[1] = pt1, o[2] = pt2, o[3] = pt3, o[4] = n_units, o[5] = (long long)kvh, o[6] = wave + 16 * (long long)__smid(), o[7] = b;
+      }
+    }
+#endif
     if (wave != 0) return;
   }
 
@@ -467,6 +511,16 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       }
     }
   }
+#ifdef PACE_PROBE_TIMING
+  if (lane == 0) {
+    const long long pt3 = wall_clock64();
+    const unsigned int slot = atomicAdd(&g_probe_n, 1u);
+    if (slot < (1u << 20) / 8) {
+      long long* o = g_probe + 8ull * slot;
+      o[0] = pt0, o[1] = pt1, o[2] = pt2, o[3] = pt3, o[4] = n_units, o[5] = (long long)kvh, o[6] = wave + 16 * (long long)__smid(), o[7] = b;
+    }
+  }
+#endif
 }
 
 // Merge the partitions of one query row: out = sum_p 2^(m_p - M) o_p / sum_p 2^(m_p - M) l_p.
@@ -507,11 +561,12 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
 // Launch shape per query-tile count: waves per workgroup and unit buffers per wave.
 struct Shape {
   int nqt, nw, occ;
+  int occ_max;  // 8: no limit; 2: with five waves per workgroup, one workgroup per compute unit
 };
 
 static Shape shape_for(int tiles) {
   if (tiles <= 1) {
-    Shape s = {1, 4, 2};
+    Shape s = {1, 4, 2, 8};
     // Tuning override for the single-tile (decode) kernel: "NW,OCC".
     if (const char* e = getenv("PACE_KV_DECODE_SHAPE")) {
       int nw = 0, occ = 0;
@@ -519,11 +574,23 @@ static Shape shape_for(int tiles) {
     }
     return s;
   }
-  if (tiles == 2) return Shape{2, 4, 2};
-  return Shape{4, 2, 1};
+  if (tiles == 2) return Shape{2, 4, 2, 8};
+  return Shape{4, 2, 1, 8};
 }
 
-// Tokens one workgroup may cover: each wave holds at most 128 block ids.
+static int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
+// Tokens one work item may cover: each wave holds at most 128 block ids.
 static int max_partition(int nw) { return nw * 2048; }
 
 static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
@@ -543,10 +610,12 @@ static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t bat
   return (int)per;
 }
 
-template <int D, int NQT, int NW, int OCC>
-static void launch(const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
+template <int D, int NQT, int NW, int OCC, int OCC_MAX>
+static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   const bool fused = p.n_new > 0;
-#define PACE_GO(M_, F_) hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, F_>), grid, dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+  const unsigned blocks = (unsigned)p.total_items;
+#define PACE_GO(M_, F_) \
+  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
   if (has_mask) {
     if (fused) PACE_GO(true, true); else PACE_GO(true, false);
   } else {
@@ -556,17 +625,17 @@ static void launch(const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream
 }
 
 template <int D>
-static bool launch_shape(const Shape& sh, const PagedAttnParams& p, dim3 grid, bool has_mask, hipStream_t s) {
-#define PACE_TRY(NQT_, NW_, OCC_)                                  \
-  if (sh.nqt == NQT_ && sh.nw == NW_ && sh.occ == OCC_) {            \
-    launch<D, NQT_, NW_, OCC_>(p, grid, has_mask, s);                \
-    return true;                                                     \
+static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mask, hipStream_t s) {
+#define PACE_TRY(NQT_, NW_, OCC_, MAX_)                                          \
+  if (sh.nqt == NQT_ && sh.nw == NW_ && sh.occ == OCC_ && sh.occ_max == MAX_) {     \
+    launch<D, NQT_, NW_, OCC_, MAX_>(p, has_mask, s);                               \
+    return true;                                                                    \
   }
-  PACE_TRY(1, 4, 2)
-  PACE_TRY(1, 4, 3)
-  PACE_TRY(1, 8, 2)
-  PACE_TRY(2, 4, 2)
-  PACE_TRY(4, 2, 1)
+  PACE_TRY(1, 4, 2, 8)
+  PACE_TRY(1, 4, 2, 2)
+  PACE_TRY(1, 8, 2, 8)
+  PACE_TRY(2, 4, 2, 8)
+  PACE_TRY(4, 2, 1, 8)
 #undef PACE_TRY
   return false;
 }
@@ -643,18 +712,28 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     p.part_o = static_cast<float*>(a->workspace);
     p.part_ml = p.part_o + rows_total * max_parts * pool->head_dim;
   }
-  PACE_REQUIRE((int64_t)a->batch * p.n_qgroups <= 65535 && pool->num_kv_heads <= 65535, "%s: grid too large", who);
-  dim3 grid(max_parts, pool->num_kv_heads, a->batch * p.n_qgroups);
+  p.num_kv_heads = pool->num_kv_heads;
   p.items = nullptr;
+  long long pairs = (long long)a->batch * max_parts;  // (sequence, partition) pairs of the dense grid
   if (a->work_items) {
-    PACE_REQUIRE(a->n_work_items >= 1 && p.n_qgroups <= 65535, "%s: bad n_work_items %d", who, a->n_work_items);
+    PACE_REQUIRE(a->n_work_items >= 1, "%s: bad n_work_items %d", who, a->n_work_items);
     p.items = a->work_items;
-    grid = dim3(a->n_work_items, pool->num_kv_heads, p.n_qgroups);
+    pairs = a->n_work_items;
   }
+  p.total_items = pairs * pool->num_kv_heads * p.n_qgroups;
+  PACE_REQUIRE(p.total_items < (1ll << 31), "%s: grid too large", who);
+  Shape launch_shape_sel = sh;
+  // Two rounds of one workgroup per compute unit beat one round of two: when two workgroups
+  // share a compute unit, the waves placed second on each SIMD fall behind and leave a long
+  // under-filled tail.  Applies to the fused decode shape (five waves per workgroup, so that
+  // a two-waves-per-SIMD limit means one workgroup per compute unit).
+  if (sh.nqt == 1 && sh.nw == 4 && p.n_new > 0 && !getenv("PACE_KV_DECODE_SHAPE") && p.total_items > compute_units() &&
+      p.total_items <= 2ll * compute_units())
+    launch_shape_sel.occ_max = 2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
-  const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, grid, has_mask, s) : launch_shape<64>(sh, p, grid, has_mask, s);
-  PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d", who, sh.nqt, sh.nw, sh.occ);
+  const bool ok = pool->head_dim == 128 ? launch_shape<128>(launch_shape_sel, p, has_mask, s) : launch_shape<64>(launch_shape_sel, p, has_mask, s);
+  PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
@@ -671,6 +750,18 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
 }  // namespace pace_kv
 
 using namespace pace_kv;
+
+#ifdef PACE_PROBE_TIMING
+extern "C" int pace_probe_read(long long* host, unsigned int* n, int reset) {
+  hipMemcpyFromSymbol(n, HIP_SYMBOL(g_probe_n), sizeof(unsigned int));
+  hipMemcpyFromSymbol(host, HIP_SYMBOL(g_probe), sizeof(long long) * (1 << 20));
+  if (reset) {
+    unsigned int z = 0;
+    hipMemcpyToSymbol(HIP_SYMBOL(g_probe_n), &z, sizeof(z));
+  }
+  return 0;
+}
+#endif
 
 extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t max_seq_len,
                                                     int32_t partition_tokens, int32_t num_kv_heads) {

@@ -422,8 +422,8 @@ WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="decode-8b")
     ap.add_argument("--path", choices=("api", "direct"), default="direct",
                     help="decode-8b only. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
