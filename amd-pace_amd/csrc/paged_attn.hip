@@ -49,7 +49,8 @@ struct PagedAttnParams {
   int32_t n_qgroups;
   int32_t num_kv_heads;
   long long total_items;  // work items of the launch: KV heads x row groups x (sequence, partition) pairs
-  const int32_t* items;  // optional (sequence, partition) pairs, one per blockIdx.x
+  const int32_t* items;  // optional (sequence, partition) pairs
+  const int32_t* seq_parts;  // optional partitions per sequence (else derived from part_tokens)
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)
@@ -329,9 +330,10 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   const int len_b = p.seq_lens[b] + p.len_bias;
   // An idle slot (past the end of the work, or a partition this sequence does not have) runs
   // as an empty sequence without query rows: it loads and stores nothing but keeps the barriers.
-  const bool active = active_item && part < partition_count(len_b, p.part_tokens);
+  const int n_parts_b = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len_b, p.part_tokens);
+  const bool active = active_item && part < n_parts_b;
   const int len = active ? len_b : 0;
-  const int n_parts = partition_count(len, p.part_tokens);
+  const int n_parts = active ? n_parts_b : 1;
   if (!active) part = 0;
   const int P = partition_size(len, n_parts);
   const int start = p.kv_start ? p.kv_start[b] : 0;
@@ -532,7 +534,7 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   const int hq = (int)((row / S) % p.num_q_heads);
   const int b = (int)(row / ((int64_t)S * p.num_q_heads));
   const int len = p.seq_lens[b] + p.len_bias;
-  const int n_parts = partition_count(len, p.part_tokens);
+  const int n_parts = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len, p.part_tokens);
   const float* ml = p.part_ml + row * p.max_parts * 2;
   const float* po = p.part_o + row * p.max_parts * D;
   float M = kNegInf;
@@ -564,7 +566,7 @@ struct Shape {
   int occ_max;  // 8: no limit; 2: with five waves per workgroup, one workgroup per compute unit
 };
 
-static Shape shape_for(int tiles) {
+static Shape shape_for(int tiles, bool fused) {
   if (tiles <= 1) {
     Shape s = {1, 4, 2, 8};
     // Tuning override for the single-tile (decode) kernel: "NW,OCC".
@@ -574,7 +576,10 @@ static Shape shape_for(int tiles) {
     }
     return s;
   }
-  if (tiles == 2) return Shape{2, 4, 2, 8};
+  // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit.
+  // Four waves per workgroup (three streaming + the append wave when fused) keep two
+  // workgroups on a compute unit.
+  if (tiles == 2) return Shape{2, fused ? 3 : 4, 2, 8};
   return Shape{4, 2, 1, 8};
 }
 
@@ -593,10 +598,17 @@ static int compute_units() {
 // Tokens one work item may cover: each wave holds at most 128 block ids.
 static int max_partition(int nw) { return nw * 2048; }
 
+// Largest partition any shape of this tile count can take (fused or not), so that one
+// resolved value is valid for every launch of the same problem size.
+static int partition_cap(int tiles) {
+  const Shape a = shape_for(tiles, false), b = shape_for(tiles, true);
+  return max_partition(a.nw < b.nw ? a.nw : b.nw);
+}
+
 static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
   const int tiles = (rows + 15) / 16;
-  const Shape sh = shape_for(tiles);
-  const int granule = 32 * sh.nw;
+  const Shape sh = shape_for(tiles, false);
+  const int granule = 128;
   if (requested > 0) return requested;
   // Enough workgroups to give every compute unit (256) two of them; a batch that
   // already does so is not split at all.
@@ -606,7 +618,7 @@ static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t bat
   int64_t per = ((int64_t)max_seq_len + parts - 1) / parts;
   per = (per + granule - 1) / granule * granule;
   if (per < granule) per = granule;
-  if (per > max_partition(sh.nw)) per = max_partition(sh.nw);
+  if (per > partition_cap(tiles)) per = partition_cap(tiles);
   return (int)per;
 }
 
@@ -635,6 +647,7 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   PACE_TRY(1, 4, 2, 2)
   PACE_TRY(1, 8, 2, 8)
   PACE_TRY(2, 4, 2, 8)
+  PACE_TRY(2, 3, 2, 8)
   PACE_TRY(4, 2, 1, 8)
 #undef PACE_TRY
   return false;
@@ -673,11 +686,17 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
   const int tiles = (rows + 15) / 16;
-  const Shape sh = shape_for(tiles);
+  const bool fused_req = a->k_new != nullptr;
+  const Shape sh = shape_for(tiles, fused_req);
   const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
   PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
-               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, max_partition(sh.nw));
-  const int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
+               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(tiles));
+  int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
+  if (a->seq_parts) {
+    PACE_REQUIRE(a->work_items != nullptr && a->max_parts >= 1,
+                 "%s: seq_parts needs a work list and max_parts (the largest entry of seq_parts)", who);
+    max_parts = a->max_parts;
+  }
 
   PagedAttnParams p;
   p.q = static_cast<const uint16_t*>(a->q);
@@ -714,6 +733,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   }
   p.num_kv_heads = pool->num_kv_heads;
   p.items = nullptr;
+  p.seq_parts = a->seq_parts;
   long long pairs = (long long)a->batch * max_parts;  // (sequence, partition) pairs of the dense grid
   if (a->work_items) {
     PACE_REQUIRE(a->n_work_items >= 1, "%s: bad n_work_items %d", who, a->n_work_items);
@@ -776,6 +796,12 @@ extern "C" size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_h
   const int part = resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, rows);
   const int max_parts = (max_seq_len + part - 1) / part;
   if (max_parts <= 1) return 0;
+  return (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float);
+}
+
+extern "C" size_t pace_paged_attn_workspace_bytes_for_parts(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
+                                                            int32_t max_parts) {
+  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_parts <= 1) return 0;
   return (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float);
 }
 

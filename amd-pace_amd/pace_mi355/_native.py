@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",
@@ -25,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "pace_kv_copy_blocks",
     "pace_paged_attn_partition_tokens",
     "pace_paged_attn_workspace_bytes",
+    "pace_paged_attn_workspace_bytes_for_parts",
     "pace_paged_attn_decode",
     "pace_paged_attn_verify",
     "pace_attn_dense",
@@ -86,6 +87,8 @@ class PagedAttnArgs(Structure):
         ("n_new", c_int32),
         ("work_items", c_void_p),
         ("n_work_items", c_int32),
+        ("seq_parts", c_void_p),
+        ("max_parts", c_int32),
         ("seq_len_bias", c_int32),
     ]
 
@@ -134,6 +137,8 @@ def load() -> ctypes.CDLL:
     lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 6
     lib.pace_paged_attn_workspace_bytes.restype = c_size_t
     lib.pace_paged_attn_workspace_bytes.argtypes = [c_int32] * 7
+    lib.pace_paged_attn_workspace_bytes_for_parts.restype = c_size_t
+    lib.pace_paged_attn_workspace_bytes_for_parts.argtypes = [c_int32] * 5
     A = POINTER(PagedAttnArgs)
     lib.pace_paged_attn_decode.restype = ctypes.c_int
     lib.pace_paged_attn_decode.argtypes = [P, A, c_void_p]

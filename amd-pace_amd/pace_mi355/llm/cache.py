@@ -408,7 +408,17 @@ class PagedKVCache(KVCacheBase):
             if max_len > 1.5 * mean:
                 want = max(1024, (int(mean) + 127) // 128 * 128)
         part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
-        ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
+        items = parts = None
+        max_parts = 1
+        if part:
+            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, self.num_kv_heads))
+            row_groups = -(-(S * (hq // self.num_kv_heads)) // 64)
+            slots = max(1, 512 // (self.num_kv_heads * row_groups))
+            items, parts, max_parts = st.plan_attention(self.lens, part, cap, slots)
+        if parts is not None:
+            ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
+        else:
+            ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
         ws = st.workspace(ws_bytes)
         table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
         a = nat.PagedAttnArgs()
@@ -436,9 +446,10 @@ class PagedKVCache(KVCacheBase):
             a.mask, a.causal = None, 1
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         a.max_seq_len, a.partition_tokens = max_len, part
-        items = st.work_items(self.lens, part) if part else None
         if items is not None:
             a.work_items, a.n_work_items = items.data_ptr(), items.shape[0]
+        if parts is not None:
+            a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
         a.scale = 1.0 / math.sqrt(D)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes

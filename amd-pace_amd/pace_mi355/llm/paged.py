@@ -95,6 +95,8 @@ class PagedState:
         self.min_capacity = 0  # tokens every sequence can hold in the blocks it already owns
         self._items_key = None
         self._items_dev: Optional[torch.Tensor] = None
+        self._parts_dev: Optional[torch.Tensor] = None
+        self._max_parts = 1
 
     # -- capacity ---------------------------------------------------------------
     def _grow_table(self, need_cols: int) -> None:
@@ -159,23 +161,54 @@ class PagedState:
         self._lens_host = lens.copy()
         return self._lens_dev, 0
 
-    def work_items(self, lens: np.ndarray, part_tokens: int) -> Optional[torch.Tensor]:
-        """Device ``int32 [n][2]`` list of the (sequence, partition) pairs of a ragged batch, longest
-        partitions first; ``None`` for a batch of equal lengths (a dense grid has no empty entries)."""
-        if lens.size == 0 or (lens == lens[0]).all():
-            return None
-        n_parts = np.maximum(1, -(-lens // part_tokens))
-        key = (part_tokens, n_parts.tobytes(), np.argsort(-lens, kind="stable")[:8].tobytes())
+    def plan_attention(self, lens: np.ndarray, part_tokens: int, part_cap: int, slots: int):
+        """How to cut the sequences of a batch for one attention launch.
+
+        Returns ``(items, seq_parts, max_parts)``: ``items`` is a device ``int32 [n][2]`` list of
+        (sequence, partition) pairs, longest partitions first, or ``None`` when a dense grid has no
+        empty entries (equal lengths, one partition rule).  ``seq_parts`` (device ``int32 [B]``) is
+        set when the whole launch fits the GPU in one round: the partition counts are then chosen
+        so that the partitions are as equal as possible and fill the ``slots`` workgroup slots
+        (largest-remainder apportionment), instead of all sequences being cut at one length.
+        """
+        if lens.size == 0:
+            return None, None, 1
+        base = np.maximum(1, -(-lens // part_tokens))
+        uniform = bool((lens == lens[0]).all())
+        cap_parts = np.maximum(1, -(-lens // part_cap))
+        if not uniform and int(cap_parts.sum()) < slots and int(base.sum()) <= slots:
+            key = ("even", part_cap, slots, (lens // 64).tobytes())
+            if key != self._items_key:
+                n = cap_parts.copy()
+                size = lens / n
+                while int(n.sum()) < slots:
+                    b = int(np.argmax(size))
+                    if lens[b] / (n[b] + 1) < 256:
+                        break
+                    n[b] += 1
+                    size[b] = lens[b] / n[b]
+                self._store_items(key, lens, n, with_parts=True)
+            return self._items_dev, self._parts_dev, self._max_parts
+        if uniform:
+            return None, None, int(base.max())
+        key = ("cut", part_tokens, base.tobytes(), np.argsort(-lens, kind="stable")[:8].tobytes())
         if key != self._items_key:
-            seq = np.repeat(np.arange(lens.size), n_parts)
-            first = np.repeat(np.cumsum(n_parts) - n_parts, n_parts)
-            part = np.arange(seq.size) - first
-            size = np.repeat(lens / n_parts, n_parts)
-            order = np.argsort(-size, kind="stable")
-            items = np.stack([seq, part], axis=1)[order].astype(np.int32)
-            self._items_dev = torch.from_numpy(items).pin_memory().to(self.device, non_blocking=True)
-            self._items_key = key
-        return self._items_dev
+            self._store_items(key, lens, base, with_parts=False)
+        return self._items_dev, None, int(base.max())
+
+    def _store_items(self, key, lens: np.ndarray, n_parts: np.ndarray, with_parts: bool) -> None:
+        seq = np.repeat(np.arange(lens.size), n_parts)
+        first = np.repeat(np.cumsum(n_parts) - n_parts, n_parts)
+        part = np.arange(seq.size) - first
+        size = np.repeat(lens / n_parts, n_parts)
+        order = np.argsort(-size, kind="stable")
+        items = np.stack([seq, part], axis=1)[order].astype(np.int32)
+        self._items_dev = torch.from_numpy(items).pin_memory().to(self.device, non_blocking=True)
+        self._parts_dev = (
+            torch.from_numpy(n_parts.astype(np.int32)).pin_memory().to(self.device, non_blocking=True) if with_parts else None
+        )
+        self._max_parts = int(n_parts.max())
+        self._items_key = key
 
     def workspace(self, nbytes: int) -> Optional[torch.Tensor]:
         if nbytes == 0:

@@ -121,11 +121,19 @@ class FixedStep:
         if partition == 0 and max_len > 1.5 * float(lens_after.mean()):  # same rule as PagedKVCache.attend
             partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
         part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, partition, cache.num_kv_heads))
+        cap = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, cache.num_kv_heads))
+        row_groups = -(-(S * (hq // cache.num_kv_heads)) // 64)
+        slots = max(1, 512 // (cache.num_kv_heads * row_groups))
+        # ragged batches: compact longest-first work list; single-round launches: evened-out partition counts
+        self.items, self.parts, max_parts = cache.state.plan_attention(lens_after, part, cap, slots)
         a.max_seq_len, a.partition_tokens, a.scale = max_len, part, 1.0 / math.sqrt(D)
-        ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, cache.num_kv_heads))
+        if self.parts is not None:
+            ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
+            a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
+        else:
+            ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, cache.num_kv_heads))
         self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
-        self.items = cache.state.work_items(lens_after, part)  # ragged batches: compact, longest-first work list
         if self.items is not None:
             a.work_items, a.n_work_items = self.items.data_ptr(), self.items.shape[0]
         self.fused = fused

@@ -155,6 +155,14 @@ typedef struct pace_paged_attn_args {
    * shortens the tail of a ragged batch).  Needs an explicit partition_tokens. */
   const int32_t* work_items;
   int32_t n_work_items;
+  /* Optional partition count per sequence (device int32 [batch], NULL = ceil(seq_len /
+   * partition_tokens)); sequence b is cut into seq_parts[b] equal partitions, none longer than
+   * pace_paged_attn_partition_tokens(...)'s upper bound.  Needs work_items listing exactly
+   * (b, 0 .. seq_parts[b]-1), max_parts = the largest entry, and a workspace of
+   * pace_paged_attn_workspace_bytes_for_parts(...).  Lets the caller even out the work when
+   * the whole launch fits the GPU in one round. */
+  const int32_t* seq_parts;
+  int32_t max_parts;
   int32_t seq_len_bias;       /* host-side constant added to every seq_lens entry, so that uniform
                                  appends / rollbacks need no device update of the lengths */
 } pace_paged_attn_args_t;
@@ -169,6 +177,9 @@ int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int
 size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len,
                                        int32_t head_dim, int32_t max_seq_len,
                                        int32_t partition_tokens, int32_t num_kv_heads);
+
+size_t pace_paged_attn_workspace_bytes_for_parts(int32_t batch, int32_t num_q_heads, int32_t q_len,
+                                                 int32_t head_dim, int32_t max_parts);
 
 /*
  * Decode attention over the paged cache, q_len == 1.

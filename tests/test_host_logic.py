@@ -238,3 +238,42 @@ def test_evict_and_compaction_plan_properties():
         assert st.table[b, : st.n_blocks[b]].tolist() == [remap.get(x, x) for x in logical[b].tolist()]
     assert sorted(st.allocator.free_ids().tolist()) == list(range(live, 120))
     assert len(st.plan_compaction()) == 0  # idempotent
+
+
+# ---- attention launch planning ----
+def test_plan_attention_uniform_batch_uses_dense_grid():
+    st = _state(batch=4, max_len=8192, blocks=4 * 512)
+    items, parts, max_parts = st.plan_attention(np.full(4, 4097), 4224, 8192, 64)
+    assert items is None and parts is None and max_parts == 1
+    items, parts, max_parts = st.plan_attention(np.full(4, 4097), 1024, 8192, 64)
+    assert items is None and parts is None and max_parts == 5
+
+
+def test_plan_attention_multi_round_batch_is_cut_and_sorted_longest_first():
+    st = _state(batch=6, max_len=20000, blocks=10)
+    lens = np.array([100, 5000, 16385, 300, 2048, 9000])
+    items, parts, max_parts = st.plan_attention(lens, 2048, 8192, slots=8)  # 8 slots < 18 partitions: several rounds
+    assert parts is None and max_parts == 9
+    it = items.numpy()
+    n = np.maximum(1, -(-lens // 2048))
+    assert len(it) == n.sum()
+    assert sorted(map(tuple, it.tolist())) == sorted((b, p) for b in range(6) for p in range(n[b]))
+    sizes = (lens / n)[it[:, 0]]
+    assert (np.diff(sizes) <= 1e-9).all(), "longest partitions first"
+    again, _, _ = st.plan_attention(lens + 1, 2048, 8192, slots=8)  # same partition counts: cached list
+    assert again is items
+
+
+def test_plan_attention_single_round_batch_gets_even_partitions():
+    st = _state(batch=5, max_len=9000, blocks=10)
+    lens = np.array([1024, 8192, 4000, 2500, 6000])
+    items, parts, max_parts = st.plan_attention(lens, 4736, 6144, slots=16)
+    n = parts.numpy()
+    assert n.sum() == 16 and max_parts == n.max()
+    assert (lens / n).max() <= 1.6 * lens.sum() / 16
+    assert ((lens / n) <= 6144).all() and (n >= 1).all()
+    it = items.numpy()
+    assert sorted(map(tuple, it.tolist())) == sorted((b, p) for b in range(5) for p in range(n[b]))
+    # never splits below 256 tokens per partition
+    _, parts, _ = st.plan_attention(np.array([300, 700]), 4736, 6144, slots=64)
+    assert parts.numpy().tolist() == [1, 2]
