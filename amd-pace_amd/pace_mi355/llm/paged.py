@@ -196,6 +196,12 @@ class PagedState:
             self._store_items(key, lens, base, with_parts=False)
         return self._items_dev, None, int(base.max())
 
+    def _upload(self, host: torch.Tensor) -> torch.Tensor:
+        """Asynchronous copy to the device through fresh pinned memory (plain tensor on a CPU state)."""
+        if self.device.type != "cuda":
+            return host
+        return host.pin_memory().to(self.device, non_blocking=True)
+
     def _store_items(self, key, lens: np.ndarray, n_parts: np.ndarray, with_parts: bool) -> None:
         seq = np.repeat(np.arange(lens.size), n_parts)
         first = np.repeat(np.cumsum(n_parts) - n_parts, n_parts)
@@ -203,10 +209,8 @@ class PagedState:
         size = np.repeat(lens / n_parts, n_parts)
         order = np.argsort(-size, kind="stable")
         items = np.stack([seq, part], axis=1)[order].astype(np.int32)
-        self._items_dev = torch.from_numpy(items).pin_memory().to(self.device, non_blocking=True)
-        self._parts_dev = (
-            torch.from_numpy(n_parts.astype(np.int32)).pin_memory().to(self.device, non_blocking=True) if with_parts else None
-        )
+        self._items_dev = self._upload(torch.from_numpy(items))
+        self._parts_dev = self._upload(torch.from_numpy(n_parts.astype(np.int32))) if with_parts else None
         self._max_parts = int(n_parts.max())
         self._items_key = key
 
