@@ -251,7 +251,7 @@ def test_plan_attention_uniform_batch_uses_dense_grid():
 
 def test_plan_attention_multi_round_batch_is_cut_and_sorted_longest_first():
     st = _state(batch=6, max_len=20000, blocks=10)
-    lens = np.array([100, 5000, 16385, 300, 2048, 9000])
+    lens = np.array([100, 5000, 16385, 300, 2000, 9000])
     items, parts, max_parts = st.plan_attention(lens, 2048, 8192, slots=8)  # 8 slots < 18 partitions: several rounds
     assert parts is None and max_parts == 9
     it = items.numpy()
