@@ -57,6 +57,74 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
 }
 
 // ---------------------------------------------------------------------------------
+// Block append (many tokens per sequence: prefill chunks).  One 256-thread workgroup
+// fills one destination block of one (sequence, head): the token rows that land in the
+// block are staged row-major in LDS, then written out in slab order, 16 bytes per lane
+// -- K chunks straight from the rows, V chunks transposed (eight tokens of one dim).
+// Slabs of blocks the append only partly covers are written element-wise for V so that
+// earlier tokens of the block stay untouched.
+// ---------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t pool, const uint16_t* __restrict__ k_new,
+                                                              const uint16_t* __restrict__ v_new, int64_t sb, int64_t sh,
+                                                              int64_t st, int32_t n_tokens, const AppendDest dest,
+                                                              int32_t first_block_hint) {
+  constexpr int CHUNKS = D / 8;
+  constexpr int BT = PACE_KV_BLOCK_TOKENS;
+  __shared__ uint16_t ks[BT * D];
+  __shared__ uint16_t vs[BT * (D + 8)];  // padded rows: column reads hit different banks
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int64_t pos0 = (int64_t)dest.seq_lens[b] + dest.pos_offset;  // position of new token 0
+  if (pos0 < 0) return;
+  // Destination blocks touched by this sequence: pos0/16 .. (pos0+n_tokens-1)/16.
+  const int jb = (int)(pos0 / BT) + blockIdx.x;
+  const int64_t blk_pos0 = (int64_t)jb * BT;
+  const int t_lo = (int)max((int64_t)0, blk_pos0 - pos0);                 // first new token in this block
+  const int t_hi = (int)min((int64_t)n_tokens, blk_pos0 + BT - pos0);     // one past the last
+  if (t_lo >= t_hi || jb >= dest.table_stride) return;  // uniform over the workgroup
+  const int64_t blk = dest.table[(int64_t)b * dest.table_stride + jb];
+  if (blk < 0 || blk >= pool.num_blocks) return;  // never write outside the pool
+  const int off_lo = (int)(pos0 + t_lo - blk_pos0), n_here = t_hi - t_lo;  // slots off_lo .. off_lo+n_here-1
+  const uint16_t* kin = k_new + (int64_t)b * sb + (int64_t)h * sh;
+  const uint16_t* vin = v_new + (int64_t)b * sb + (int64_t)h * sh;
+  for (int c = threadIdx.x; c < n_here * CHUNKS; c += 256) {
+    const int r = c / CHUNKS, ch = c % CHUNKS;
+    const int64_t src = (int64_t)(t_lo + r) * st + ch * 8;
+    *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = *reinterpret_cast<const u32x4*>(kin + src);
+    *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = *reinterpret_cast<const u32x4*>(vin + src);
+  }
+  __syncthreads();
+  uint16_t* kslab = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
+  uint16_t* vslab = reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
+  const bool whole = (n_here == BT);
+  // K: slab chunk c = (tile, dim chunk, slot) holds dims 8*chunk.. of token tok(tile, slot).
+  for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
+    const int tile = c / (CHUNKS * 8), chunk = (c / 8) % CHUNKS, slot = c % 8;
+    const int tok = ((slot >> 2) << 3) | (tile << 2) | (slot & 3);
+    if (tok >= off_lo && tok < off_lo + n_here)
+      *reinterpret_cast<u32x4*>(kslab + c * 8) = *reinterpret_cast<const u32x4*>(&ks[tok * D + chunk * 8]);
+  }
+  // V: slab chunk c = (dim tile, token half, dim) holds tokens 8*half..+7 of one dim.
+  for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
+    const int jt = c / 32, half = (c / 16) % 2, dn = c % 16;
+    const int dim = jt * 16 + dn;
+    if (whole) {
+      u32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w[e] = (uint32_t)vs[(8 * half + 2 * e) * (D + 8) + dim] | ((uint32_t)vs[(8 * half + 2 * e + 1) * (D + 8) + dim] << 16);
+      *reinterpret_cast<u32x4*>(vslab + c * 8) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int tok = 8 * half + e;
+        if (tok >= off_lo && tok < off_lo + n_here) vslab[c * 8 + e] = vs[tok * (D + 8) + dim];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // Gather.  One 256-thread workgroup rebuilds one logical block (16 tokens) of one KV
 // head of one sequence in the dense [B][H*n_rep][L][D] layout.  K chunks are read
 // from their slab position; V slabs are staged in LDS and read back transposed.
@@ -144,6 +212,23 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
   PACE_REQUIRE(aligned16(k_new) && aligned16(v_new), "%s: k_new / v_new must be 16-byte aligned", who);
   PACE_REQUIRE(stride_b % 8 == 0 && stride_h % 8 == 0 && stride_t % 8 == 0,
                "%s: input strides must be multiples of 8 elements", who);
+  hipStream_t s_early = static_cast<hipStream_t>(stream);
+  if (paged && n_tokens >= 8) {
+    // Enough tokens per sequence to fill slabs: one workgroup per destination block.
+    PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
+    const unsigned blocks_x = (unsigned)((n_tokens + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS + 1);
+    dim3 grid(blocks_x, pool->num_kv_heads, batch);
+    const uint16_t* kq = static_cast<const uint16_t*>(k_new);
+    const uint16_t* vq = static_cast<const uint16_t*>(v_new);
+    if (pool->head_dim == 128)
+      hipLaunchKernelGGL(kv_append_block_kernel<128>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
+                         n_tokens, dest, 0);
+    else
+      hipLaunchKernelGGL(kv_append_block_kernel<64>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
+                         n_tokens, dest, 0);
+    PACE_HIP_CHECK(hipGetLastError());
+    return PACE_KV_OK;
+  }
   const int64_t rows = (int64_t)batch * n_tokens * pool->num_kv_heads;
   PACE_REQUIRE(rows < (int64_t)1 << 31, "%s: too many rows (%lld)", who, (long long)rows);
   const int chunks = pool->head_dim / 8;

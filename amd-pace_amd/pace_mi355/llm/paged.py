@@ -63,6 +63,11 @@ class BlockAllocator:
             self._is_free[i] = False
         self._free = [i for i in self._free if i not in want]
 
+    def reset_free(self, is_free: np.ndarray) -> None:
+        """Replace the free list wholesale (lowest ids are handed out first again)."""
+        self._is_free = is_free.copy()
+        self._free = np.nonzero(is_free)[0][::-1].tolist()
+
     def free_ids(self) -> np.ndarray:
         return np.nonzero(self._is_free)[0]
 
@@ -274,11 +279,12 @@ class PagedState:
             return
         remap = np.arange(self.allocator.num_blocks, dtype=np.int32)
         remap[moves[:, 0]] = moves[:, 1]
-        self.allocator.take(moves[:, 1].tolist())
+        live = np.zeros(self.allocator.num_blocks, dtype=bool)
         for b in range(self.batch):
             n = int(self.n_blocks[b])
             self.table[b, :n] = remap[self.table[b, :n]]
-        self.allocator.free(moves[:, 0].tolist())
+            live[self.table[b, :n]] = True
+        self.allocator.reset_free(~live)
         self._table_dirty = True
 
     def live_block_count(self) -> int:
