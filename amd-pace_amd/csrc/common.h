@@ -31,6 +31,10 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 int check_pool(const pace_kv_pool_t* pool, const char* who);
 
+// Dense bf16 attention on the matrix cores (paged_attn.hip); false = shape not handled, nothing launched.
+bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
+                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;

@@ -154,6 +154,15 @@ extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void
                  "pace_attn_dense: mask dims [%d][%d][%d] not broadcastable to [%d][%d][%d]", mB, mN, mS, B, N, S);
   }
   PACE_REQUIRE(B <= 65535 && N <= 65535, "pace_attn_dense: batch / heads exceed grid limits");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // bf16 with head_dim 64 / 128 runs on the matrix cores; everything else (fp32, other head
+  // sizes) takes the general kernel below.
+  if (qkv_dtype == PACE_DTYPE_BF16 &&
+      launch_dense_mfma(q, k, v, out, B, N, S, L, H, mask, mask_dtype == PACE_DTYPE_F32, mB, mN, mS,
+                        1.0f / sqrtf((float)H), s)) {
+    PACE_HIP_CHECK(hipGetLastError());
+    return PACE_KV_OK;
+  }
   DenseParams p;
   p.q = q, p.k = k, p.v = v, p.out = out, p.mask = mask;
   p.B = B, p.N = N, p.S = S, p.L = L, p.H = H;
@@ -162,7 +171,6 @@ extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void
   p.scale = 1.0f / sqrtf((float)H);
   const size_t smem = ((size_t)kRows * H + (size_t)p.TL * (H + 1) + (size_t)kRows * (p.TL + 1) + 3 * kRows) * sizeof(float);
   dim3 grid((S + kRows - 1) / kRows, N, B);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const bool f32 = qkv_dtype == PACE_DTYPE_F32;
   const bool mf32 = mask_dtype == PACE_DTYPE_F32;
   if (f32 && mf32)
