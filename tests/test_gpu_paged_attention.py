@@ -53,7 +53,8 @@ def test_decode_empty_sequence_gives_zero(device):
     assert_attention_close(out[1:], ref[1:], "non-empty row")
 
 
-@pytest.mark.parametrize("S,lens,partition", [(8, [40, 200, 1029], 256), (9, [9, 64], 0), (3, [5, 300], 128), (16, [16, 100], 0)])
+@pytest.mark.parametrize("S,lens,partition", [(8, [40, 200, 1029], 256), (9, [9, 64], 0), (3, [5, 300], 128), (16, [16, 100], 0),
+                                               (40, [40, 333], 0), (130, [130, 700, 257], 256)])
 def test_verify_causal_matches_oracle(device, S, lens, partition):
     """S new tokens already appended; row s reads tokens <= len - S + s (llama.py:292-299)."""
     B, hkv, n_rep, D = len(lens), 2, 4, 128
@@ -164,4 +165,25 @@ def test_pending_append_is_flushed_by_other_operations(device):
     assert cache._pending is None
     K, V = model.dense(2)
     gk, gv = cache.gather()
+    assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
+
+
+def test_chunked_prefill_through_the_paged_path(device):
+    """A prompt fed in chunks: each chunk is appended and attends causally to everything so far
+    (more query rows than one workgroup holds, several row groups per KV head)."""
+    B, hkv, n_rep, D = 2, 2, 4, 128
+    from pace_mi355.llm import PagedKVCache
+    from oracle.paged_ref import RaggedCacheModel
+
+    cache = PagedKVCache(512, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, D)
+    for step, T in enumerate([100, 33, 64, 7]):
+        k, v = seeded_kv(50 + step, B, hkv, T, D)
+        q = seeded_q(60 + step, B, hkv * n_rep, T, D)
+        pk, pv = cache.update_cache(k.to(device), v.to(device), 2)
+        model.append(k, v)
+        out = cache.attend(q.to(device))
+        assert_attention_close(out, model.attention(q, n_rep), f"chunk {step} of {T} tokens")
+    gk, gv = cache.gather()
+    K, V = model.dense(n_rep)
     assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
