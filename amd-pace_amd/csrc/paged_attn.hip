@@ -23,6 +23,7 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "rope.h"
 
 namespace pace_kv {
 
@@ -62,6 +63,9 @@ struct PagedAttnParams {
   int32_t n_new;
   float* part_o;      // [B][Hq][S][max_parts][D]
   float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
+  // Optional rotary embedding (rope.cos == NULL: off): q rows are rotated as they are loaded,
+  // the fused append's new keys before they are used and stored.  rotary_dim == D here.
+  RopeDev rope;
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -97,10 +101,33 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
   for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
 }
 
+// Rotate one head row held in operand order: x[kk] = dims 32*kk + 8g .. +8 of the row (lane
+// quarter g).  Both members of every rotation pair sit in the same lane: dim d pairs with
+// d + D/2 (register kk + KK/2) or, interleaved, with its neighbour inside the 16 bytes.
+template <int D>
+__device__ __forceinline__ void rotate_row_regs(const RopeDev& rope, int row, int g, u32x4 (&x)[D / 32]) {
+  constexpr int KK = D / 32;
+  const int64_t base = (int64_t)row * (D / 2);
+  if (!rope.interleaved) {
+#pragma unroll
+    for (int kk = 0; kk < KK / 2; ++kk) {
+      const int64_t col = base + 32 * kk + 8 * g;
+      rope_rotate_halves(x[kk], x[kk + KK / 2], rope_load8(rope.cos, rope.is_f32, col), rope_load8(rope.sin, rope.is_f32, col));
+    }
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int64_t col = base + 16 * kk + 4 * g;
+      rope_rotate_adjacent(x[kk], rope_load4(rope.cos, rope.is_f32, col), rope_load4(rope.sin, rope.is_f32, col));
+    }
+  }
+}
+
 // The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
 // (token idx of the unit = new token idx; tokens >= n_new are zero and get masked).
-template <int D>
-__device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnParams& p, int b, int kvh, int n_new, int n, int g) {
+template <int D, bool ROPE>
+__device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnParams& p, int b, int kvh, int pos0, int n_new, int n,
+                                              int g) {
   const uint16_t* kb = p.k_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
   const uint16_t* vb = p.v_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
   const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -110,6 +137,7 @@ __device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnPar
 #pragma unroll
     for (int kk = 0; kk < D / 32; ++kk)
       r.k[t][kk] = idx < n_new ? *reinterpret_cast<const u32x4*>(kb + (int64_t)idx * p.n_st + kk * 32 + 8 * g) : zero;
+    if (ROPE && idx < n_new) rotate_row_regs<D>(p.rope, rope_row(p.rope, b, idx, pos0 + idx), g, r.k[t]);
   }
 #pragma unroll
   for (int j = 0; j < D / 16; ++j) {
@@ -124,22 +152,36 @@ __device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnPar
 }
 
 // Write the step's new tokens of (b, kvh) into their pool slots (positions pool_end ..).
-template <int D>
+// With ROPE a lane moves two 8-dim chunks of a token (the two halves of eight rotation
+// pairs) and rotates the key chunks on the way; without, one chunk.
+template <int D, bool ROPE>
 __device__ __forceinline__ void write_new_tokens(const PagedAttnParams& p, int b, int kvh, int pool_end, int n_new, int lane) {
-  constexpr int CH = D / 8;
-  for (int item = lane; item < n_new * CH; item += 64) {
-    const int idx = item / CH, chunk = item % CH;
+  constexpr int PER_ROW = ROPE ? D / 16 : D / 8;
+  for (int item = lane; item < n_new * PER_ROW; item += 64) {
+    const int idx = item / PER_ROW, ci = item % PER_ROW;
     const int pos = pool_end + idx;
     const int jb = pos / PACE_KV_BLOCK_TOKENS;
     if (jb >= p.table_stride) continue;
     const int64_t blk = p.table[(int64_t)b * p.table_stride + jb];
     if (blk < 0 || blk >= p.num_blocks) continue;  // never write outside the pool
-    const int64_t src = (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh + (int64_t)idx * p.n_st + chunk * 8;
-    const u32x4 kv = *reinterpret_cast<const u32x4*>(p.k_new + src);
-    const u32x4 vv = *reinterpret_cast<const u32x4*>(p.v_new + src);
-    store_kv_chunk<D>(const_cast<uint16_t*>(p.kpool) + blk * p.k_bs + (int64_t)kvh * p.k_hs,
-                      const_cast<uint16_t*>(p.vpool) + blk * p.v_bs + (int64_t)kvh * p.v_hs, pos % PACE_KV_BLOCK_TOKENS,
-                      chunk, kv, vv);
+    const int64_t src = (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh + (int64_t)idx * p.n_st;
+    uint16_t* kslab = const_cast<uint16_t*>(p.kpool) + blk * p.k_bs + (int64_t)kvh * p.k_hs;
+    uint16_t* vslab = const_cast<uint16_t*>(p.vpool) + blk * p.v_bs + (int64_t)kvh * p.v_hs;
+    if (ROPE) {
+      int ca, cb;
+      rope_chunk_pair(p.rope, ci, ca, cb);
+      u32x4 ka = *reinterpret_cast<const u32x4*>(p.k_new + src + ca * 8);
+      u32x4 kb = *reinterpret_cast<const u32x4*>(p.k_new + src + cb * 8);
+      const u32x4 va = *reinterpret_cast<const u32x4*>(p.v_new + src + ca * 8);
+      const u32x4 vb = *reinterpret_cast<const u32x4*>(p.v_new + src + cb * 8);
+      rope_rotate_chunks(p.rope, rope_row(p.rope, b, idx, pos), ci, ka, kb);
+      store_kv_chunk<D>(kslab, vslab, pos % PACE_KV_BLOCK_TOKENS, ca, ka, va);
+      store_kv_chunk<D>(kslab, vslab, pos % PACE_KV_BLOCK_TOKENS, cb, kb, vb);
+    } else {
+      const u32x4 kv = *reinterpret_cast<const u32x4*>(p.k_new + src + ci * 8);
+      const u32x4 vv = *reinterpret_cast<const u32x4*>(p.v_new + src + ci * 8);
+      store_kv_chunk<D>(kslab, vslab, pos % PACE_KV_BLOCK_TOKENS, ci, kv, vv);
+    }
   }
 }
 
@@ -292,10 +334,11 @@ struct WaveBlockIds {
 // NW waves per workgroup split the partition's units among themselves and merge their
 // softmax states through LDS.  OCC is the least number of waves that must fit on one SIMD
 // (caps the register budget) and OCC_MAX the most that may share it; latency is hidden by
-// the other resident waves, each wave keeps one unit (16 KiB) in flight.  With FUSED, one more wave per workgroup handles the
-// step's new tokens (attends to them from the caller's buffers and stores them into the
-// pool), so that its dependent round trips overlap with the streaming waves.
-template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED>
+// the other resident waves, each wave keeps one unit (16 KiB) in flight.  With FUSED, one
+// more wave per workgroup handles the step's new tokens (attends to them from the caller's
+// buffers and stores them into the pool), so that its dependent round trips overlap with the
+// streaming waves.  With ROPE, query rows and the new keys are rotated on their way in.
+template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED, bool ROPE>
 __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC_MAX))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
@@ -374,6 +417,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       u32x4 z = {0u, 0u, 0u, 0u};
       qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
     }
+    if (ROPE && valid) rotate_row_regs<D>(p.rope, rope_row(p.rope, b, s, len - S + s), g, qreg[qt]);
 #pragma unroll
     for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -399,8 +443,8 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   UnitRegs<D> buf;
   if (FUSED) {
     if (wave == NW && n_new > 0 && part == n_parts - 1) {
-      load_new_unit<D>(buf, p, b, kvh, n_new, n, g);
-      if (qg == 0) write_new_tokens<D>(p, b, kvh, pool_end, n_new, lane);
+      load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
+      if (qg == 0) write_new_tokens<D, ROPE>(p, b, kvh, pool_end, n_new, lane);
       compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g);
     }
   }
@@ -626,12 +670,14 @@ template <int D, int NQT, int NW, int OCC, int OCC_MAX>
 static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   const bool fused = p.n_new > 0;
   const unsigned blocks = (unsigned)p.total_items;
-#define PACE_GO(M_, F_) \
-  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
-  if (has_mask) {
-    if (fused) PACE_GO(true, true); else PACE_GO(true, false);
+#define PACE_GO(M_, F_, R_) \
+  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+  if (p.rope.cos) {  // never together with an explicit mask (checked by the caller)
+    if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
+  } else if (has_mask) {
+    if (fused) PACE_GO(true, true, false); else PACE_GO(true, false, false);
   } else {
-    if (fused) PACE_GO(false, true); else PACE_GO(false, false);
+    if (fused) PACE_GO(false, true, false); else PACE_GO(false, false, false);
   }
 #undef PACE_GO
 }
@@ -881,6 +927,15 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
                      (a->new_stride_t % 8) == 0,
                  "%s: k_new / v_new must be 16-byte aligned with strides that are multiples of 8 elements", who);
   }
+  RopeDev rope_dev = {};
+  if (a->rope) {
+    if (int rc = make_rope_dev(a->rope, pool->head_dim, false, who, &rope_dev)) return rc;
+    PACE_REQUIRE(rope_dev.rot == pool->head_dim, "%s: rotary_dim %d must equal head_dim %d when rope rides in the attention launch",
+                 who, rope_dev.rot, pool->head_dim);
+    PACE_REQUIRE(a->mask == nullptr, "%s: rope in the attention launch cannot be combined with an explicit mask", who);
+    PACE_REQUIRE(!a->k_new || a->n_new == a->q_len, "%s: with rope, the fused append takes n_new == q_len (got %d, %d)", who,
+                 a->n_new, a->q_len);
+  }
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
   const int tiles = (rows + 15) / 16;
@@ -919,6 +974,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.n_sb = a->new_stride_b, p.n_sh = a->new_stride_h, p.n_st = a->new_stride_t;
   p.n_new = a->k_new ? a->n_new : 0;
   p.n_qgroups = (tiles + sh.nqt - 1) / sh.nqt;
+  p.rope = rope_dev;
 
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",
@@ -23,6 +23,8 @@ EXPORTED_SYMBOLS = (
     "pace_kv_append_paged",
     "pace_kv_gather",
     "pace_kv_copy_blocks",
+    "pace_rope_apply",
+    "pace_rope_append_paged",
     "pace_paged_attn_partition_tokens",
     "pace_paged_attn_workspace_bytes",
     "pace_paged_attn_workspace_bytes_for_parts",
@@ -46,6 +48,21 @@ class PoolDesc(Structure):
         ("num_kv_heads", c_int32),
         ("head_dim", c_int32),
         ("block_size", c_int32),
+    ]
+
+
+class RopeDesc(Structure):
+    """``pace_rope_t``."""
+
+    _fields_ = [
+        ("cos", c_void_p),
+        ("sin", c_void_p),
+        ("table_dtype", c_int32),
+        ("table_rows", c_int32),
+        ("rotary_dim", c_int32),
+        ("interleaved", c_int32),
+        ("positions", c_void_p),
+        ("pos_stride_b", c_int32),
     ]
 
 
@@ -90,6 +107,7 @@ class PagedAttnArgs(Structure):
         ("seq_parts", c_void_p),
         ("max_parts", c_int32),
         ("seq_len_bias", c_int32),
+        ("rope", POINTER(RopeDesc)),
     ]
 
 
@@ -133,6 +151,15 @@ def load() -> ctypes.CDLL:
     ]
     lib.pace_kv_copy_blocks.restype = ctypes.c_int
     lib.pace_kv_copy_blocks.argtypes = [P, P, c_void_p, c_int32, c_void_p]
+    R = POINTER(RopeDesc)
+    rows = [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32]  # in, out, strides b/h/t, heads
+    lib.pace_rope_apply.restype = ctypes.c_int
+    lib.pace_rope_apply.argtypes = [R] + rows + rows + [c_int32, c_int32, c_int32, c_void_p]
+    lib.pace_rope_append_paged.restype = ctypes.c_int
+    lib.pace_rope_append_paged.argtypes = (
+        [P, R] + rows + [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32]
+        + [c_void_p, c_int32, c_void_p, c_int32, c_void_p]
+    )
     lib.pace_paged_attn_partition_tokens.restype = c_int32
     lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 6
     lib.pace_paged_attn_workspace_bytes.restype = c_size_t

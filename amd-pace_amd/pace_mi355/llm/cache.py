@@ -148,7 +148,8 @@ class PagedKVCache(KVCacheBase):
         # reads them from the caller's tensors and stores them into the pool in the same launch;
         # anything else that needs the pool or the lengths first flushes them with a plain append.
         self.fuse_append = True
-        self._pending: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None
+        self._pending: Optional[Tuple[torch.Tensor, torch.Tensor, int, object]] = None
+        self._query_rope = None
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
     # -- set-up -----------------------------------------------------------------
@@ -200,12 +201,19 @@ class PagedKVCache(KVCacheBase):
         )
 
     # -- reference interface ----------------------------------------------------
-    def update_cache(self, key_states: torch.Tensor, value_states: torch.Tensor, concat_dim: int):
-        """Append ``T`` tokens to every sequence (reference ``cache.py:268-326``)."""
+    def update_cache(self, key_states: torch.Tensor, value_states: torch.Tensor, concat_dim: int, rope=None):
+        """Append ``T`` tokens to every sequence (reference ``cache.py:268-326``).
+
+        ``rope`` (what ``RotaryEmbedding.forward`` returned for this step) hands over the
+        *un-rotated* keys: they are rotated on their way into the pool, and the attention
+        call that follows rotates its *un-rotated* queries the same way -- the
+        rope / repeat_kv / update_cache / attention sequence of
+        ``pace/llm/models/llama.py:147-165`` as one launch for steps of up to 32 tokens.
+        """
         self._pin_concat_dim(concat_dim)
         PACE_LLM_ASSERT(key_states.dim() == 4 and concat_dim == 2, "PagedKVCache expects [B, H, T, D] with concat_dim=2")
         self._lazy_init(key_states)
-        self._append(key_states, value_states, None)
+        self._append(key_states, value_states, None, rope)
         return self.key, self.value
 
     def remove_cache(self, remove_len: int) -> None:
@@ -231,8 +239,10 @@ class PagedKVCache(KVCacheBase):
         self._append(key_states, value_states, np.asarray(counts, dtype=np.int64))
         return self.key, self.value
 
-    def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray]) -> None:
+    def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray], rope=None) -> None:
         B, h_in, T, D = k.shape
+        if rope is not None and (counts is not None or tuple(rope.rows.shape) != (B, T)):
+            raise RuntimeError("rope rows must be [B, T] and cannot be combined with per-sequence counts")
         if B != self.batch or D != self.head_dim or h_in % self.num_kv_heads:
             raise RuntimeError(f"update of shape {tuple(k.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={D}]")
         if v.shape != k.shape:
@@ -249,9 +259,10 @@ class PagedKVCache(KVCacheBase):
             if self.seq_len + T > st.min_capacity:
                 st.ensure_capacity(new_lens)
             if self.fuse_append and T <= 32:
-                self._pending = (k, v, head_step)
+                self._pending = (k, v, head_step, rope)
             else:
-                self._launch_append(k, v, head_step, new_lens)
+                self._launch_append(k, v, head_step, new_lens, rope)
+            self._query_rope = rope  # the next attention call rotates its queries with it
         else:
             if (counts < 0).any() or (counts > T).any():
                 raise ValueError("counts must lie in [0, T]")
@@ -269,10 +280,20 @@ class PagedKVCache(KVCacheBase):
         if self.key is None:
             self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
 
-    def _launch_append(self, k: torch.Tensor, v: torch.Tensor, head_step: int, lens_after: np.ndarray) -> None:
+    def _launch_append(self, k: torch.Tensor, v: torch.Tensor, head_step: int, lens_after: np.ndarray, rope=None) -> None:
         st = self.state
         T = k.shape[2]
         (lens_dev, bias), table = st.device_lens(lens_after), st.device_table()
+        if rope is not None:
+            desc = rope.desc()
+            nat.check(
+                nat.load().pace_rope_append_paged(
+                    ctypes.byref(self._desc), ctypes.byref(desc), None, None, 0, 0, 0, 0,
+                    k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
+                    self.batch, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias - T, nat.current_stream_ptr(),
+                )
+            )
+            return
         nat.check(
             nat.load().pace_kv_append_paged(
                 ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
@@ -283,9 +304,9 @@ class PagedKVCache(KVCacheBase):
     def _flush(self) -> None:
         """Store a held-back append into the pool now."""
         if self._pending is not None:
-            k, v, head_step = self._pending
+            k, v, head_step, rope = self._pending
             self._pending = None
-            self._launch_append(k, v, head_step, self.lens)
+            self._launch_append(k, v, head_step, self.lens, rope)
 
     def truncate(self, remove: Sequence[int]) -> None:
         """Per-sequence rollback: forget the last ``remove[b]`` tokens of sequence ``b``
@@ -396,6 +417,17 @@ class PagedKVCache(KVCacheBase):
             raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.head_dim}]")
         if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
             query = query.contiguous()
+        rope, self._query_rope = self._query_rope, None
+        rope_desc = None
+        if rope is not None:
+            if tuple(rope.rows.shape) != (B, S):
+                raise RuntimeError(f"rope rows {tuple(rope.rows.shape)} do not match the query [B={B}, S={S}]")
+            rope_desc = rope.desc()
+            if attention_mask is not None or rope_desc.rotary_dim != D:
+                # cases the attention launch does not fold in: rotate the queries (and a held-back append) first
+                self._flush()
+                query, _ = rope(query, None)
+                rope_desc = None
         out = torch.empty((B, hq, S, D), dtype=torch.bfloat16, device=query.device)
         st = self.state
         max_len = self.seq_len
@@ -453,8 +485,12 @@ class PagedKVCache(KVCacheBase):
         a.scale = 1.0 / math.sqrt(D)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes
+        if rope_desc is not None:
+            a.rope = ctypes.pointer(rope_desc)
         if self._pending is not None:
-            k, v, head_step = self._pending
+            k, v, head_step, k_rope = self._pending
+            if (k_rope is None) != (rope_desc is None) or k.shape[2] != S and rope_desc is not None:
+                raise RuntimeError("a held-back append and the attention call disagree about the rotary embedding")
             self._pending = None  # this launch stores them into the pool
             a.k_new, a.v_new, a.n_new = k.data_ptr(), v.data_ptr(), k.shape[2]
             a.new_stride_b, a.new_stride_h, a.new_stride_t = k.stride(0), k.stride(1) * head_step, k.stride(2)

@@ -1,0 +1,249 @@
+"""Rotary position embedding operator with the reference's interface
+(``pace/ops/rotary_embedding.py:202-481``), executed by the gfx950 library.
+
+The constructor builds the same ``cos_cache`` / ``sin_cache`` buffers
+(rows = positions, columns = rotary_dim / 2 frequencies) for the reference's five
+scaling kinds.  ``forward`` returns a callable, as the reference does, but one that
+keeps the *table rows* of the tokens instead of gathered cos / sin tensors, so the
+rotation can run
+
+  * on dense tensors            -- ``rope(query=q, key=k)``            -> ``pace_rope_apply``
+  * folded into the cache append -- ``cache.update_cache(k, v, 2, rope=rope)``
+                                                                     -> ``pace_rope_append_paged``
+  * folded into the attention launch together with the append (decode / verify steps).
+
+bf16 device tensors with head_dim 64 or 128 only; anything else raises (there is
+no second implementation).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Any, Callable, Dict, Optional, Tuple, Union
+
+import torch
+
+from .. import _native as nat
+from ..utils.logging import PACE_ASSERT
+from .base import OperatorBase
+from .enum import BackendType, OperatorType
+
+
+def _frequencies(base: float, rotary_dim: int, rescale=None) -> torch.Tensor:
+    expo = torch.arange(0, rotary_dim, 2, dtype=torch.float) / rotary_dim
+    scale = torch.tensor(rescale, dtype=torch.float32) if rescale else 1
+    return 1.0 / (scale * (base ** expo))
+
+
+def _table(freq: torch.Tensor, rows, amplitude: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    angles = torch.einsum("i,j -> ij", torch.arange(rows, dtype=torch.float), freq)
+    return angles.cos() * amplitude, angles.sin() * amplitude
+
+
+def _default_tables(cfg, dim, rows, theta, **_):
+    return _table(_frequencies(theta, dim), rows)
+
+
+def _linear_tables(cfg, dim, rows, theta, **_):
+    # the factor multiplies cos / sin themselves, as in the reference (:119-130)
+    return _table(_frequencies(theta, dim), rows, cfg["scaling_factor"])
+
+
+def _dynamic_tables(cfg, dim, rows, theta, **_):
+    s = cfg["scaling_factor"]
+    longest = rows * s
+    theta = theta * ((s * longest / rows) - (s - 1)) ** (dim / (dim - 2))
+    return _table(_frequencies(theta, dim), longest)
+
+
+def _llama3_tables(cfg, dim, rows, theta, **_):
+    f = _frequencies(theta, dim)
+    factor, low, high = cfg["factor"], cfg["low_freq_factor"], cfg["high_freq_factor"]
+    orig = cfg["original_max_position_embeddings"]
+    wavelen = 2 * math.pi / f
+    smooth = (orig / wavelen - low) / (high - low) if low != high else 0
+    f = torch.where(
+        wavelen < orig / high,
+        f,
+        torch.where(wavelen > orig / low, f / factor, (1 - smooth) * f / factor + smooth * f),
+    )
+    return _table(f, rows)
+
+
+_TABLE_BUILDERS: Dict[str, Callable] = {
+    "default": _default_tables,
+    "linear": _linear_tables,
+    "dynamic": _dynamic_tables,
+    "llama3": _llama3_tables,
+}
+
+
+def _check_rows(x: torch.Tensor, name: str) -> None:
+    if not x.is_cuda or x.dtype != torch.bfloat16 or x.dim() != 4:
+        raise NotImplementedError(f"rotary embedding runs on bf16 device tensors [B, H, S, D]; {name} is "
+                                  f"{x.dtype} {tuple(x.shape)} on {x.device}")
+    if x.shape[-1] not in (64, 128):
+        raise NotImplementedError(f"rotary embedding supports head_dim 64 or 128, got {x.shape[-1]}")
+
+
+def _strided(x: torch.Tensor) -> torch.Tensor:
+    ok = x.stride(3) == 1 and x.data_ptr() % 16 == 0 and all(
+        s % 8 == 0 and (s > 0 or n == 1) for s, n in zip(x.stride()[:3], x.shape[:3]))
+    return x if ok else x.contiguous()
+
+
+def launch_rope_apply(desc: nat.RopeDesc, query: Optional[torch.Tensor], key: Optional[torch.Tensor]):
+    """Rotate dense ``query`` / ``key`` [B, H, S, D] into new tensors with ``pace_rope_apply``."""
+    outs = []
+    args = []
+    ref = query if query is not None else key
+    B, _, S, D = ref.shape
+    for x, name in ((query, "query"), (key, "key")):
+        if x is None:
+            outs.append(None)
+            args += [None, None, 0, 0, 0, 0]
+            continue
+        _check_rows(x, name)
+        if x.shape[0] != B or x.shape[2] != S or x.shape[3] != D:
+            raise RuntimeError(f"query / key disagree: {tuple(query.shape)} vs {tuple(key.shape)}")
+        xin = _strided(x)
+        out = torch.empty_strided(xin.shape, xin.stride(), dtype=xin.dtype, device=xin.device) if xin is x else xin
+        outs.append(out)
+        args += [xin.data_ptr(), out.data_ptr(), xin.stride(0), xin.stride(1), xin.stride(2), xin.shape[1]]
+    nat.check(nat.load().pace_rope_apply(ctypes.byref(desc), *args, B, S, D, nat.current_stream_ptr()))
+    return outs[0], outs[1]
+
+
+class RopeCall:
+    """What ``RotaryEmbedding.forward`` returns: the rotation of one model step.
+
+    Callable like the reference's ``partial(apply_rotary_emb, cos=..., sin=...)``:
+    ``rope(query=q, key=k)`` or ``rope(q, k, is_neox_style=False)``.  The cache and
+    the attention backend take the object itself to fold the rotation into their launches.
+    """
+
+    def __init__(self, module: "RotaryEmbedding", rows: torch.Tensor):
+        self.module = module
+        self.rows = rows  # int32 [B, S] table rows, on the device
+        self.is_neox_style = True
+
+    def desc(self, is_neox_style: Optional[bool] = None) -> nat.RopeDesc:
+        neox = self.is_neox_style if is_neox_style is None else is_neox_style
+        cos, sin = self.module.device_tables(self.rows.device)
+        d = nat.RopeDesc()
+        d.cos, d.sin = cos.data_ptr(), sin.data_ptr()
+        d.table_dtype = nat.DTYPE_BF16
+        d.table_rows, d.rotary_dim = cos.shape[0], 2 * cos.shape[1]
+        d.interleaved = 0 if neox else 1
+        d.positions, d.pos_stride_b = self.rows.data_ptr(), self.rows.stride(0)
+        return d
+
+    def with_style(self, is_neox_style: bool) -> "RopeCall":
+        other = RopeCall(self.module, self.rows)
+        other.is_neox_style = bool(is_neox_style)
+        return other
+
+    def __call__(self, query: torch.Tensor, key: torch.Tensor, is_neox_style: Optional[bool] = None):
+        return launch_rope_apply(self.desc(is_neox_style), query, key)
+
+
+class RotaryEmbedding(OperatorBase):
+    """Reference signature (``pace/ops/rotary_embedding.py:257-268``)."""
+
+    @property
+    def operator_type(self) -> OperatorType:
+        return OperatorType.ROTARYEMBEDDING
+
+    def __init__(
+        self,
+        rope_scaling: Optional[Dict[str, Any]],
+        rotary_dim: int,
+        max_position_embeddings: int,
+        rope_theta: Union[int, float],
+        partial_rotary_factor: float = 1.0,
+        dtype: Optional[torch.dtype] = None,
+        backend_impl: Optional[BackendType] = None,  # unused, as in the reference
+        **rope_kwargs,
+    ):
+        super().__init__(backend_impl=backend_impl, dtype=dtype)
+        if partial_rotary_factor < 1.0:
+            rotary_dim = int(rotary_dim * partial_rotary_factor)
+        self.rotary_dim = rotary_dim
+        self.partial_rotary_factor = partial_rotary_factor
+        self.rope_kwargs = rope_kwargs
+        self.rope_scaling = rope_scaling
+        self.rope_type = "default" if rope_scaling is None else rope_scaling.get("rope_type", rope_scaling.get("type"))
+        self.max_position_embeddings = max_position_embeddings
+        self.rope_theta = rope_theta
+        if self.rope_type == "longrope":
+            cos, sin = self._longrope_tables()
+        else:
+            PACE_ASSERT(self.rope_type in _TABLE_BUILDERS, f"Unsupported RoPE type: {self.rope_type}")
+            cos, sin = _TABLE_BUILDERS[self.rope_type](rope_scaling, rotary_dim, max_position_embeddings, rope_theta)
+        self.register_buffer("cos_cache", cos, persistent=False)
+        self.register_buffer("sin_cache", sin, persistent=False)
+        self._device_tables: Dict[Any, Tuple[torch.Tensor, torch.Tensor]] = {}
+
+    def _longrope_tables(self):
+        cfg, rows = self.rope_scaling, self.max_position_embeddings
+        orig = self.rope_kwargs.get("original_max_position_embeddings", rows)
+        self.original_max_position_embeddings = orig
+        ratio = rows / orig
+        amp = 1.0 if ratio <= 1.0 else math.sqrt(1 + math.log(ratio) / math.log(orig))
+        if cfg.get("attention_factor") is not None:
+            amp = cfg["attention_factor"]
+        short = _table(_frequencies(self.rope_theta, self.rotary_dim, cfg["short_factor"]), orig, amp)
+        long_ = _table(_frequencies(self.rope_theta, self.rotary_dim, cfg["long_factor"]), rows, amp)
+        return torch.cat([short[0], long_[0]], dim=0), torch.cat([short[1], long_[1]], dim=0)
+
+    def device_tables(self, device) -> Tuple[torch.Tensor, torch.Tensor]:
+        """bf16 copies of the tables on ``device`` (what ``.to(x.dtype)`` yields for bf16 activations)."""
+        key = str(device)
+        if key not in self._device_tables:
+            self._device_tables[key] = (
+                self.cos_cache.to(device=device, dtype=torch.bfloat16).contiguous(),
+                self.sin_cache.to(device=device, dtype=torch.bfloat16).contiguous(),
+            )
+        return self._device_tables[key]
+
+    def table_rows(self, position_ids: torch.Tensor, offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Rows of the tables the tokens read (reference ``forward``, ``:381-394``)."""
+        if self.rope_type == "longrope":
+            k = self.original_max_position_embeddings
+            shift = (torch.any(position_ids > k).float() * torch.full_like(position_ids, k)).long()
+            idx = position_ids + shift
+            return idx + offsets if offsets is not None else idx
+        return position_ids
+
+    def forward(self, x: torch.Tensor, position_ids: torch.Tensor, return_cos_sin: bool = False,
+                offsets: Optional[torch.Tensor] = None):
+        rows = self.table_rows(position_ids, offsets)
+        if return_cos_sin:
+            flat = rows.flatten()
+            cos = self.cos_cache.index_select(0, flat).unflatten(0, rows.shape).to(x.dtype)
+            sin = self.sin_cache.index_select(0, flat).unflatten(0, rows.shape).to(x.dtype)
+            return cos, sin
+        if not x.is_cuda:
+            raise NotImplementedError("rotary embedding runs on the GPU; activations are on " + str(x.device))
+        return RopeCall(self, rows.to(device=x.device, dtype=torch.int32).contiguous())
+
+    def apply_rotary_emb(self, query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                         unsqueeze_dim: int = 1, is_neox_style: bool = True):
+        """Rotate with gathered ``cos`` / ``sin`` [B, S, rotary_dim/2] (reference ``:445-474``)."""
+        if unsqueeze_dim != 1:
+            raise NotImplementedError("rotary embedding takes [B, H, S, D] tensors (unsqueeze_dim=1)")
+        _check_rows(query, "query")
+        B, S = cos.shape[0], cos.shape[1]
+        cos2 = cos.to(torch.bfloat16).reshape(B * S, -1).contiguous()
+        sin2 = sin.to(torch.bfloat16).reshape(B * S, -1).contiguous()
+        rows = torch.arange(B * S, dtype=torch.int32, device=query.device).view(B, S)
+        d = nat.RopeDesc()
+        d.cos, d.sin, d.table_dtype = cos2.data_ptr(), sin2.data_ptr(), nat.DTYPE_BF16
+        d.table_rows, d.rotary_dim = B * S, 2 * cos2.shape[1]
+        d.interleaved = 0 if is_neox_style else 1
+        d.positions, d.pos_stride_b = rows.data_ptr(), rows.stride(0)
+        return launch_rope_apply(d, query, key)
+
+    def extra_repr(self) -> str:
+        return (f"rope_type={self.rope_type}, rotary_dim={self.rotary_dim}, "
+                f"max_position_embeddings={self.max_position_embeddings}, rope_theta={self.rope_theta}")

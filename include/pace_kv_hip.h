@@ -15,6 +15,7 @@
  *   - KVCacheBase.remove_cache          pace/llm/cache.py:224-240, 352-368 (host metadata only)
  *   - update_cache_with_beam_indices    pace/llm/cache.py:161-167
  *   - repeat_kv (folded into the kernels) pace/llm/models/llama.py:50-61
+ *   - RotaryEmbedding.apply_rotary_emb   pace/ops/rotary_embedding.py:412-474 (the step before the append)
  *
  * Storage: a block pool.  Block size is 16 tokens.  One (block, KV head) slab
  * holds 16 tokens x head_dim values in an order private to the library (see
@@ -118,6 +119,58 @@ int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32
 int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst,
                         const int32_t* pairs, int32_t n_pairs, void* stream);
 
+/*
+ * Rotary position embedding, the step the models run on q and k right before the
+ * append (pace/llm/models/llama.py:147-158; operator pace/ops/rotary_embedding.py:370-474).
+ * cos / sin: device tables [table_rows][rotary_dim/2] as RotaryEmbedding builds them
+ * (cos_cache / sin_cache, pace/ops/rotary_embedding.py:366-367), bf16 or fp32; fp32 entries
+ * are rounded to bf16 on load, which is what forward()'s `.to(x.dtype)` does (:399-400).
+ * Token t of sequence b uses table row positions[b*pos_stride_b + t]; with positions == NULL
+ * the row is the token's position in its sequence.  Rows outside the table are clamped.
+ * The first rotary_dim dims of every head row are rotated, the rest pass through
+ * (:421-430; pace/llm/models/gptj.py:115-131).  Results are bit-identical to the reference's
+ * bf16 tensor arithmetic (each product and the sum rounded separately).
+ */
+typedef struct pace_rope {
+  const void* cos;
+  const void* sin;
+  int32_t table_dtype;   /* PACE_DTYPE_BF16 / PACE_DTYPE_F32                              */
+  int32_t table_rows;
+  int32_t rotary_dim;    /* multiple of 16, <= head_dim                                   */
+  int32_t interleaved;   /* 0: neox style, dim i pairs with i + rotary_dim/2 (is_neox_style=True);
+                            1: GPT-J style, dim 2i pairs with 2i+1                         */
+  const int32_t* positions; /* optional device int32 [batch][tokens]                      */
+  int32_t pos_stride_b;
+} pace_rope_t;
+
+/*
+ * RotaryEmbedding.apply_rotary_emb on dense tensors (pace/ops/rotary_embedding.py:445-474):
+ * q [batch][num_q_heads][n_tokens][head_dim] and k [batch][num_k_heads][n_tokens][head_dim],
+ * bf16, element strides given (innermost contiguous), rotated into q_out / k_out (same
+ * strides; may alias the inputs).  Either tensor may be NULL.  rope->positions is required.
+ */
+int pace_rope_apply(const pace_rope_t* rope, const void* q, void* q_out,
+                    int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t, int32_t num_q_heads,
+                    const void* k, void* k_out,
+                    int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_t, int32_t num_k_heads,
+                    int32_t batch, int32_t n_tokens, int32_t head_dim, void* stream);
+
+/*
+ * Rotate-and-append in one launch: the rope(q, k) + update_cache(k, v) sequence of
+ * pace/llm/models/llama.py:147-158.  q is rotated into q_out (may alias q; NULL q = keys
+ * only); k_new is rotated and stored, v_new stored, at positions seq_lens[b] + pos_offset + t
+ * through the block table exactly as pace_kv_append_paged does.  With rope->positions == NULL
+ * the same position selects the table row.  k_new / v_new are not modified.
+ */
+int pace_rope_append_paged(const pace_kv_pool_t* pool, const pace_rope_t* rope,
+                           const void* q, void* q_out,
+                           int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t, int32_t num_q_heads,
+                           const void* k_new, const void* v_new,
+                           int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                           int32_t batch, int32_t n_tokens,
+                           const int32_t* block_table, int32_t table_stride,
+                           const int32_t* seq_lens, int32_t pos_offset, void* stream);
+
 typedef struct pace_paged_attn_args {
   const void* q;          /* bf16 [batch][num_q_heads][q_len][head_dim]               */
   int64_t q_stride_b, q_stride_h, q_stride_s; /* elements; innermost contiguous      */
@@ -165,6 +218,13 @@ typedef struct pace_paged_attn_args {
   int32_t max_parts;
   int32_t seq_len_bias;       /* host-side constant added to every seq_lens entry, so that uniform
                                  appends / rollbacks need no device update of the lengths */
+  /* Optional rotary embedding folded into the launch (NULL = off; needs rotary_dim == head_dim).
+   * q holds the un-rotated queries: each row is rotated as it is loaded.  With the fused append,
+   * k_new holds the un-rotated keys: they are rotated before they are attended to and stored
+   * (n_new must equal q_len).  Positions: rope->positions [batch][q_len], or NULL for
+   * seq_len - q_len + s.  One launch then covers rope + append + attention of
+   * pace/llm/models/llama.py:147-165. */
+  const pace_rope_t* rope;
 } pace_paged_attn_args_t;
 
 /* The context split size (tokens per workgroup) the library uses for these sizes when

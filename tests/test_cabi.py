@@ -56,6 +56,7 @@ def test_struct_layouts_match_the_header():
 
     assert fields("pace_kv_pool") == [f[0] for f in _native.PoolDesc._fields_]
     assert fields("pace_paged_attn_args") == [f[0] for f in _native.PagedAttnArgs._fields_]
+    assert fields("pace_rope") == [f[0] for f in _native.RopeDesc._fields_]
     assert ctypes.sizeof(_native.PoolDesc) == 64
 
 
@@ -76,6 +77,16 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.pace_attn_dense(16, 16, 16, 16, 1, 1, 1, 1, 1, 300, None, 0, 1, 1, 1, None) == -1
     assert b"head_dim 300 unsupported" in lib.pace_kv_last_error()
     assert lib.pace_paged_attn_workspace_bytes(0, 32, 1, 128, 4096, 0, 8) == 0
+    rope = _native.RopeDesc(cos=16, sin=32, table_dtype=1, table_rows=8, rotary_dim=24, interleaved=0, positions=16,
+                            pos_stride_b=1)
+    rows = (16, 16, 8, 8, 8, 1)
+    assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 64, None) == -1
+    assert b"rotary_dim 24 must be a multiple of 16" in lib.pace_kv_last_error()
+    rope.rotary_dim, rope.positions = 64, None
+    assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 64, None) == -1
+    assert b"positions are required" in lib.pace_kv_last_error()
+    assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 96, None) == -1
+    assert b"head_dim 96 unsupported" in lib.pace_kv_last_error()
 
 
 def test_torch_op_is_defined_with_reference_schema_and_checks():
