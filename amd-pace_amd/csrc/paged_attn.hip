@@ -104,23 +104,46 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
 // Rotate one head row held in operand order: x[kk] = dims 32*kk + 8g .. +8 of the row (lane
 // quarter g).  Both members of every rotation pair sit in the same lane: dim d pairs with
 // d + D/2 (register kk + KK/2) or, interleaved, with its neighbour inside the 16 bytes.
+// Split in two so that the table loads can be issued early and consumed late.
 template <int D>
-__device__ __forceinline__ void rotate_row_regs(const RopeDev& rope, int row, int g, u32x4 (&x)[D / 32]) {
+__device__ __forceinline__ void rope_fetch_row(const RopeDev& rope, int row, int g, u32x4 (&tab)[D / 32]) {
   constexpr int KK = D / 32;
   const int64_t base = (int64_t)row * (D / 2);
   if (!rope.interleaved) {
 #pragma unroll
     for (int kk = 0; kk < KK / 2; ++kk) {
       const int64_t col = base + 32 * kk + 8 * g;
-      rope_rotate_halves(x[kk], x[kk + KK / 2], rope_load8(rope.cos, rope.is_f32, col), rope_load8(rope.sin, rope.is_f32, col));
+      tab[2 * kk] = rope_load8(rope.cos, rope.is_f32, col);
+      tab[2 * kk + 1] = rope_load8(rope.sin, rope.is_f32, col);
     }
   } else {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       const int64_t col = base + 16 * kk + 4 * g;
-      rope_rotate_adjacent(x[kk], rope_load4(rope.cos, rope.is_f32, col), rope_load4(rope.sin, rope.is_f32, col));
+      const u32x2 c4 = rope_load4(rope.cos, rope.is_f32, col), s4 = rope_load4(rope.sin, rope.is_f32, col);
+      tab[kk] = u32x4{c4[0], c4[1], s4[0], s4[1]};
     }
   }
+}
+
+template <int D>
+__device__ __forceinline__ void rope_apply_row(const RopeDev& rope, const u32x4 (&tab)[D / 32], u32x4 (&x)[D / 32]) {
+  constexpr int KK = D / 32;
+  if (!rope.interleaved) {
+#pragma unroll
+    for (int kk = 0; kk < KK / 2; ++kk) rope_rotate_halves(x[kk], x[kk + KK / 2], tab[2 * kk], tab[2 * kk + 1]);
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+      rope_rotate_adjacent(x[kk], u32x2{tab[kk][0], tab[kk][1]}, u32x2{tab[kk][2], tab[kk][3]});
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void rotate_row_regs(const RopeDev& rope, int row, int g, u32x4 (&x)[D / 32]) {
+  u32x4 tab[D / 32];
+  rope_fetch_row<D>(rope, row, g, tab);
+  rope_apply_row<D>(rope, tab, x);
 }
 
 // The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
@@ -354,20 +377,21 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   const long long pt0 = wall_clock64();
 #endif
   // Linear work index -> (KV head, row group, sequence, partition); KV head fastest.
-  const long long L = blockIdx.x;
-  const bool active_item = L < p.total_items;
+  // (32-bit arithmetic: the host keeps total_items below 2^31.)
+  const uint32_t L = blockIdx.x;
+  const bool active_item = L < (uint32_t)p.total_items;
   int kvh = 0, part = 0, b = 0, qg = 0;
   if (active_item) {
-    kvh = (int)(L % p.num_kv_heads);
-    const long long rest = L / p.num_kv_heads;
+    kvh = (int)(L % (uint32_t)p.num_kv_heads);
+    const uint32_t rest = L / (uint32_t)p.num_kv_heads;
     if (p.items) {  // compact work list: no empty entries, longest partitions first
-      qg = (int)(rest % p.n_qgroups);
-      const long long item = rest / p.n_qgroups;
-      b = p.items[2 * item], part = p.items[2 * item + 1];
+      qg = (int)(rest % (uint32_t)p.n_qgroups);
+      const uint32_t item = rest / (uint32_t)p.n_qgroups;
+      b = p.items[2 * (int64_t)item], part = p.items[2 * (int64_t)item + 1];
     } else {
-      part = (int)(rest % p.max_parts);
-      const long long bz = rest / p.max_parts;
-      b = (int)(bz / p.n_qgroups), qg = (int)(bz % p.n_qgroups);
+      part = (int)(rest % (uint32_t)p.max_parts);
+      const uint32_t bz = rest / (uint32_t)p.max_parts;
+      b = (int)(bz / (uint32_t)p.n_qgroups), qg = (int)(bz % (uint32_t)p.n_qgroups);
     }
   }
   const int len_b = p.seq_lens[b] + p.len_bias;
@@ -395,9 +419,21 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
 
   // Query rows of this wave (B operand of the first product) and per-row limits.
   u32x4 qreg[NQT][KK];
+  u32x4 qtab[ROPE ? NQT : 1][KK];  // cos / sin of the rows: fetched here, applied once the first unit is on its way
   RowState<D, NQT> st;
   int row_s[NQT], row_h[NQT];
   int min_limit = 0x7fffffff;
+  // Table rows first: a position id that has to be loaded is waited for before any other load
+  // of the wave is in flight.
+  int tab_row[ROPE ? NQT : 1];
+  if (ROPE) {
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      const int r = (qg * NQT + qt) * 16 + n;
+      const int s = r < R ? r / p.n_rep : 0;
+      tab_row[qt] = rope_row(p.rope, b, s, len - S + s);
+    }
+  }
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     const int r = (qg * NQT + qt) * 16 + n;
@@ -417,7 +453,14 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       u32x4 z = {0u, 0u, 0u, 0u};
       qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
     }
-    if (ROPE && valid) rotate_row_regs<D>(p.rope, rope_row(p.rope, b, s, len - S + s), g, qreg[qt]);
+    if (ROPE) {
+      if (valid) {
+        rope_fetch_row<D>(p.rope, tab_row[qt], g, qtab[qt]);
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
 #pragma unroll
     for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -441,6 +484,20 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   }
 
   UnitRegs<D> buf;
+  if (ROPE) {
+    // Put the first unit's loads in flight, then rotate the query rows while they travel.  The
+    // rotation is written out in both arms: after a join the wait for the (older) table loads
+    // would have to assume the worst and cover the unit's loads as well.
+    if (n_units > 0) {
+      load_unit<D>(buf, p, kvh, ids.get(0), ids.get(1), n, g);
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);  // padding rows stay zero
+      asm volatile("; query rows rotated, first unit in flight");  // keeps the two arms from being merged
+    } else {
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
+    }
+  }
   if (FUSED) {
     if (wave == NW && n_new > 0 && part == n_parts - 1) {
       load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
@@ -452,7 +509,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   const long long pt1 = wall_clock64();
 #endif
   for (int uu = 0; uu < n_units; ++uu) {
-    load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
+    if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const int t0 = tok_begin + 32 * uu;
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g);

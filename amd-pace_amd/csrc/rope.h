@@ -24,16 +24,19 @@ struct RopeDev {
   int32_t pos_sb;
 };
 
-__device__ __forceinline__ float rope_rnd(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
-
-// One pair (x1, x2) of bf16 bit patterns rotated by (c, s), all bf16 bit patterns.
-__device__ __forceinline__ void rope_pair(uint32_t x1, uint32_t x2, uint32_t c, uint32_t s, uint32_t& o1, uint32_t& o2) {
-  const float a = bf16_bits_to_f32(x1), b = bf16_bits_to_f32(x2);
-  const float cf = bf16_bits_to_f32(c), sf = bf16_bits_to_f32(s);
-  const float t1 = rope_rnd(a * cf), t2 = rope_rnd(b * sf);
-  const float t3 = rope_rnd(b * cf), t4 = rope_rnd(a * sf);
-  o1 = f32_to_bf16_bits(t1 - t2);
-  o2 = f32_to_bf16_bits(t3 + t4);
+// Two pairs at once -- the low and the high bf16 of the packed words x1, x2 rotated by the low
+// and high bf16 of c, s -- so that every rounding is one packed conversion.
+__device__ __forceinline__ void rope_pair2(uint32_t x1, uint32_t x2, uint32_t c, uint32_t s, uint32_t& o1, uint32_t& o2) {
+  const float a0 = bf16_bits_to_f32(x1 & 0xffffu), a1 = __uint_as_float(x1 & 0xffff0000u);
+  const float b0 = bf16_bits_to_f32(x2 & 0xffffu), b1 = __uint_as_float(x2 & 0xffff0000u);
+  const float c0 = bf16_bits_to_f32(c & 0xffffu), c1 = __uint_as_float(c & 0xffff0000u);
+  const float s0 = bf16_bits_to_f32(s & 0xffffu), s1 = __uint_as_float(s & 0xffff0000u);
+  const uint32_t ac = pack_bf16x2(a0 * c0, a1 * c1), bs = pack_bf16x2(b0 * s0, b1 * s1);
+  const uint32_t bc = pack_bf16x2(b0 * c0, b1 * c1), as = pack_bf16x2(a0 * s0, a1 * s1);
+  o1 = pack_bf16x2(bf16_bits_to_f32(ac & 0xffffu) - bf16_bits_to_f32(bs & 0xffffu),
+                   __uint_as_float(ac & 0xffff0000u) - __uint_as_float(bs & 0xffff0000u));
+  o2 = pack_bf16x2(bf16_bits_to_f32(bc & 0xffffu) + bf16_bits_to_f32(as & 0xffffu),
+                   __uint_as_float(bc & 0xffff0000u) + __uint_as_float(as & 0xffff0000u));
 }
 
 // Eight consecutive table values starting at element `off` (a multiple of 8), as packed bf16.
@@ -60,23 +63,23 @@ __device__ __forceinline__ u32x2 rope_load4(const void* tab, int is_f32, int64_t
 __device__ __forceinline__ void rope_rotate_halves(u32x4& lo, u32x4& hi, const u32x4 c8, const u32x4 s8) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    uint32_t a0, b0, a1, b1;
-    rope_pair(lo[e] & 0xffffu, hi[e] & 0xffffu, c8[e] & 0xffffu, s8[e] & 0xffffu, a0, b0);
-    rope_pair(lo[e] >> 16, hi[e] >> 16, c8[e] >> 16, s8[e] >> 16, a1, b1);
-    lo[e] = a0 | (a1 << 16);
-    hi[e] = b0 | (b1 << 16);
+    uint32_t a, b;
+    rope_pair2(lo[e], hi[e], c8[e], s8[e], a, b);
+    lo[e] = a, hi[e] = b;
   }
 }
 
 // Adjacent pairing: x holds dims d..d+7 = four pairs (2i, 2i+1); c4 / s4 the table columns d/2..d/2+3.
 __device__ __forceinline__ void rope_rotate_adjacent(u32x4& x, const u32x2 c4, const u32x2 s4) {
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const uint32_t c = (e & 1) ? (c4[e >> 1] >> 16) : (c4[e >> 1] & 0xffffu);
-    const uint32_t s = (e & 1) ? (s4[e >> 1] >> 16) : (s4[e >> 1] & 0xffffu);
+  for (int e = 0; e < 2; ++e) {
+    // words 2e, 2e+1 hold the pairs (x1 | x2 << 16); regroup into x1s and x2s of both pairs
+    const uint32_t w0 = x[2 * e], w1 = x[2 * e + 1];
+    const uint32_t x1 = (w0 & 0xffffu) | (w1 << 16), x2 = (w0 >> 16) | (w1 & 0xffff0000u);
     uint32_t a, b;
-    rope_pair(x[e] & 0xffffu, x[e] >> 16, c, s, a, b);
-    x[e] = a | (b << 16);
+    rope_pair2(x1, x2, c4[e], s4[e], a, b);
+    x[2 * e] = (a & 0xffffu) | (b << 16);
+    x[2 * e + 1] = (a >> 16) | (b & 0xffff0000u);
   }
 }
 

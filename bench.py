@@ -95,7 +95,7 @@ class FixedStep:
     """Direct C-ABI calls with metadata frozen at "T new tokens on top of the prefilled cache":
     the new tokens land on the same positions every step, so each step moves the same bytes."""
 
-    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True):
+    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True, rope=None):
         import numpy as np
         from pace_mi355 import _native as nat
 
@@ -140,12 +140,27 @@ class FixedStep:
         if fused:  # the attention launch reads the new tokens from k_new / v_new and stores them into the pool
             a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
             a.new_stride_b, a.new_stride_h, a.new_stride_t = k_new.stride(0), k_new.stride(1), k_new.stride(2)
+        # rope (a pace_rope_t with positions == NULL: rows follow the sequence positions): folded into the
+        # attention launch when the append is, else into the append launch, which then also rotates q
+        self.rope, self.q_rot = rope, None
+        if rope is not None and fused:
+            a.rope = ctypes.pointer(rope)
+        elif rope is not None:
+            self.q_rot = torch.empty_like(q)
+            a.q = self.q_rot.data_ptr()
         self.args, self.q = a, q
         self.attn = self.lib.pace_paged_attn_decode if S == 1 else self.lib.pace_paged_attn_verify
         self.stream = nat.current_stream_ptr()
 
     def append(self):
         k, v = self.k, self.v
+        if self.rope is not None:
+            q, qo = self.q, self.q_rot
+            self.nat.check(self.lib.pace_rope_append_paged(
+                ctypes.byref(self.cache._desc), ctypes.byref(self.rope), q.data_ptr(), qo.data_ptr(), q.stride(0), q.stride(1),
+                q.stride(2), q.shape[1], k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2), self.B, self.T,
+                self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr(), -self.T, self.stream))
+            return
         self.nat.check(self.lib.pace_kv_append_paged(
             ctypes.byref(self.cache._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2), self.B, self.T,
             self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr(), -self.T, self.stream))
@@ -242,6 +257,7 @@ def wl_decode_8b(torch, dev, args):
     g = torch.Generator(device=dev).manual_seed(2)
     k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
     q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
+    keep = []
     if args.path == "api":
         from pace_mi355.ops import MultiHeadAttention
 
@@ -255,7 +271,18 @@ def wl_decode_8b(torch, dev, args):
             if ev:
                 ev[1].record()
     else:
-        step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse)
+        rope = None
+        if args.rope:  # q and k arrive un-rotated; llama-3 tables as RotaryEmbedding builds them
+            from pace_mi355 import _native as nat
+            from pace_mi355.ops import RotaryEmbedding
+
+            mod = RotaryEmbedding(dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                       original_max_position_embeddings=8192), D, 8192, 500000.0)
+            cos, sin = mod.device_tables(dev)
+            keep.extend([cos, sin])
+            rope = nat.RopeDesc(cos=cos.data_ptr(), sin=sin.data_ptr(), table_dtype=nat.DTYPE_BF16, table_rows=cos.shape[0],
+                                rotary_dim=D, interleaved=0, positions=None, pos_stride_b=0)
+        step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse, rope=rope)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     if args.path == "api":  # average context over the timed steps
         ctx = ctx + args.warmup + (args.steps - 1) // 2
@@ -269,7 +296,7 @@ def wl_decode_8b(torch, dev, args):
         dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline("paged_attn_kernel<128,1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
                  {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
-        {"path": args.path, "append_fused": fused})
+        {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct")})
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
@@ -451,6 +478,9 @@ def main() -> int:
                          "MultiHeadAttention")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--rope", action="store_true",
+                    help="decode-8b, direct path: q and k arrive un-rotated and the rotary embedding rides in the launch "
+                         "(with --no-fuse: in the append launch)")
     ap.add_argument("--no-fuse", action="store_true",
                     help="launch the append as its own kernel instead of fusing it into the attention launch")
     ap.add_argument("--no-permute", action="store_true", help="keep physical blocks in logical order (diagnostic)")
