@@ -154,23 +154,45 @@ __device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnPar
   const uint16_t* kb = p.k_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
   const uint16_t* vb = p.v_new + (int64_t)b * p.n_sb + (int64_t)kvh * p.n_sh;
   const u32x4 zero = {0u, 0u, 0u, 0u};
+  // Every load is issued unconditionally from a clamped (valid) token row and masked afterwards:
+  // without branches around them the loads all go out before the first wait.
+  u32x4 tab[ROPE ? 2 : 1][D / 32];
+  bool live[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int idx = 8 * (n >> 2) + 4 * t + (n & 3);
+    live[t] = idx < n_new;
+    const int tok = live[t] ? idx : 0;
+    if (ROPE) rope_fetch_row<D>(p.rope, rope_row(p.rope, b, tok, pos0 + tok), g, tab[t]);
+    const uint16_t* row = kb + (int64_t)tok * p.n_st + 8 * g;
 #pragma unroll
-    for (int kk = 0; kk < D / 32; ++kk)
-      r.k[t][kk] = idx < n_new ? *reinterpret_cast<const u32x4*>(kb + (int64_t)idx * p.n_st + kk * 32 + 8 * g) : zero;
-    if (ROPE && idx < n_new) rotate_row_regs<D>(p.rope, rope_row(p.rope, b, idx, pos0 + idx), g, r.k[t]);
+    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(row + kk * 32);
   }
 #pragma unroll
-  for (int j = 0; j < D / 16; ++j) {
-    u32x4 w = zero;
+  for (int t = 0; t < 2; ++t) {
+    if (ROPE) rope_apply_row<D>(p.rope, tab[t], r.k[t]);
+#pragma unroll
+    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = live[t] ? r.k[t][kk] : zero;
+  }
+  // V: 2-byte gathers (dim 16j + n of tokens 8g..8g+7), four dim tiles (32 loads) per round.
+  constexpr int JR = 4;
+#pragma unroll
+  for (int j0 = 0; j0 < D / 16; j0 += JR) {
+    uint32_t vals[JR][8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int tok = 8 * g + e;
-      if (tok < n_new) w[e >> 1] |= (uint32_t)vb[(int64_t)tok * p.n_st + 16 * j + n] << (16 * (e & 1));
+      const uint16_t* row = vb + (int64_t)(tok < n_new ? tok : 0) * p.n_st + n;
+#pragma unroll
+      for (int j = 0; j < JR; ++j) vals[j][e] = row[16 * (j0 + j)];
     }
-    r.v[j] = w;
+#pragma unroll
+    for (int j = 0; j < JR; ++j) {
+      u32x4 w = zero;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w[e >> 1] |= (8 * g + e < n_new ? vals[j][e] : 0u) << (16 * (e & 1));
+      r.v[j0 + j] = w;
+    }
   }
 }
 
