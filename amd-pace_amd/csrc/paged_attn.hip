@@ -430,8 +430,12 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   // Tokens [pool_end, len) are this step's new tokens when the append is fused in.
   const int n_new = FUSED ? min(p.n_new, len) : 0;
   const int pool_end = len - n_new;
-  const int tok_end = min(pool_end, part_begin + P);
   const int S = p.q_len, R = active ? S * p.n_rep : 0;
+  // Causal rows read tokens <= len - S + s: nothing past the limit of the group's last row is
+  // needed, which halves the work of a prefill chunk (whole units are skipped, not masked).
+  const int last_row = min(R, (qg + 1) * NQT * 16) - 1;
+  const int group_end = (p.causal && last_row >= 0) ? len - S + last_row / p.n_rep + 1 : len;
+  const int tok_end = min(min(pool_end, part_begin + P), group_end);
   // This wave's share of the partition's 32-token units.
   const int part_units = max(0, (tok_end - part_begin + 31) / 32);
   const int per_wave = (part_units + NW - 1) / NW;

@@ -348,6 +348,28 @@ def wl_verify(torch, dev, args):
                  {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2)}))
 
 
+def wl_prefill(torch, dev, args):
+    """One chunk of a chunked prefill: 512 new tokens per sequence appended to 3584 cached ones, then
+    causal attention of the chunk over the cache (the reference runs prefill as the same update_cache +
+    attention pair with q_len = prompt length, pace/llm/models/llama.py:286-299)."""
+    B, hq, hkv, D, past, S = 8, 32, 8, 128, 3584, 512
+    cache = build_cache(torch, dev, [past] * B, hq, hkv, D, seed=8, headroom=S + 64)
+    cache.partition_tokens = args.partition
+    g = torch.Generator(device=dev).manual_seed(9)
+    kd, vd = _randn_bf16(torch, (B, hkv, S, D), g, dev), _randn_bf16(torch, (B, hkv, S, D), g, dev)
+    q = _randn_bf16(torch, (B, hq, S, D), g, dev)
+    step = FixedStep(torch, cache, q, kd, vd, args.partition, fused=False)
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    # causal: row s of the chunk reads past + s + 1 tokens
+    flops = 4.0 * B * hq * D * sum(past + s + 1 for s in range(S))
+    kv_once = decode_bytes([past + S] * B, hq, hkv, D, q_len=S)
+    return result_line(
+        args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
+        "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
+        roofline("paged_attn_kernel<128,4,...> (prefill chunk; K/V counted once)", kv_once, attn_ms,
+                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2)}))
+
+
 def wl_compact(torch, dev, args):
     import numpy as np
 
@@ -463,8 +485,8 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
     }
 
 
-WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify, "compact": wl_compact,
-             "copy-calibration": wl_copy_calibration}
+WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill,
+             "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 
 def main() -> int:
