@@ -150,6 +150,7 @@ class PagedKVCache(KVCacheBase):
         self.fuse_append = True
         self._pending: Optional[Tuple[torch.Tensor, torch.Tensor, int, object]] = None
         self._query_rope = None
+        self.cow_blocks_copied = 0  # blocks copied on write after forks (per layer pool)
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
     # -- set-up -----------------------------------------------------------------
@@ -254,6 +255,8 @@ class PagedKVCache(KVCacheBase):
         lib = nat.load()
         stream = nat.current_stream_ptr()
         self._flush()
+        if st.tails_dirty:
+            self._unshare()
         if counts is None:
             new_lens = self.lens + T
             if self.seq_len + T > st.min_capacity:
@@ -319,6 +322,7 @@ class PagedKVCache(KVCacheBase):
         self.seq_len = int(self.lens.max(initial=0))
         if remove.any():
             self._release()
+            self.state.lengths_shrank()
 
     def _release(self) -> None:
         # Blocks are shared by every layer: only the longest view of a sequence frees.
@@ -333,6 +337,7 @@ class PagedKVCache(KVCacheBase):
         for p in peers:
             p._flush()
         new_lens = self.state.evict(b, logical_blocks, self.lens)
+        self.state.lengths_shrank()
         for p in peers:
             p.lens = new_lens.copy()
             p.seq_len = int(new_lens.max(initial=0))
@@ -353,35 +358,34 @@ class PagedKVCache(KVCacheBase):
         return len(moves)
 
     def reorder(self, beam_idx: Sequence[int]) -> None:
+        """Sequence ``i`` becomes old sequence ``beam_idx[i]``.  No K/V moves here: the block
+        tables are re-pointed and the blocks get several owners; the one block per sequence that
+        the next append writes into is copied then (copy-on-write, ``_unshare``)."""
         st = self.state
         peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
         for p in peers:
             p._flush()
-        old_table, old_n, old_lens = st.table.copy(), st.n_blocks.copy(), self.lens.copy()
-        pairs: List[Tuple[int, int]] = []
-        new_rows = []
-        for src in beam_idx:
-            n = int(old_n[src])
-            fresh = st.allocator.allocate(n)
-            pairs += list(zip(old_table[src, :n].tolist(), fresh))
-            new_rows.append(fresh)
-        if pairs:
-            dev = torch.tensor(pairs, dtype=torch.int32).pin_memory().to(self.pool.device, non_blocking=True)
+        src = [int(i) for i in beam_idx]
+        st.fork(src)
+        for p in peers:
+            p.lens = p.lens[src].copy()
+            p.seq_len = int(p.lens.max(initial=0))
+
+    def _unshare(self) -> None:
+        """Give every sequence a private copy of the block its next token lands in (all layers)."""
+        st = self.state
+        peers = [p for p in self._shared.get("layers", [self]) if p.pool is not None]
+        for p in peers:
+            p._flush()
+        lens = np.min([p.lens for p in peers], axis=0)  # the earliest position any layer will write
+        pairs = st.unshare_tails(lens)
+        if len(pairs):
+            dev = torch.from_numpy(pairs).pin_memory().to(self.pool.device, non_blocking=True)
             lib = nat.load()
             for pool in st.pools:
                 desc = self._describe(pool)
                 nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), dev.data_ptr(), len(pairs), nat.current_stream_ptr()))
-        for b in range(st.batch):
-            st.allocator.free(old_table[b, : int(old_n[b])].tolist())
-        st.table[:] = 0
-        for i, row in enumerate(new_rows):
-            st.table[i, : len(row)] = row
-            st.n_blocks[i] = len(row)
-        st._table_dirty = True
-        new_lens = old_lens[list(beam_idx)]
-        for p in peers:
-            p.lens = new_lens.copy()
-            p.seq_len = int(new_lens.max(initial=0))
+        self.cow_blocks_copied += len(pairs)
 
     def gather(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
         """Dense ``[B, Hkv*n_rep, L, D]`` copies of K and V (zeros past each length)."""

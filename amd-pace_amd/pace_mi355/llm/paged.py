@@ -23,12 +23,15 @@ def blocks_for(n_tokens: int) -> int:
 
 
 class BlockAllocator:
-    """LIFO free list over pool block ids ``0 .. num_blocks-1`` (lowest ids first)."""
+    """LIFO free list over pool block ids ``0 .. num_blocks-1`` (lowest ids first), with a
+    reference count per block: sequences forked from one another (beam search) point at the
+    same blocks until one of them writes."""
 
     def __init__(self, num_blocks: int):
         self.num_blocks = int(num_blocks)
         self._free: List[int] = list(range(self.num_blocks - 1, -1, -1))
         self._is_free = np.ones(self.num_blocks, dtype=bool)
+        self.refs = np.zeros(self.num_blocks, dtype=np.int32)
 
     @property
     def num_free(self) -> int:
@@ -42,17 +45,32 @@ class BlockAllocator:
         out = self._free[-n:][::-1]
         del self._free[-n:]
         self._is_free[out] = False
+        self.refs[out] = 1
         return out
 
+    def share(self, ids: Iterable[int]) -> None:
+        """One more owner for each of ``ids`` (an id may occur several times)."""
+        ids = np.asarray(list(ids), dtype=np.int64)
+        if ids.size:
+            if self._is_free[ids].any():
+                raise ValueError("cannot share a free block")
+            np.add.at(self.refs, ids, 1)
+
     def free(self, ids: Iterable[int]) -> None:
+        """Drop one owner of each of ``ids``; a block returns to the free list with its last owner."""
         ids = [int(i) for i in ids]
         if not ids:
             return
-        if self._is_free[ids].any() or len(set(ids)) != len(ids):
-            dup = [i for i in ids if self._is_free[i]] or ids
-            raise ValueError(f"block {dup[0]} freed twice")
-        self._is_free[ids] = True
-        self._free.extend(ids)
+        arr = np.asarray(ids, dtype=np.int64)
+        if self._is_free[arr].any():
+            raise ValueError(f"block {[i for i in ids if self._is_free[i]][0]} freed twice")
+        np.subtract.at(self.refs, arr, 1)
+        if (self.refs[arr] < 0).any():
+            raise ValueError(f"block {[i for i in ids if self.refs[i] < 0][0]} freed twice")
+        gone = [i for i in dict.fromkeys(ids) if self.refs[i] == 0]
+        if gone:
+            self._is_free[gone] = True
+            self._free.extend(gone)
 
     def take(self, ids: Iterable[int]) -> None:
         """Mark specific ids as used (compaction destinations)."""
@@ -61,12 +79,14 @@ class BlockAllocator:
             if not self._is_free[i]:
                 raise ValueError(f"block {i} is not free")
             self._is_free[i] = False
+            self.refs[i] = 1
         self._free = [i for i in self._free if i not in want]
 
-    def reset_free(self, is_free: np.ndarray) -> None:
+    def reset_free(self, is_free: np.ndarray, refs: Optional[np.ndarray] = None) -> None:
         """Replace the free list wholesale (lowest ids are handed out first again)."""
         self._is_free = is_free.copy()
         self._free = np.nonzero(is_free)[0][::-1].tolist()
+        self.refs = refs.astype(np.int32) if refs is not None else (~is_free).astype(np.int32)
 
     def free_ids(self) -> np.ndarray:
         return np.nonzero(self._is_free)[0]
@@ -98,6 +118,8 @@ class PagedState:
         self._lens_host: Optional[np.ndarray] = None
         self._workspace: Optional[torch.Tensor] = None
         self.min_capacity = 0  # tokens every sequence can hold in the blocks it already owns
+        self.has_shared = False  # some block has more than one owner (after a fork)
+        self.tails_dirty = False  # a sequence's last, partly filled block may have other owners
         self._items_key = None
         self._items_dev: Optional[torch.Tensor] = None
         self._parts_dev: Optional[torch.Tensor] = None
@@ -139,6 +161,59 @@ class PagedState:
         if freed:
             self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
         return freed
+
+    def lengths_shrank(self) -> None:
+        """A rollback or an eviction can make a block with several owners the last block of a
+        sequence again: the next append has to look at the tails once more."""
+        if self.has_shared:
+            self.has_shared = bool((self.allocator.refs > 1).any())
+            self.tails_dirty = self.has_shared
+
+    # -- forks (beam search) ----------------------------------------------------
+    def fork(self, source_rows: Sequence[int]) -> None:
+        """Sequence ``i`` becomes a copy of old sequence ``source_rows[i]`` without moving a byte:
+        the new table rows point at the same blocks, which then have several owners.  The block a
+        later append would write into is copied first (``unshare_tails``)."""
+        src = [int(i) for i in source_rows]
+        if len(src) != self.batch or any(i < 0 or i >= self.batch for i in src):
+            raise IndexError(f"fork expects {self.batch} source rows in [0, {self.batch})")
+        old_table, old_n = self.table.copy(), self.n_blocks.copy()
+        for i in src:  # new owners first, so that no block is freed in between
+            self.allocator.share(old_table[i, : int(old_n[i])].tolist())
+        for b in range(self.batch):
+            self.allocator.free(old_table[b, : int(old_n[b])].tolist())
+        self.table[:] = 0
+        for i, srow in enumerate(src):
+            n = int(old_n[srow])
+            self.table[i, :n] = old_table[srow, :n]
+            self.n_blocks[i] = n
+        self.has_shared = bool((self.allocator.refs > 1).any())
+        self.tails_dirty = self.has_shared
+        self._table_dirty = True
+        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
+
+    def unshare_tails(self, lens: np.ndarray) -> np.ndarray:
+        """Copy-on-write before an append at positions ``lens[b] ..``: a partly filled last block
+        that has other owners is replaced by a fresh block.  Returns the ``(src, dst)`` pairs whose
+        data the caller must copy (in every layer's pool) before anything is written."""
+        pairs: List[Tuple[int, int]] = []
+        self.tails_dirty = False
+        if not self.has_shared:
+            return np.zeros((0, 2), np.int32)
+        for b in range(self.batch):
+            pos = int(lens[b])
+            jb = pos // BLOCK
+            if pos % BLOCK == 0 or jb >= int(self.n_blocks[b]):
+                continue  # the append starts a block of its own
+            old = int(self.table[b, jb])
+            if self.allocator.refs[old] > 1:
+                new = self.allocator.allocate(1)[0]
+                self.allocator.free([old])
+                self.table[b, jb] = new
+                pairs.append((old, new))
+                self._table_dirty = True
+        self.has_shared = bool((self.allocator.refs > 1).any())
+        return np.asarray(pairs, dtype=np.int32).reshape(-1, 2)
 
     # -- device mirrors ---------------------------------------------------------
     def device_table(self) -> torch.Tensor:
@@ -264,7 +339,7 @@ class PagedState:
         fewest copies: every live block at or above ``n_live`` moves into a free
         id below it.  Returns ``[n_moves, 2]`` int32 ``(src, dst)``; the two id
         sets are disjoint."""
-        live = np.concatenate([self.table[b, : int(self.n_blocks[b])] for b in range(self.batch)] or [np.zeros(0, np.int32)])
+        live = np.unique(np.concatenate([self.table[b, : int(self.n_blocks[b])] for b in range(self.batch)] or [np.zeros(0, np.int32)]))
         n_live = live.size
         src = np.sort(live[live >= n_live])
         is_live = np.zeros(self.allocator.num_blocks, dtype=bool)
@@ -279,13 +354,14 @@ class PagedState:
             return
         remap = np.arange(self.allocator.num_blocks, dtype=np.int32)
         remap[moves[:, 0]] = moves[:, 1]
-        live = np.zeros(self.allocator.num_blocks, dtype=bool)
+        refs = np.zeros(self.allocator.num_blocks, dtype=np.int32)
         for b in range(self.batch):
             n = int(self.n_blocks[b])
             self.table[b, :n] = remap[self.table[b, :n]]
-            live[self.table[b, :n]] = True
-        self.allocator.reset_free(~live)
+            np.add.at(refs, self.table[b, :n], 1)
+        self.allocator.reset_free(refs == 0, refs)
         self._table_dirty = True
 
     def live_block_count(self) -> int:
-        return int(self.n_blocks.sum())
+        """Pool blocks in use (a block with several owners counts once)."""
+        return int((self.allocator.refs > 0).sum())

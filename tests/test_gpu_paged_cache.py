@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_bits_equal, seeded_kv
+from helpers import assert_attention_close, assert_bits_equal, seeded_kv, seeded_q
 from oracle.cache_ref import DynamicKVCacheRef, repeat_kv, valid_prefix
 from oracle.paged_ref import RaggedCacheModel
 
@@ -111,6 +111,56 @@ def test_beam_reorder(device):
     gk, gv = cache.gather()
     assert_bits_equal(gk, K, "K after beam reorder")
     assert_bits_equal(gv, V, "V after beam reorder")
+
+
+def test_beam_search_steps_copy_on_write(device):
+    """Several reorder / append rounds as beam search issues them (pace/llm/generator.py:606-610):
+    contents equal the reference's index_select semantics bit for bit, while only the block each
+    beam writes into is ever copied."""
+    B, H, D = 4, 2, 128
+    cache = _paged(256, num_blocks=64)
+    model = RaggedCacheModel(B, H, D)
+    k, v = seeded_kv(50, B, H, 37, D)
+    cache.update_cache(k.to(device), v.to(device), 2)
+    model.append(k, v)
+    q = seeded_q(51, B, H, 1, D)
+
+    def check(what):
+        K, V = model.dense()
+        gk, gv = cache.gather()
+        assert_bits_equal(gk, K, "K " + what)
+        assert_bits_equal(gv, V, "V " + what)
+
+    plans = [[0, 0, 2, 1], [3, 3, 3, 0], [0, 1, 2, 3], [1, 0, 0, 0], [2, 2, 1, 1], [0, 0, 0, 0]]
+    for step, idx in enumerate(plans * 3):
+        cache.update_cache_with_beam_indices(torch.tensor(idx))
+        model.reorder(idx)
+        check(f"after reorder {step}")
+        k, v = seeded_kv(60 + step, B, H, 1, D)
+        cache.update_cache(k.to(device), v.to(device), 2)
+        model.append(k, v)
+        out = cache.attend(q.to(device))
+        assert_attention_close(out, model.attention(q, 1), f"decode after reorder {step}")
+        check(f"after append {step}")
+    # 18 steps x 4 beams: at most one block per beam and step, none when a beam kept its own tail
+    assert 0 < cache.cow_blocks_copied <= 18 * 4
+    used = cache.state.live_block_count()
+    assert used <= 4 * 4 + 4, f"{used} blocks in use: forks must share their common prefix"
+    # rollback and eviction on top of shared blocks
+    cache.truncate([3, 0, 20, 1])
+    model.truncate([3, 0, 20, 1])
+    k, v = seeded_kv(90, B, H, 5, D)
+    cache.update_cache(k.to(device), v.to(device), 2)
+    model.append(k, v)
+    check("after rollback + append")
+    cache.evict_blocks(1, [0])
+    model.evict_blocks(1, [0], 16)
+    cache.compact()
+    check("after evict + compact")
+    k, v = seeded_kv(91, B, H, 2, D)
+    cache.update_cache(k.to(device), v.to(device), 2)
+    model.append(k, v)
+    check("after the last append")
 
 
 def test_manager_layers_share_block_table(device):

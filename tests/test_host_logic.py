@@ -240,6 +240,56 @@ def test_evict_and_compaction_plan_properties():
     assert len(st.plan_compaction()) == 0  # idempotent
 
 
+def test_fork_shares_blocks_and_copy_on_write_touches_only_shared_tails():
+    """Beam reorder as table surgery (the reference copies the whole cache, pace/llm/cache.py:161-167)."""
+    st = _state(batch=4, max_len=160, blocks=40)
+    lens = np.array([40, 40, 40, 40])  # 3 blocks each, the last holds 8 tokens
+    st.ensure_capacity(lens)
+    rows = {b: st.table[b, :3].tolist() for b in range(4)}
+    st.fork([2, 2, 0, 2])
+    assert [st.table[i, :3].tolist() for i in range(4)] == [rows[2], rows[2], rows[0], rows[2]]
+    assert st.allocator.refs[rows[2]].tolist() == [3, 3, 3] and st.allocator.refs[rows[0]].tolist() == [1, 1, 1]
+    assert st.allocator.num_free == 40 - 6 and st.live_block_count() == 6  # rows 1 and 3 were dropped
+    assert st.has_shared and st.tails_dirty
+    pairs = st.unshare_tails(lens)
+    # the three owners of rows[2]'s tail: two get a private copy, the last one keeps the original
+    assert len(pairs) == 2 and set(pairs[:, 0].tolist()) == {rows[2][2]}
+    assert st.allocator.refs[rows[2][2]] == 1 and not st.tails_dirty and st.has_shared
+    tails = [int(st.table[i, 2]) for i in range(4)]
+    assert len(set(tails)) == 4
+    assert len(st.unshare_tails(lens)) == 0
+    # full blocks stay shared; a sequence that ends on a block boundary needs no copy at all
+    st2 = _state(batch=2, max_len=160, blocks=40)
+    st2.ensure_capacity(np.array([32, 32]))
+    st2.fork([1, 1])
+    assert len(st2.unshare_tails(np.array([32, 32]))) == 0
+    # rollback into a shared full block makes it a tail again
+    st2.release_beyond(np.array([20, 20]))
+    st2.lengths_shrank()
+    assert st2.tails_dirty
+    assert len(st2.unshare_tails(np.array([20, 20]))) == 1
+    # dropping every owner frees the block exactly once
+    st2.release_beyond(np.array([0, 0]))
+    assert st2.allocator.num_free == 40 and not (st2.allocator.refs > 0).any()
+    with pytest.raises(IndexError):
+        st2.fork([0, 5])
+
+
+def test_compaction_moves_a_shared_block_once():
+    st = _state(batch=3, max_len=160, blocks=30)
+    st.ensure_capacity(np.array([48, 48, 48]))
+    st.fork([0, 0, 2])            # blocks of old row 1 are freed: holes at ids 3..5
+    moves = st.plan_compaction()
+    assert st.live_block_count() == 6 and len(moves) == 3
+    shared_before = st.table[0, :3].tolist()
+    st.apply_moves(moves)
+    assert st.table[0, :3].tolist() == st.table[1, :3].tolist()
+    remap = dict(zip(moves[:, 0].tolist(), moves[:, 1].tolist()))
+    assert st.table[0, :3].tolist() == [remap.get(x, x) for x in shared_before]
+    assert st.allocator.refs[st.table[0, :3]].tolist() == [2, 2, 2]
+    assert sorted(st.allocator.free_ids().tolist()) == list(range(6, 30))
+
+
 # ---- attention launch planning ----
 def test_plan_attention_uniform_batch_uses_dense_grid():
     st = _state(batch=4, max_len=8192, blocks=4 * 512)
