@@ -8,6 +8,7 @@ from .cache import (  # noqa: F401
 )
 from .contiguous import BMCKVCache, DynamicKVCache  # noqa: F401
 from .ops import LLMBackendType, LLMOperatorType  # noqa: F401
+from . import speculative  # noqa: F401
 
 __all__ = [
     "KVCacheType", "KVCacheManager", "KVCacheBase", "PagedKVCache", "PagedKVView",

@@ -233,14 +233,18 @@ class PagedKVCache(KVCacheBase):
         self.reorder([int(i) for i in beam_idx.tolist()])
 
     # -- paged-only surface -----------------------------------------------------
-    def append_ragged(self, key_states: torch.Tensor, value_states: torch.Tensor, counts: Sequence[int]):
-        """Append ``counts[b]`` of the ``T`` given tokens to sequence ``b``."""
+    def append_ragged(self, key_states: torch.Tensor, value_states: torch.Tensor, counts: Sequence[int],
+                      right_aligned: bool = False):
+        """Append ``counts[b]`` of the ``T`` given tokens to sequence ``b``: the first ones of its
+        row, or with ``right_aligned`` the last ones (the alignment multi-token attention uses for
+        its query rows, so a ragged verify step passes q, k and v padded the same way)."""
         self._pin_concat_dim(2)
         self._lazy_init(key_states)
-        self._append(key_states, value_states, np.asarray(counts, dtype=np.int64))
+        self._append(key_states, value_states, np.asarray(counts, dtype=np.int64), right_aligned=right_aligned)
         return self.key, self.value
 
-    def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray], rope=None) -> None:
+    def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray], rope=None,
+                right_aligned: bool = False) -> None:
         B, h_in, T, D = k.shape
         if rope is not None and (counts is not None or tuple(rope.rows.shape) != (B, T)):
             raise RuntimeError("rope rows must be [B, T] and cannot be combined with per-sequence counts")
@@ -271,7 +275,7 @@ class PagedKVCache(KVCacheBase):
                 raise ValueError("counts must lie in [0, T]")
             new_lens = self.lens + counts
             st.ensure_capacity(new_lens)
-            slots = torch.from_numpy(st.slots(self.lens, counts, T)).pin_memory().to(k.device, non_blocking=True)
+            slots = torch.from_numpy(st.slots(self.lens, counts, T, right_aligned)).pin_memory().to(k.device, non_blocking=True)
             nat.check(
                 lib.pace_kv_append(
                     ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),

@@ -302,14 +302,19 @@ class PagedState:
         return self._workspace
 
     # -- slot arithmetic --------------------------------------------------------
-    def slots(self, starts: np.ndarray, counts: np.ndarray, width: int) -> np.ndarray:
-        """``[B, width]`` int64 slot ids of tokens ``starts[b] .. starts[b]+counts[b]-1``; -1 pads."""
+    def slots(self, starts: np.ndarray, counts: np.ndarray, width: int, right_aligned: bool = False) -> np.ndarray:
+        """``[B, width]`` int64 slot ids of tokens ``starts[b] .. starts[b]+counts[b]-1``; -1 pads.
+        The ``counts[b]`` tokens of a row are its first ones, or its last ones with ``right_aligned``."""
         out = np.full((self.batch, width), -1, dtype=np.int64)
         for b in range(self.batch):
             n = int(counts[b])
             if n:
                 pos = np.arange(int(starts[b]), int(starts[b]) + n)
-                out[b, :n] = self.table[b, pos // BLOCK].astype(np.int64) * BLOCK + pos % BLOCK
+                ids = self.table[b, pos // BLOCK].astype(np.int64) * BLOCK + pos % BLOCK
+                if right_aligned:
+                    out[b, width - n:] = ids
+                else:
+                    out[b, :n] = ids
         return out
 
     # -- block-level plans ------------------------------------------------------

@@ -12,6 +12,10 @@ cache_ref      contiguous caches of the reference (``pace/llm/cache.py``)
 attention_ref  attention semantics (``pace/ops/backends/native.py:32-47``,
                ``csrc/ops/kernels/attention_kernels.cpp:162-257``) and the
                4-D causal mask the models build (``pace/llm/models/llama.py:284-310``)
+rope_ref       rotary embedding (``pace/ops/rotary_embedding.py``): tables, row
+               selection and the rotation with its bf16 rounding sequence
+speculative_ref  acceptance of speculated tokens and the rollback length for one
+               sequence (``pace/llm/generator.py:669-713``)
 paged_ref      contiguous-semantics model of the block-paged operations
                (append by slot, gather, truncate, evict, compact)
 
@@ -30,6 +34,11 @@ Pinning status (what independent evidence fixes each function):
                        the installed transformers' class of the same name
                        (a different release) -- the 4.51.3 behaviour itself
                        is **parity unpinned** by any reference test.
+  * rope_ref.*         no reference test exists; complex multiplication in fp64,
+                       rotation invariants, integer-bit emulation of the bf16
+                       roundings, transformers' inverse frequencies -- pinned,
+                       except the longrope row-selection rule: **parity unpinned**.
+  * speculative_ref.*  brute force against "1 + longest common prefix" -- pinned.
   * paged_ref.*        row permutations of the pinned contiguous cache; checked
                        against ``DynamicKVCacheRef`` replay of surviving tokens.
 """
