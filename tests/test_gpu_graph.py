@@ -1,0 +1,88 @@
+"""The entry points only enqueue kernels on the stream they are given -- no allocation, no
+memset, no host synchronisation -- so a decode step can be captured into a HIP graph and
+replayed.  Replays are checked against the eager result with eager work in between."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from helpers import assert_bits_equal, seeded_kv, seeded_q
+
+pytestmark = pytest.mark.gpu
+
+
+def _frozen_step(cache, q, k_new, v_new, out, ws, rope=None):
+    """C-ABI call with every argument fixed: one new token per sequence on top of the cache as it is."""
+    from pace_mi355 import _native as nat
+
+    lib = nat.load()
+    B, hq, S, D = q.shape
+    T = k_new.shape[2]
+    st = cache.state
+    lens_after = cache.lens + T
+    st.ensure_capacity(lens_after)
+    table = st.device_table()
+    lens_dev = torch.from_numpy(lens_after.astype("int32")).to(q.device)
+    a = nat.PagedAttnArgs()
+    a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+    a.block_table, a.table_stride, a.seq_lens = table.data_ptr(), table.stride(0), lens_dev.data_ptr()
+    a.causal, a.batch, a.num_q_heads, a.q_len = 1, B, hq, S
+    a.max_seq_len, a.partition_tokens, a.scale = int(lens_after.max()), 256, 1.0 / math.sqrt(D)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
+    a.new_stride_b, a.new_stride_h, a.new_stride_t = k_new.stride(0), k_new.stride(1), k_new.stride(2)
+    if rope is not None:
+        a.rope = ctypes.pointer(rope)
+    keep = (table, lens_dev, a, rope)
+
+    def launch():
+        fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
+        nat.check(fn(ctypes.byref(cache._desc), ctypes.byref(a), nat.current_stream_ptr()))
+
+    return launch, keep
+
+
+@pytest.mark.parametrize("S", [1, 4])
+def test_decode_step_replays_from_a_hip_graph(device, S):
+    from pace_mi355.llm import PagedKVCache
+
+    B, hkv, n_rep, D = 4, 2, 4, 128
+    lens = [700, 33, 1500, 256]  # several partitions: the merge kernel is part of the graph
+    cache = PagedKVCache(2048, num_kv_heads=hkv, n_rep=n_rep)
+    k, v = seeded_kv(1, B, hkv, max(lens), D)
+    cache.append_ragged(k.to(device), v.to(device), lens)
+    q = seeded_q(2, B, hkv * n_rep, S, D).to(device)
+    k1, v1 = (t.to(device) for t in seeded_kv(3, B, hkv, S, D))
+    out = torch.zeros(B, hkv * n_rep, S, D, dtype=torch.bfloat16, device=device)
+    ws = torch.empty(8 << 20, dtype=torch.uint8, device=device)
+    launch, keep = _frozen_step(cache, q, k1, v1, out, ws)
+    launch()
+    torch.cuda.synchronize()
+    eager = out.clone()
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        launch()  # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            launch()
+    for i in range(4):
+        out.zero_()
+        q_scratch = torch.randn(1 << 16, device=device).sum()  # unrelated eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(out, eager, f"replay {i}")
+        assert torch.isfinite(q_scratch)
+    # new inputs in the same buffers are picked up by the next replay
+    q.copy_(seeded_q(9, B, hkv * n_rep, S, D))
+    launch()
+    torch.cuda.synchronize()
+    eager2 = out.clone()
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert_bits_equal(out, eager2, "replay with new query")
+    assert not torch.equal(eager2, eager)
