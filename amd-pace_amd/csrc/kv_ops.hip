@@ -67,8 +67,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
 template <int D>
 __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t pool, const uint16_t* __restrict__ k_new,
                                                               const uint16_t* __restrict__ v_new, int64_t sb, int64_t sh,
-                                                              int64_t st, int32_t n_tokens, const AppendDest dest,
-                                                              int32_t first_block_hint) {
+                                                              int64_t st, int32_t n_tokens, const AppendDest dest) {
   constexpr int CHUNKS = D / 8;
   constexpr int BT = PACE_KV_BLOCK_TOKENS;
   __shared__ uint16_t ks[BT * D];
@@ -222,10 +221,10 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
     const uint16_t* vq = static_cast<const uint16_t*>(v_new);
     if (pool->head_dim == 128)
       hipLaunchKernelGGL(kv_append_block_kernel<128>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
-                         n_tokens, dest, 0);
+                         n_tokens, dest);
     else
       hipLaunchKernelGGL(kv_append_block_kernel<64>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
-                         n_tokens, dest, 0);
+                         n_tokens, dest);
     PACE_HIP_CHECK(hipGetLastError());
     return PACE_KV_OK;
   }

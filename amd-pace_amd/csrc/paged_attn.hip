@@ -20,8 +20,6 @@
 //   so probabilities never leave their lane between the two products, and the
 //   softmax state (running max, sum, output accumulators) of query row n lives
 //   in the four lanes (n, 0..3).
-#include <stdlib.h>
-
 #include "common.h"
 #include "rope.h"
 
@@ -694,15 +692,7 @@ struct Shape {
 };
 
 static Shape shape_for(int tiles, bool fused) {
-  if (tiles <= 1) {
-    Shape s = {1, 4, 2, 8};
-    // Tuning override for the single-tile (decode) kernel: "NW,OCC".
-    if (const char* e = getenv("PACE_KV_DECODE_SHAPE")) {
-      int nw = 0, occ = 0;
-      if (sscanf(e, "%d,%d", &nw, &occ) == 2) s.nw = nw, s.occ = occ;
-    }
-    return s;
-  }
+  if (tiles <= 1) return Shape{1, 4, 2, 8};
   // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit.
   // Four waves per workgroup (three streaming + the append wave when fused) keep two
   // workgroups on a compute unit.
@@ -774,7 +764,6 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   }
   PACE_TRY(1, 4, 2, 8)
   PACE_TRY(1, 4, 2, 2)
-  PACE_TRY(1, 8, 2, 8)
   PACE_TRY(2, 4, 2, 8)
   PACE_TRY(2, 3, 2, 8)
   PACE_TRY(4, 2, 1, 8)
@@ -1084,7 +1073,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   // share a compute unit, the waves placed second on each SIMD fall behind and leave a long
   // under-filled tail.  Applies to the fused decode shape (five waves per workgroup, so that
   // a two-waves-per-SIMD limit means one workgroup per compute unit).
-  if (sh.nqt == 1 && sh.nw == 4 && p.n_new > 0 && !getenv("PACE_KV_DECODE_SHAPE") && p.total_items > compute_units() &&
+  if (sh.nqt == 1 && sh.nw == 4 && p.n_new > 0 && p.total_items > compute_units() &&
       p.total_items <= 2ll * compute_units())
     launch_shape_sel.occ_max = 2;
   hipStream_t s = static_cast<hipStream_t>(stream);

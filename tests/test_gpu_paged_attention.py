@@ -187,3 +187,42 @@ def test_chunked_prefill_through_the_paged_path(device):
     gk, gv = cache.gather()
     K, V = model.dense(n_rep)
     assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
+
+
+@pytest.mark.parametrize("T", [1, 5, 32])
+def test_first_step_on_an_empty_cache(device, T):
+    """The very first update: nothing is cached yet, the attention launch sees only the tokens it
+    stores itself (fused) -- same as the reference's first update_cache + attention."""
+    from pace_mi355.llm import PagedKVCache
+    from oracle.paged_ref import RaggedCacheModel
+
+    B, hkv, n_rep, D = 3, 2, 4, 128
+    cache = PagedKVCache(128, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, D)
+    for step in range(3):
+        k, v = seeded_kv(40 + step, B, hkv, T, D)
+        q = seeded_q(50 + step, B, hkv * n_rep, T, D)
+        cache.update_cache(k.to(device), v.to(device), 2)
+        assert cache._pending is not None
+        model.append(k, v)
+        out = cache.attend(q.to(device))
+        assert_attention_close(out, model.attention(q, n_rep), f"T={T} step {step}")
+    gk, gv = cache.gather(n_rep=1)
+    K, V = model.dense(1)
+    assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
+
+
+def test_fused_append_with_sequences_of_length_zero_and_one(device):
+    """Ragged batch where some sequences hold nothing before the step."""
+    cache, model = _build(device, 4, 2, 4, 128, [0, 1, 15, 16], seed=77)
+    k1, v1 = seeded_kv(78, 4, 2, 1, 128)
+    q = seeded_q(79, 4, 8, 1, 128)
+    cache.update_cache(k1.to(device), v1.to(device), 2)
+    model.append(k1, v1)
+    out = cache.attend(q.to(device))
+    assert_attention_close(out, model.attention(q, 4), "lens 0/1/15/16 + 1")
+    # a sequence of one token attends to exactly that token: out == v
+    torch.testing.assert_close(out[0].float().cpu(), repeat_kv(v1, 4)[0].float(), atol=1e-2, rtol=1e-2)
+    gk, gv = cache.gather(n_rep=1)
+    K, V = model.dense(1)
+    assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
