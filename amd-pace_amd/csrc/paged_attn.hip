@@ -696,7 +696,12 @@ static Shape shape_for(int tiles, bool fused) {
   // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit.
   // Four waves per workgroup (three streaming + the append wave when fused) keep two
   // workgroups on a compute unit.
-  if (tiles == 2) return Shape{2, fused ? 3 : 4, 2, 8};
+  // Four tiles (64 query rows, one wave per SIMD) read K/V once for up to 64 rows, which pays
+  // while the launch is bound by HBM (a verify step of a wide GQA group).  Beyond 64 rows K/V
+  // are re-read per row group anyway and the launch is bound by the matrix cores, where two
+  // waves per SIMD hide the softmax arithmetic behind the other wave's products: measured on a
+  // 512-token prefill chunk, 607 TFLOP/s with two tiles against 468 with four and 450 with one.
+  if (tiles == 2 || tiles > 4) return Shape{2, fused ? 3 : 4, 2, 8};
   return Shape{4, 2, 1, 8};
 }
 

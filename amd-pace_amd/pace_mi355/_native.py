@@ -183,6 +183,15 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+def row_groups(query_rows: int) -> int:
+    """Workgroups one (sequence, KV head, partition) needs for ``query_rows`` = q_len * n_rep rows:
+    the library packs 16, 32 or 64 rows per workgroup (two 16-row tiles for 17..32 rows and for
+    anything beyond 64, four for 33..64)."""
+    tiles = max(1, -(-int(query_rows) // 16))
+    per_group = 1 if tiles <= 1 else (2 if tiles == 2 or tiles > 4 else 4)
+    return -(-tiles // per_group)
+
+
 def check(rc: int) -> None:
     """Raise ``NativeError`` carrying the library's message when ``rc`` is a failure."""
     if rc != 0:

@@ -452,8 +452,7 @@ class PagedKVCache(KVCacheBase):
         max_parts = 1
         if part:
             cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, self.num_kv_heads))
-            row_groups = -(-(S * (hq // self.num_kv_heads)) // 64)
-            slots = max(1, 512 // (self.num_kv_heads * row_groups))
+            slots = max(1, 512 // (self.num_kv_heads * nat.row_groups(S * (hq // self.num_kv_heads))))
             items, parts, max_parts = st.plan_attention(self.lens, part, cap, slots)
         if parts is not None:
             ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))

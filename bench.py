@@ -122,8 +122,7 @@ class FixedStep:
             partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
         part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, partition, cache.num_kv_heads))
         cap = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, cache.num_kv_heads))
-        row_groups = -(-(S * (hq // cache.num_kv_heads)) // 64)
-        slots = max(1, 512 // (cache.num_kv_heads * row_groups))
+        slots = max(1, 512 // (cache.num_kv_heads * nat.row_groups(S * (hq // cache.num_kv_heads))))
         # ragged batches: compact longest-first work list; single-round launches: evened-out partition counts
         self.items, self.parts, max_parts = cache.state.plan_attention(lens_after, part, cap, slots)
         a.max_seq_len, a.partition_tokens, a.scale = max_len, part, 1.0 / math.sqrt(D)
