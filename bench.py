@@ -34,11 +34,12 @@ for _p in (REPO, os.path.join(REPO, "amd-pace_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix-core peak, published
 METRIC = "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 1 GPU"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, scaled by the
 # same counters on the copy-calibration workload (figures and commands: profiles/decode_8b_paged_attn_kernel.txt).
-MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_069_400_000}
+MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_069_100_000}
 
 
 def kv_token_bytes(kv_heads, head_dim):
@@ -362,11 +363,14 @@ def wl_prefill(torch, dev, args):
     # causal: row s of the chunk reads past + s + 1 tokens
     flops = 4.0 * B * hq * D * sum(past + s + 1 for s in range(S))
     kv_once = decode_bytes([past + S] * B, hq, hkv, D, q_len=S)
+    tflops = flops / (attn_ms * 1e-3) / 1e12
     return result_line(
         args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
         "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
-        roofline("paged_attn_kernel<128,4,...> (prefill chunk; K/V counted once)", kv_once, attn_ms,
-                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2)}))
+        {"bound": "mfma", "kernel": "paged_attn_kernel<128,2,...> (prefill chunk)", "achieved": round(tflops, 1),
+         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+         "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5),
+         "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)})
 
 
 def wl_compact(torch, dev, args):
