@@ -2,6 +2,7 @@
 // All three are pure byte movers bounded by HBM bandwidth; every global access
 // is a 16-byte lane access, coalesced over rows of the token-major side.
 #include "common.h"
+#include "rope.h"
 
 namespace pace_kv {
 
@@ -64,10 +65,11 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
 // Slabs of blocks the append only partly covers are written element-wise for V so that
 // earlier tokens of the block stay untouched.
 // ---------------------------------------------------------------------------------
-template <int D>
+template <int D, bool ROPE>
 __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t pool, const uint16_t* __restrict__ k_new,
                                                               const uint16_t* __restrict__ v_new, int64_t sb, int64_t sh,
-                                                              int64_t st, int32_t n_tokens, const AppendDest dest) {
+                                                              int64_t st, int32_t n_tokens, const AppendDest dest,
+                                                              const RopeDev rope) {
   constexpr int CHUNKS = D / 8;
   constexpr int BT = PACE_KV_BLOCK_TOKENS;
   __shared__ uint16_t ks[BT * D];
@@ -86,11 +88,29 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
   const int off_lo = (int)(pos0 + t_lo - blk_pos0), n_here = t_hi - t_lo;  // slots off_lo .. off_lo+n_here-1
   const uint16_t* kin = k_new + (int64_t)b * sb + (int64_t)h * sh;
   const uint16_t* vin = v_new + (int64_t)b * sb + (int64_t)h * sh;
-  for (int c = threadIdx.x; c < n_here * CHUNKS; c += 256) {
-    const int r = c / CHUNKS, ch = c % CHUNKS;
-    const int64_t src = (int64_t)(t_lo + r) * st + ch * 8;
-    *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = *reinterpret_cast<const u32x4*>(kin + src);
-    *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = *reinterpret_cast<const u32x4*>(vin + src);
+  if (ROPE) {
+    // keys are rotated on their way into LDS: a thread takes the two chunks of eight rotation pairs
+    for (int c = threadIdx.x; c < n_here * (CHUNKS / 2); c += 256) {
+      const int r = c / (CHUNKS / 2), ci = c % (CHUNKS / 2);
+      const int t = t_lo + r;
+      int ca, cb;
+      rope_chunk_pair(rope, ci, ca, cb);
+      const int64_t src = (int64_t)t * st;
+      u32x4 ka = *reinterpret_cast<const u32x4*>(kin + src + ca * 8);
+      u32x4 kb = *reinterpret_cast<const u32x4*>(kin + src + cb * 8);
+      rope_rotate_chunks(rope, rope_row(rope, b, t, (int)(pos0 + t)), ci, ka, kb);
+      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ca * 8]) = ka;
+      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + cb * 8]) = kb;
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ca * 8]) = *reinterpret_cast<const u32x4*>(vin + src + ca * 8);
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + cb * 8]) = *reinterpret_cast<const u32x4*>(vin + src + cb * 8);
+    }
+  } else {
+    for (int c = threadIdx.x; c < n_here * CHUNKS; c += 256) {
+      const int r = c / CHUNKS, ch = c % CHUNKS;
+      const int64_t src = (int64_t)(t_lo + r) * st + ch * 8;
+      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = *reinterpret_cast<const u32x4*>(kin + src);
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = *reinterpret_cast<const u32x4*>(vin + src);
+    }
   }
   __syncthreads();
   uint16_t* kslab = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
@@ -201,6 +221,34 @@ __global__ __launch_bounds__(256) void kv_copy_blocks_kernel(pace_kv_pool_t src,
 
 using namespace pace_kv;
 
+namespace pace_kv {
+// Launches the block-wise append (n_tokens >= 8 per sequence, destination through the block table),
+// rotating the keys on the way when rope is given.  Arguments are already checked.
+int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void* k_new, const void* v_new, int64_t stride_b,
+                        int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens, const int32_t* block_table,
+                        int32_t table_stride, const int32_t* seq_lens, int32_t pos_offset, const RopeDev* rope,
+                        hipStream_t stream) {
+  PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
+  const AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset};
+  const unsigned blocks_x = (unsigned)((n_tokens + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS + 1);
+  dim3 grid(blocks_x, pool->num_kv_heads, batch);
+  const uint16_t* kq = static_cast<const uint16_t*>(k_new);
+  const uint16_t* vq = static_cast<const uint16_t*>(v_new);
+  const RopeDev none = {};
+#define PACE_BLOCK_APPEND(DIM, R_)                                                                                        \
+  hipLaunchKernelGGL((kv_append_block_kernel<DIM, R_>), grid, dim3(256), 0, stream, *pool, kq, vq, stride_b, stride_h, stride_t, \
+                     n_tokens, dest, rope ? *rope : none)
+  if (pool->head_dim == 128) {
+    if (rope) PACE_BLOCK_APPEND(128, true); else PACE_BLOCK_APPEND(128, false);
+  } else {
+    if (rope) PACE_BLOCK_APPEND(64, true); else PACE_BLOCK_APPEND(64, false);
+  }
+#undef PACE_BLOCK_APPEND
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
+}
+}  // namespace pace_kv
+
 static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
                       int64_t stride_b, int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
                       const AppendDest& dest, bool paged, void* stream) {
@@ -212,22 +260,9 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
   PACE_REQUIRE(stride_b % 8 == 0 && stride_h % 8 == 0 && stride_t % 8 == 0,
                "%s: input strides must be multiples of 8 elements", who);
   hipStream_t s_early = static_cast<hipStream_t>(stream);
-  if (paged && n_tokens >= 8) {
-    // Enough tokens per sequence to fill slabs: one workgroup per destination block.
-    PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
-    const unsigned blocks_x = (unsigned)((n_tokens + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS + 1);
-    dim3 grid(blocks_x, pool->num_kv_heads, batch);
-    const uint16_t* kq = static_cast<const uint16_t*>(k_new);
-    const uint16_t* vq = static_cast<const uint16_t*>(v_new);
-    if (pool->head_dim == 128)
-      hipLaunchKernelGGL(kv_append_block_kernel<128>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
-                         n_tokens, dest);
-    else
-      hipLaunchKernelGGL(kv_append_block_kernel<64>, grid, dim3(256), 0, s_early, *pool, kq, vq, stride_b, stride_h, stride_t,
-                         n_tokens, dest);
-    PACE_HIP_CHECK(hipGetLastError());
-    return PACE_KV_OK;
-  }
+  if (paged && n_tokens >= 8)  // enough tokens per sequence to fill slabs: one workgroup per destination block
+    return launch_block_append(who, pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest.table,
+                               dest.table_stride, dest.seq_lens, dest.pos_offset, nullptr, s_early);
   const int64_t rows = (int64_t)batch * n_tokens * pool->num_kv_heads;
   PACE_REQUIRE(rows < (int64_t)1 << 31, "%s: too many rows (%lld)", who, (long long)rows);
   const int chunks = pool->head_dim / 8;

@@ -119,6 +119,12 @@ __device__ __forceinline__ void rope_rotate_chunks(const RopeDev& r, int row, in
   }
 }
 
+// Block-wise append with optional key rotation (kv_ops.hip).
+int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void* k_new, const void* v_new, int64_t stride_b,
+                        int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens, const int32_t* block_table,
+                        int32_t table_stride, const int32_t* seq_lens, int32_t pos_offset, const RopeDev* rope,
+                        hipStream_t stream);
+
 // Host: checks a pace_rope_t and fills the device view.  Returns 0 or PACE_KV_EINVAL.
 int make_rope_dev(const pace_rope_t* rope, int head_dim, bool need_positions, const char* who, RopeDev* out);
 

@@ -171,10 +171,19 @@ extern "C" int pace_rope_append_paged(const pace_kv_pool_t* pool, const pace_rop
     p.q = static_cast<const uint16_t*>(q), p.q_out = static_cast<uint16_t*>(q_out);
     p.q_sb = q_stride_b, p.q_sh = q_stride_h, p.q_st = q_stride_t, p.Hq = num_q_heads;
   }
+  p.table = block_table, p.table_stride = table_stride, p.seq_lens = seq_lens, p.pos_offset = pos_offset;
+  p.T = n_tokens;
+  if (n_tokens >= 8) {
+    // Many tokens per sequence: keys and values go through the block-wise append (slab-ordered
+    // 16-byte stores, keys rotated while staged); the queries are rotated by a launch of their own.
+    if (int rc = launch_block_append(who, pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, block_table,
+                                     table_stride, seq_lens, pos_offset, &p.rope, static_cast<hipStream_t>(stream)))
+      return rc;
+    if (!q) return PACE_KV_OK;
+    return launch_rows(p, pool->head_dim, batch, stream, who);  // Hk == 0: query rows only
+  }
   p.k = static_cast<const uint16_t*>(k_new), p.v = static_cast<const uint16_t*>(v_new);
   p.k_sb = stride_b, p.k_sh = stride_h, p.k_st = stride_t, p.Hk = pool->num_kv_heads;
   p.pool = *pool, p.to_pool = 1;
-  p.table = block_table, p.table_stride = table_stride, p.seq_lens = seq_lens, p.pos_offset = pos_offset;
-  p.T = n_tokens;
   return launch_rows(p, pool->head_dim, batch, stream, who);
 }
