@@ -38,6 +38,7 @@ struct PagedAttnParams {
   int32_t table_stride;
   const int32_t* seq_lens;
   int32_t len_bias;
+  const int32_t* len_bias_dev;  // optional device-side addend (advanced between graph replays)
   const int32_t* kv_start;
   const void* mask;
   int32_t mask_is_f32;
@@ -414,7 +415,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       b = (int)(bz / (uint32_t)p.n_qgroups), qg = (int)(bz % (uint32_t)p.n_qgroups);
     }
   }
-  const int len_b = p.seq_lens[b] + p.len_bias;
+  const int len_b = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
   // An idle slot (past the end of the work, or a partition this sequence does not have) runs
   // as an empty sequence without query rows: it loads and stores nothing but keeps the barriers.
   const int n_parts_b = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len_b, p.part_tokens);
@@ -658,7 +659,7 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   const int s = (int)(row % S);
   const int hq = (int)((row / S) % p.num_q_heads);
   const int b = (int)(row / ((int64_t)S * p.num_q_heads));
-  const int len = p.seq_lens[b] + p.len_bias;
+  const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
   const int n_parts = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len, p.part_tokens);
   const float* ml = p.part_ml + row * p.max_parts * 2;
   const float* po = p.part_o + row * p.max_parts * D;
@@ -1039,7 +1040,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.v_bs = pool->v_block_stride, p.v_hs = pool->v_head_stride;
   p.num_blocks = pool->num_blocks;
   p.table = a->block_table, p.table_stride = a->table_stride;
-  p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.kv_start = a->kv_start;
+  p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.len_bias_dev = a->seq_len_bias_ptr, p.kv_start = a->kv_start;
   p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
   p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
   p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",
@@ -108,6 +108,7 @@ class PagedAttnArgs(Structure):
         ("max_parts", c_int32),
         ("seq_len_bias", c_int32),
         ("rope", POINTER(RopeDesc)),
+        ("seq_len_bias_ptr", c_void_p),
     ]
 
 

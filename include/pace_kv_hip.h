@@ -225,6 +225,11 @@ typedef struct pace_paged_attn_args {
    * seq_len - q_len + s.  One launch then covers rope + append + attention of
    * pace/llm/models/llama.py:147-165. */
   const pace_rope_t* rope;
+  /* Optional device int32 (NULL = off) added to every length like seq_len_bias.  A decode step captured
+   * into a HIP graph bakes in every host-side argument; with this the graph itself can advance the
+   * lengths between replays (a one-element increment kernel inside the graph).  max_seq_len must then
+   * bound the lengths over all replays, and the block table must already hold their blocks. */
+  const int32_t* seq_len_bias_ptr;
 } pace_paged_attn_args_t;
 
 /* The context split size (tokens per workgroup) the library uses for these sizes when

@@ -86,3 +86,68 @@ def test_decode_step_replays_from_a_hip_graph(device, S):
     torch.cuda.synchronize()
     assert_bits_equal(out, eager2, "replay with new query")
     assert not torch.equal(eager2, eager)
+
+
+def test_captured_decode_loop_advances_lengths_on_the_device(device):
+    """A whole decode loop from one captured step: the graph holds the fused append + attention
+    launch and a one-element increment of the device-side length addend, so every replay appends
+    at the next position and attends over one more token.  No host-side argument changes."""
+    from oracle.paged_ref import RaggedCacheModel
+    from pace_mi355 import _native as nat
+    from pace_mi355.llm import PagedKVCache
+
+    B, hkv, n_rep, D, steps = 3, 2, 4, 128, 40
+    lens0 = [100, 17, 333]
+    cache = PagedKVCache(512, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, D)
+    k, v = seeded_kv(1, B, hkv, max(lens0), D)
+    cache.append_ragged(k.to(device), v.to(device), lens0)
+    model.append(k, v, lens0)
+    st = cache.state
+    st.ensure_capacity(cache.lens + steps)           # blocks for every future position, before capture
+    table = st.device_table()
+    lens_dev = torch.tensor(lens0, dtype=torch.int32, device=device)
+    step_no = torch.zeros(1, dtype=torch.int32, device=device)
+    q = torch.zeros(B, hkv * n_rep, 1, D, dtype=torch.bfloat16, device=device)
+    k1, v1 = torch.zeros(B, hkv, 1, D, dtype=torch.bfloat16, device=device), torch.zeros(B, hkv, 1, D, dtype=torch.bfloat16, device=device)
+    out = torch.zeros_like(q)
+    ws = torch.empty(4 << 20, dtype=torch.uint8, device=device)
+    lib = nat.load()
+    a = nat.PagedAttnArgs()
+    a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+    a.block_table, a.table_stride, a.seq_lens = table.data_ptr(), table.stride(0), lens_dev.data_ptr()
+    a.seq_len_bias, a.seq_len_bias_ptr = 1, step_no.data_ptr()   # length = lens0 + 1 + steps done so far
+    a.causal, a.batch, a.num_q_heads, a.q_len = 1, B, hkv * n_rep, 1
+    a.max_seq_len, a.partition_tokens, a.scale = max(lens0) + steps, 128, 1.0 / math.sqrt(D)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.k_new, a.v_new, a.n_new = k1.data_ptr(), v1.data_ptr(), 1
+    a.new_stride_b, a.new_stride_h, a.new_stride_t = k1.stride(0), k1.stride(1), k1.stride(2)
+
+    def launch():
+        nat.check(lib.pace_paged_attn_decode(ctypes.byref(cache._desc), ctypes.byref(a), nat.current_stream_ptr()))
+        step_no.add_(1)
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launch()
+    for i in range(steps):
+        kn, vn = seeded_kv(100 + i, B, hkv, 1, D)
+        qn = seeded_q(200 + i, B, hkv * n_rep, 1, D)
+        k1.copy_(kn), v1.copy_(vn), q.copy_(qn)
+        graph.replay()
+        model.append(kn, vn)
+        if i % 7 == 0 or i == steps - 1:
+            torch.cuda.synchronize()
+            from helpers import assert_attention_close
+            assert_attention_close(out, model.attention(qn, n_rep), f"replay {i}")
+    torch.cuda.synchronize()
+    assert int(step_no.item()) == steps
+    cache.lens = cache.lens + steps
+    cache.seq_len = int(cache.lens.max())
+    gk, gv = cache.gather(n_rep=1)
+    K, V = model.dense(1)
+    assert_bits_equal(gk, K, "pool K after the captured loop")
+    assert_bits_equal(gv, V, "pool V after the captured loop")
