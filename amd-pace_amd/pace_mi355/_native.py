@@ -204,4 +204,7 @@ def current_stream_ptr() -> int:
     """Raw ``hipStream_t`` of torch's current stream on the current device."""
     import torch
 
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:  # one C call instead of building a Stream object
+        return int(raw(torch.cuda.current_device()))
     return int(torch.cuda.current_stream().cuda_stream)

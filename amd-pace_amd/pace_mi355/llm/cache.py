@@ -134,7 +134,10 @@ class PagedKVCache(KVCacheBase):
         self.state: Optional[PagedState] = None
         self.pool: Optional[torch.Tensor] = None
         self._desc: Optional[nat.PoolDesc] = None
-        self.lens: np.ndarray = np.zeros(0, dtype=np.int64)
+        self._uniform: Optional[bool] = None  # every sequence has the same length (None: not known)
+        self._plan_key = None
+        self._plan_val = None
+        self.lens = np.zeros(0, dtype=np.int64)
         self.seq_len = 0
         self.concat_dim = None
         self.key: Optional[PagedKVView] = None
@@ -152,6 +155,16 @@ class PagedKVCache(KVCacheBase):
         self._query_rope = None
         self.cow_blocks_copied = 0  # blocks copied on write after forks (per layer pool)
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
+
+    @property
+    def lens(self) -> np.ndarray:
+        """Tokens held per sequence (host copy)."""
+        return self._lens
+
+    @lens.setter
+    def lens(self, value: np.ndarray) -> None:
+        self._lens = value
+        self._uniform = None
 
     # -- set-up -----------------------------------------------------------------
     def _lazy_init(self, key_states: torch.Tensor) -> None:
@@ -282,7 +295,9 @@ class PagedKVCache(KVCacheBase):
                     B, T, slots.data_ptr(), stream,
                 )
             )
+        uniform = self._uniform if counts is None else None  # equal appends keep equal lengths equal
         self.lens = new_lens
+        self._uniform = uniform
         self.seq_len = self.seq_len + T if counts is None else int(new_lens.max(initial=0))
         if self.key is None:
             self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
@@ -410,6 +425,41 @@ class PagedKVCache(KVCacheBase):
             )
         return k, v
 
+    def _plan(self, B: int, hq: int, S: int, D: int, max_len: int):
+        """How one attention launch is cut: (work items, partitions per sequence, partition size,
+        most partitions per sequence, workspace bytes).  Equal lengths -- the usual decode batch --
+        take a short path that only asks the library again when the partition count changes."""
+        lib = nat.load()
+        if self._uniform is None:
+            self._uniform = bool(self.lens.size == 0 or (self.lens == self.lens[0]).all())
+        want = self.partition_tokens
+        if self._uniform:
+            key = (B, hq, S, D, want, -(-max_len // 128))
+            if key != self._plan_key:
+                part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
+                max_parts = max(1, -(-max_len // part)) if part else 1
+                ws = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, -(-max_len // 128) * 128, part, self.num_kv_heads))
+                self._plan_key, self._plan_val = key, (None, None, part, max_parts, ws)
+            return self._plan_val
+        if want == 0 and B > 1:
+            # A ragged batch is cut at about its mean length: the long sequences then spread over
+            # several workgroups (scheduled longest first) instead of forming the tail of the launch.
+            mean = float(self.lens.mean())
+            if max_len > 1.5 * mean:
+                want = max(1024, (int(mean) + 127) // 128 * 128)
+        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
+        items = parts = None
+        max_parts = 1
+        if part:
+            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, self.num_kv_heads))
+            slots = max(1, 512 // (self.num_kv_heads * nat.row_groups(S * (hq // self.num_kv_heads))))
+            items, parts, max_parts = self.state.plan_attention(self.lens, part, cap, slots)
+        if parts is not None:
+            ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
+        else:
+            ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
+        return items, parts, part, max_parts, ws_bytes
+
     def attend(self, query: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                kv_start: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``softmax(q K^T / sqrt(D) + mask) V`` of ``query [B, Hq, S, D]`` over this cache.
@@ -440,24 +490,7 @@ class PagedKVCache(KVCacheBase):
         st = self.state
         max_len = self.seq_len
         lib = nat.load()
-        want = self.partition_tokens
-        if want == 0 and B > 1:
-            # A ragged batch is cut at about its mean length: the long sequences then spread over
-            # several workgroups (scheduled longest first) instead of forming the tail of the launch.
-            mean = float(self.lens.mean())
-            if max_len > 1.5 * mean:
-                want = max(1024, (int(mean) + 127) // 128 * 128)
-        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
-        items = parts = None
-        max_parts = 1
-        if part:
-            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, self.num_kv_heads))
-            slots = max(1, 512 // (self.num_kv_heads * nat.row_groups(S * (hq // self.num_kv_heads))))
-            items, parts, max_parts = st.plan_attention(self.lens, part, cap, slots)
-        if parts is not None:
-            ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
-        else:
-            ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
+        items, parts, part, max_parts, ws_bytes = self._plan(B, hq, S, D, max_len)
         ws = st.workspace(ws_bytes)
         table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
         a = nat.PagedAttnArgs()

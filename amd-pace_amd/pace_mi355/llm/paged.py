@@ -126,6 +126,9 @@ class PagedState:
         self._max_parts = 1
 
     # -- capacity ---------------------------------------------------------------
+    def _min_blocks(self) -> int:
+        return int(self.n_blocks.min()) if self.n_blocks.size else 0
+
     def _grow_table(self, need_cols: int) -> None:
         if need_cols <= self.table.shape[1]:
             return
@@ -145,7 +148,7 @@ class PagedState:
             self.table[b, have:want] = self.allocator.allocate(want - have)
             self.n_blocks[b] = want
             self._table_dirty = True
-        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
+        self.min_capacity = self._min_blocks() * BLOCK
 
     def release_beyond(self, lens: np.ndarray) -> int:
         """Free the blocks no token of ``lens`` touches any more; returns how many."""
@@ -159,7 +162,7 @@ class PagedState:
             freed += have - want
             self._table_dirty = True
         if freed:
-            self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
+            self.min_capacity = self._min_blocks() * BLOCK
         return freed
 
     def lengths_shrank(self) -> None:
@@ -190,7 +193,7 @@ class PagedState:
         self.has_shared = bool((self.allocator.refs > 1).any())
         self.tails_dirty = self.has_shared
         self._table_dirty = True
-        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
+        self.min_capacity = self._min_blocks() * BLOCK
 
     def unshare_tails(self, lens: np.ndarray) -> np.ndarray:
         """Copy-on-write before an append at positions ``lens[b] ..``: a partly filled last block
@@ -334,7 +337,7 @@ class PagedState:
         self.table[b, : len(keep)] = row
         self.n_blocks[b] = len(keep)
         self._table_dirty = True
-        self.min_capacity = int(self.n_blocks.min(initial=0)) * BLOCK
+        self.min_capacity = self._min_blocks() * BLOCK
         out = lens.copy()
         out[b] -= removed_tokens
         return out

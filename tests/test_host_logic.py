@@ -193,6 +193,10 @@ def test_capacity_release_and_slots():
     lens = np.array([33, 16, 0])
     st.ensure_capacity(lens)
     assert st.n_blocks.tolist() == [3, 1, 0] and st.allocator.num_free == 36
+    assert st.min_capacity == 0  # the empty sequence owns no block yet
+    st2 = _state()
+    st2.ensure_capacity(np.array([33, 16, 5]))
+    assert st2.min_capacity == 16  # what every sequence can hold without a new block
     s = st.slots(np.array([30, 0, 0]), np.array([3, 2, 0]), 4)
     assert s[0].tolist() == [st.table[0, 1] * 16 + 14, st.table[0, 1] * 16 + 15, st.table[0, 2] * 16, -1]
     assert s[1].tolist()[:2] == [st.table[1, 0] * 16, st.table[1, 0] * 16 + 1] and (s[2] == -1).all()
