@@ -1,0 +1,206 @@
+// Inner step shared by the paged and the dense attention kernels (gfx950 matrix cores).
+//
+// Inner step ("unit") = 32 tokens = two pool blocks.  With lane = (n, g),
+// n = lane % 16, g = lane / 16:
+//   S^T tile  = K[16 tokens x 32 dims] * Q^T[32 dims x 16 rows]   (v_mfma_f32_16x16x32_bf16)
+//       A operand: lane (n, g) holds 16 bytes of K row tok(n): dims 32*kk + 8g .. +8
+//       C layout : lane (n, g) holds rows 4g..4g+3 of the tile, column n = query row
+//   Token rows of the two tiles are interleaved so that lane (n, g) ends up with
+//   the scores of tokens 8g..8g+7 of the unit for query row n -- exactly the B
+//   operand slot of the second product:
+//   O^T tile  = V^T[16 dims x 32 tokens] * P^T[32 tokens x 16 rows]
+//       A operand: lane (n, g) holds 16 bytes of the token-minor V slab: dim 16j+n,
+//                  tokens 8g..8g+7 of the unit  (one coalesced 16-byte load)
+//   so probabilities never leave their lane between the two products, and the
+//   softmax state (running max, sum, output accumulators) of query row n lives
+//   in the four lanes (n, 0..3).
+#pragma once
+#include "common.h"
+#include "rope.h"
+
+namespace pace_kv {
+
+struct PagedAttnParams {
+  const uint16_t* q;
+  int64_t q_sb, q_sh, q_ss;
+  uint16_t* out;
+  int64_t o_sb, o_sh, o_ss;
+  const uint16_t* kpool;
+  const uint16_t* vpool;
+  int64_t k_bs, k_hs, v_bs, v_hs;
+  int32_t num_blocks;
+  const int32_t* table;
+  int32_t table_stride;
+  const int32_t* seq_lens;
+  int32_t len_bias;
+  const int32_t* len_bias_dev;  // optional device-side addend (advanced between graph replays)
+  const int32_t* kv_start;
+  const void* mask;
+  int32_t mask_is_f32;
+  int32_t mask_len;
+  int64_t m_sb, m_ss;
+  int32_t n_rep, q_len, num_q_heads;
+  int32_t causal;
+  int32_t n_qgroups;
+  int32_t num_kv_heads;
+  long long total_items;  // work items of the launch: KV heads x row groups x (sequence, partition) pairs
+  const int32_t* items;  // optional (sequence, partition) pairs
+  const int32_t* seq_parts;  // optional partitions per sequence (else derived from part_tokens)
+  int32_t part_tokens;
+  int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
+  float scale_log2;   // softmax scale * log2(e)
+  // Fused append: the last n_new tokens of every sequence are taken from k_new / v_new
+  // (and written to the pool by this launch) instead of being read from the pool.
+  const uint16_t* k_new;
+  const uint16_t* v_new;
+  int64_t n_sb, n_sh, n_st;
+  int32_t n_new;
+  float* part_o;      // [B][Hq][S][max_parts][D]
+  float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
+  // Optional rotary embedding (rope.cos == NULL: off): q rows are rotated as they are loaded,
+  // the fused append's new keys before they are used and stored.  rotary_dim == D here.
+  RopeDev rope;
+};
+
+constexpr float kNegInf = -__builtin_inff();
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+template <int D>
+struct UnitRegs {
+  u32x4 k[2][D / 32];  // [tile][contraction step]
+  u32x4 v[D / 16];     // [dim tile]
+};
+
+template <int D, int NQT>
+struct RowState {
+  f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
+  float m[NQT];          // running max (log2 units)
+  float l[NQT];          // this lane's share of the running sum
+  int limit[NQT];        // last readable token of the row (-1: row is padding)
+  int64_t mask_off[NQT]; // element offset of the row's mask line
+};
+
+template <int D, int NQT, bool HAS_MASK>
+__device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
+                                             RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
+                                             int start, bool full, int g) {
+  constexpr int KK = D / 32;
+  constexpr int MT = D / 16;
+#ifdef PACE_PROBE_LOADS_ONLY
+  {  // measurement aid: keep the loads, drop the arithmetic
+    u32x4 x = {0u, 0u, 0u, 0u};
+    for (int t = 0; t < 2; ++t)
+      for (int kk = 0; kk < KK; ++kk) x ^= r.k[t][kk];
+    for (int j = 0; j < MT; ++j) x ^= r.v[j];
+    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
+    st.l[0] = 1.f;
+    return;
+  }
+#endif
+  // Zero V columns past the end of the sequence so that stale pool contents
+  // (possibly non-finite bit patterns) cannot reach the accumulators.
+  u32x4 vreg[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) vreg[j] = r.v[j];
+  if (!full) {
+    const int nvalid = tok_end - (t0 + 8 * g);  // tokens of this lane's 8 that exist
+    if (nvalid < 8) {
+      u32x4 keep;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int c = nvalid - 2 * e;  // tokens 2e, 2e+1 live in dword e
+        keep[e] = c >= 2 ? 0xffffffffu : (c == 1 ? 0x0000ffffu : 0u);
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j) vreg[j] &= keep;
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[t][kk]),
+                                                      __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
+      s[t] = acc * p.scale_log2;
+    }
+    // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
+    if (HAS_MASK) {
+      const int mbase = t0 + 8 * g;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = mbase + 4 * t + i;
+          float add = kNegInf;
+          if (tok < p.mask_len && st.limit[qt] >= 0) {
+            if (p.mask_is_f32)
+              add = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok] * kLog2e;
+            else
+              add = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]) * kLog2e;
+          }
+          s[t][i] += add;
+        }
+    }
+    if (!full || HAS_MASK) {
+      const int hi = min(st.limit[qt], tok_end - 1);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = t0 + 8 * g + 4 * t + i;
+          if (tok > hi || tok < start) s[t][i] = kNegInf;
+          // a NaN score can only come from a stale K row; it is replaced above
+          // when out of range, and propagates (like the reference) when in range.
+        }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    mx = fmaxf(mx, xor_lanes(mx, 16));
+    mx = fmaxf(mx, xor_lanes(mx, 32));
+    const float m_old = st.m[qt];
+    const float m_new = fmaxf(m_old, mx);
+    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_old - m_use);  // m_old = -inf -> 0
+    float psum = 0.f;
+    f32x4 pr[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pr[t][i] = __builtin_amdgcn_exp2f(s[t][i] - m_use);
+        psum += pr[t][i];
+      }
+    st.m[qt] = m_new;
+    st.l[qt] = st.l[qt] * alpha + psum;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j) st.o[qt][j] *= alpha;
+    }
+    u32x4 pb;
+    pb[0] = pack_bf16x2(pr[0][0], pr[0][1]);
+    pb[1] = pack_bf16x2(pr[0][2], pr[0][3]);
+    pb[2] = pack_bf16x2(pr[1][0], pr[1][1]);
+    pb[3] = pack_bf16x2(pr[1][2], pr[1][3]);
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+      st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
+                                                           __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
+  }
+}
+
+// A sequence of `len` tokens is cut into ceil(len / part_tokens) partitions of equal size
+// (rounded up to whole 32-token units), so no partition is a short remainder.
+__host__ __device__ __forceinline__ int partition_count(int len, int part_tokens) {
+  return len > 0 ? (len + part_tokens - 1) / part_tokens : 1;
+}
+__host__ __device__ __forceinline__ int partition_size(int len, int n_parts) {
+  return (((len + n_parts - 1) / n_parts) + 31) & ~31;
+}
+
+}  // namespace pace_kv

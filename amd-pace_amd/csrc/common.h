@@ -31,7 +31,7 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 int check_pool(const pace_kv_pool_t* pool, const char* who);
 
-// Dense bf16 attention on the matrix cores (paged_attn.hip); false = shape not handled, nothing launched.
+// Dense bf16 attention on the matrix cores (dense_attn_mfma.hip); false = shape not handled, nothing launched.
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
                        const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream);
 

@@ -6,77 +6,10 @@
 // registers, so K and V are read from HBM once per KV head, not once per query
 // head.  A second small kernel merges the partitions of a sequence.
 //
-// Inner step ("unit") = 32 tokens = two pool blocks.  With lane = (n, g),
-// n = lane % 16, g = lane / 16:
-//   S^T tile  = K[16 tokens x 32 dims] * Q^T[32 dims x 16 rows]   (v_mfma_f32_16x16x32_bf16)
-//       A operand: lane (n, g) holds 16 bytes of K row tok(n): dims 32*kk + 8g .. +8
-//       C layout : lane (n, g) holds rows 4g..4g+3 of the tile, column n = query row
-//   Token rows of the two tiles are interleaved so that lane (n, g) ends up with
-//   the scores of tokens 8g..8g+7 of the unit for query row n -- exactly the B
-//   operand slot of the second product:
-//   O^T tile  = V^T[16 dims x 32 tokens] * P^T[32 tokens x 16 rows]
-//       A operand: lane (n, g) holds 16 bytes of the token-minor V slab: dim 16j+n,
-//                  tokens 8g..8g+7 of the unit  (one coalesced 16-byte load)
-//   so probabilities never leave their lane between the two products, and the
-//   softmax state (running max, sum, output accumulators) of query row n lives
-//   in the four lanes (n, 0..3).
-#include "common.h"
-#include "rope.h"
+// The inner step (one 32-token unit on the matrix cores) is in attn_core.h.
+#include "attn_core.h"
 
 namespace pace_kv {
-
-struct PagedAttnParams {
-  const uint16_t* q;
-  int64_t q_sb, q_sh, q_ss;
-  uint16_t* out;
-  int64_t o_sb, o_sh, o_ss;
-  const uint16_t* kpool;
-  const uint16_t* vpool;
-  int64_t k_bs, k_hs, v_bs, v_hs;
-  int32_t num_blocks;
-  const int32_t* table;
-  int32_t table_stride;
-  const int32_t* seq_lens;
-  int32_t len_bias;
-  const int32_t* len_bias_dev;  // optional device-side addend (advanced between graph replays)
-  const int32_t* kv_start;
-  const void* mask;
-  int32_t mask_is_f32;
-  int32_t mask_len;
-  int64_t m_sb, m_ss;
-  int32_t n_rep, q_len, num_q_heads;
-  int32_t causal;
-  int32_t n_qgroups;
-  int32_t num_kv_heads;
-  long long total_items;  // work items of the launch: KV heads x row groups x (sequence, partition) pairs
-  const int32_t* items;  // optional (sequence, partition) pairs
-  const int32_t* seq_parts;  // optional partitions per sequence (else derived from part_tokens)
-  int32_t part_tokens;
-  int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
-  float scale_log2;   // softmax scale * log2(e)
-  // Fused append: the last n_new tokens of every sequence are taken from k_new / v_new
-  // (and written to the pool by this launch) instead of being read from the pool.
-  const uint16_t* k_new;
-  const uint16_t* v_new;
-  int64_t n_sb, n_sh, n_st;
-  int32_t n_new;
-  float* part_o;      // [B][Hq][S][max_parts][D]
-  float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
-  // Optional rotary embedding (rope.cos == NULL: off): q rows are rotated as they are loaded,
-  // the fused append's new keys before they are used and stored.  rotary_dim == D here.
-  RopeDev rope;
-};
-
-constexpr float kNegInf = -__builtin_inff();
-constexpr float kLog2e = 1.4426950408889634f;
-
-__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
-
-template <int D>
-struct UnitRegs {
-  u32x4 k[2][D / 32];  // [tile][contraction step]
-  u32x4 v[D / 16];     // [dim tile]
-};
 
 // Issue the 16-byte loads of one 32-token unit.  ids: pool block ids of the
 // unit's two blocks (wave-uniform).
@@ -227,136 +160,6 @@ __device__ __forceinline__ void write_new_tokens(const PagedAttnParams& p, int b
       store_kv_chunk<D>(kslab, vslab, pos % PACE_KV_BLOCK_TOKENS, ci, kv, vv);
     }
   }
-}
-
-template <int D, int NQT>
-struct RowState {
-  f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
-  float m[NQT];          // running max (log2 units)
-  float l[NQT];          // this lane's share of the running sum
-  int limit[NQT];        // last readable token of the row (-1: row is padding)
-  int64_t mask_off[NQT]; // element offset of the row's mask line
-};
-
-template <int D, int NQT, bool HAS_MASK>
-__device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
-                                             RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
-                                             int start, bool full, int g) {
-  constexpr int KK = D / 32;
-  constexpr int MT = D / 16;
-#ifdef PACE_PROBE_LOADS_ONLY
-  {  // measurement aid: keep the loads, drop the arithmetic
-    u32x4 x = {0u, 0u, 0u, 0u};
-    for (int t = 0; t < 2; ++t)
-      for (int kk = 0; kk < KK; ++kk) x ^= r.k[t][kk];
-    for (int j = 0; j < MT; ++j) x ^= r.v[j];
-    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
-    st.l[0] = 1.f;
-    return;
-  }
-#endif
-  // Zero V columns past the end of the sequence so that stale pool contents
-  // (possibly non-finite bit patterns) cannot reach the accumulators.
-  u32x4 vreg[MT];
-#pragma unroll
-  for (int j = 0; j < MT; ++j) vreg[j] = r.v[j];
-  if (!full) {
-    const int nvalid = tok_end - (t0 + 8 * g);  // tokens of this lane's 8 that exist
-    if (nvalid < 8) {
-      u32x4 keep;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int c = nvalid - 2 * e;  // tokens 2e, 2e+1 live in dword e
-        keep[e] = c >= 2 ? 0xffffffffu : (c == 1 ? 0x0000ffffu : 0u);
-      }
-#pragma unroll
-      for (int j = 0; j < MT; ++j) vreg[j] &= keep;
-    }
-  }
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    f32x4 s[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[t][kk]),
-                                                      __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
-      s[t] = acc * p.scale_log2;
-    }
-    // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
-    if (HAS_MASK) {
-      const int mbase = t0 + 8 * g;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = mbase + 4 * t + i;
-          float add = kNegInf;
-          if (tok < p.mask_len && st.limit[qt] >= 0) {
-            if (p.mask_is_f32)
-              add = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok] * kLog2e;
-            else
-              add = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]) * kLog2e;
-          }
-          s[t][i] += add;
-        }
-    }
-    if (!full || HAS_MASK) {
-      const int hi = min(st.limit[qt], tok_end - 1);
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = t0 + 8 * g + 4 * t + i;
-          if (tok > hi || tok < start) s[t][i] = kNegInf;
-          // a NaN score can only come from a stale K row; it is replaced above
-          // when out of range, and propagates (like the reference) when in range.
-        }
-    }
-    float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
-    mx = fmaxf(mx, xor_lanes(mx, 16));
-    mx = fmaxf(mx, xor_lanes(mx, 32));
-    const float m_old = st.m[qt];
-    const float m_new = fmaxf(m_old, mx);
-    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_old - m_use);  // m_old = -inf -> 0
-    float psum = 0.f;
-    f32x4 pr[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        pr[t][i] = __builtin_amdgcn_exp2f(s[t][i] - m_use);
-        psum += pr[t][i];
-      }
-    st.m[qt] = m_new;
-    st.l[qt] = st.l[qt] * alpha + psum;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int j = 0; j < MT; ++j) st.o[qt][j] *= alpha;
-    }
-    u32x4 pb;
-    pb[0] = pack_bf16x2(pr[0][0], pr[0][1]);
-    pb[1] = pack_bf16x2(pr[0][2], pr[0][3]);
-    pb[2] = pack_bf16x2(pr[1][0], pr[1][1]);
-    pb[3] = pack_bf16x2(pr[1][2], pr[1][3]);
-#pragma unroll
-    for (int j = 0; j < MT; ++j)
-      st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
-                                                           __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
-  }
-}
-
-// A sequence of `len` tokens is cut into ceil(len / part_tokens) partitions of equal size
-// (rounded up to whole 32-token units), so no partition is a short remainder.
-__host__ __device__ __forceinline__ int partition_count(int len, int part_tokens) {
-  return len > 0 ? (len + part_tokens - 1) / part_tokens : 1;
-}
-__host__ __device__ __forceinline__ int partition_size(int len, int n_parts) {
-  return (((len + n_parts - 1) / n_parts) + 31) & ~31;
 }
 
 #ifdef PACE_PROBE_TIMING
@@ -775,204 +578,6 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   PACE_TRY(4, 2, 1, 8)
 #undef PACE_TRY
   return false;
-}
-
-// ---------------------------------------------------------------------------------
-// Dense bf16 attention with the same inner step: K and V are the reference's row-major
-// [B][N][L][D] tensors.  K rows feed the first product directly (16 bytes of a row per
-// lane); V rows are staged per wave in LDS and read back token-minor for the second.
-// One workgroup of 4 waves per (batch, head, group of 16*NQT query rows); the waves split
-// the L axis and merge through LDS like the paged kernel.
-// ---------------------------------------------------------------------------------
-struct DenseMfmaParams {
-  PagedAttnParams base;  // q / out / mask fields and scale are shared with the paged kernel
-  const uint16_t* k;
-  const uint16_t* v;
-  int32_t B, N, S, L;
-  int32_t mB, mN, mS;
-  int32_t n_qgroups;
-};
-
-template <int D, int NQT, bool HAS_MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1))) void dense_attn_mfma_kernel(const DenseMfmaParams dp) {
-  constexpr int KK = D / 32;
-  constexpr int MT = D / 16;
-  constexpr int NW = 4;
-  constexpr int VROW = D + 8;                     // padded LDS row (elements)
-  constexpr int STAGE = 32 * VROW;                // one wave's V unit
-  constexpr int MERGE_FLOATS = 2 * 16 * NQT * (D + 2);
-  constexpr int LDS_BYTES = (NW * STAGE * 2 > MERGE_FLOATS * 4) ? NW * STAGE * 2 : MERGE_FLOATS * 4;
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[LDS_BYTES];
-  const PagedAttnParams& p = dp.base;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
-  const int qg = blockIdx.x % dp.n_qgroups;
-  const int head = (blockIdx.x / dp.n_qgroups) % dp.N;
-  const int b = blockIdx.x / (dp.n_qgroups * dp.N);
-  const int L = dp.L, S = dp.S;
-  const uint16_t* kbase = dp.k + ((int64_t)b * dp.N + head) * (int64_t)L * D;
-  const uint16_t* vbase = dp.v + ((int64_t)b * dp.N + head) * (int64_t)L * D;
-  uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + wave * STAGE;
-
-  u32x4 qreg[NQT][KK];
-  RowState<D, NQT> st;
-  int row_s[NQT];
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    const int s = (qg * NQT + qt) * 16 + n;
-    const bool valid = s < S;
-    row_s[qt] = s;
-    st.limit[qt] = valid ? L - 1 : -1;
-    if (HAS_MASK) {
-      const int64_t mb = dp.mB == 1 ? 0 : b, mn = dp.mN == 1 ? 0 : head, ms = dp.mS == 1 ? 0 : (valid ? s : 0);
-      st.mask_off[qt] = ((mb * dp.mN + mn) * dp.mS + ms) * (int64_t)L;
-    } else {
-      st.mask_off[qt] = 0;
-    }
-    st.m[qt] = kNegInf;
-    st.l[qt] = 0.f;
-    const uint16_t* qp = p.q + (((int64_t)b * dp.N + head) * S + (valid ? s : 0)) * D + 8 * g;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      u32x4 z = {0u, 0u, 0u, 0u};
-      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
-    }
-#pragma unroll
-    for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  const int units = (L + 31) / 32;
-  const int per_wave = (units + NW - 1) / NW;
-  const int u_begin = min(units, wave * per_wave);
-  const int n_units = min(units, u_begin + per_wave) - u_begin;
-  UnitRegs<D> buf;
-  for (int uu = 0; uu < n_units; ++uu) {
-    const int t0 = 32 * (u_begin + uu);
-    // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g.. (clamped rows are masked later).
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int tok = min(L - 1, t0 + 8 * (n >> 2) + 4 * t + (n & 3));
-      const uint16_t* kp = kbase + (int64_t)tok * D + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + kk * 32);
-    }
-    // V: the unit's 32 rows go to this wave's LDS stage (coalesced 16-byte chunks) ...
-    constexpr int CH = D / 8;  // chunks per row
-#pragma unroll
-    for (int i = 0; i < 32 * CH / 64; ++i) {
-      const int c = i * 64 + lane, r = c / CH, ch = c % CH;
-      const int tok = min(L - 1, t0 + r);
-      *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = *reinterpret_cast<const u32x4*>(vbase + (int64_t)tok * D + ch * 8);
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
-    __builtin_amdgcn_wave_barrier();
-    // ... and come back token-minor: lane (n, g) takes dim 16j + n of tokens 8g..8g+7.
-#pragma unroll
-    for (int j = 0; j < MT; ++j) {
-      u32x4 w;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t lo = stage[(8 * g + 2 * e) * VROW + 16 * j + n];
-        const uint32_t hi = stage[(8 * g + 2 * e + 1) * VROW + 16 * j + n];
-        w[e] = lo | (hi << 16);
-      }
-      buf.v[j] = w;
-    }
-    __builtin_amdgcn_wave_barrier();
-    const bool full = t0 + 32 <= L;
-    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, L, 0, full, g);
-  }
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    float l = st.l[qt];
-    l += xor_lanes(l, 16);
-    l += xor_lanes(l, 32);
-    st.l[qt] = l;
-  }
-  __syncthreads();  // every wave is done with its V stage; the space becomes the merge buffer
-  float* merge_buf = reinterpret_cast<float*>(lds_raw);
-  constexpr int ROW_F = D + 2;
-  constexpr int SLOT_F = 16 * NQT * ROW_F;
-#pragma unroll
-  for (int stride = 1; stride < NW; stride *= 2) {
-    const int slot = wave / (2 * stride);
-    const bool sender = (wave & (2 * stride - 1)) == stride;
-    const bool receiver = (wave & (2 * stride - 1)) == 0;
-    if (sender) {
-#pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) {
-        float* rowp = merge_buf + slot * SLOT_F + (qt * 16 + n) * ROW_F;
-#pragma unroll
-        for (int j = 0; j < MT; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) rowp[16 * j + 4 * g + i] = st.o[qt][j][i];
-        if (g == 0) rowp[D] = st.m[qt], rowp[D + 1] = st.l[qt];
-      }
-    }
-    __syncthreads();
-    if (receiver) {
-#pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) {
-        const float* rowp = merge_buf + slot * SLOT_F + (qt * 16 + n) * ROW_F;
-        const float m_b = rowp[D], l_b = rowp[D + 1];
-        const float m_new = fmaxf(st.m[qt], m_b);
-        const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-        const float wa = __builtin_amdgcn_exp2f(st.m[qt] - m_use), wb = __builtin_amdgcn_exp2f(m_b - m_use);
-#pragma unroll
-        for (int j = 0; j < MT; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) st.o[qt][j][i] = st.o[qt][j][i] * wa + rowp[16 * j + 4 * g + i] * wb;
-        st.l[qt] = st.l[qt] * wa + l_b * wb;
-        st.m[qt] = m_new;
-      }
-    }
-    __syncthreads();
-  }
-  if (wave != 0) return;
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    if (row_s[qt] >= S) continue;
-    const float l = st.l[qt];
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* op = p.out + (((int64_t)b * dp.N + head) * S + row_s[qt]) * D + 4 * g;
-#pragma unroll
-    for (int j = 0; j < MT; ++j) {
-      u32x2 w;
-      w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
-      w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
-      *reinterpret_cast<u32x2*>(op + 16 * j) = w;
-    }
-  }
-}
-
-// Launches the dense bf16 kernel; returns false when the shape is not one it handles.
-bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
-                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream) {
-  if ((H != 64 && H != 128) || L < 1) return false;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(out) & 7u)) return false;
-  DenseMfmaParams dp = {};
-  dp.base.q = static_cast<const uint16_t*>(q);
-  dp.base.out = static_cast<uint16_t*>(out);
-  dp.base.mask = mask, dp.base.mask_is_f32 = mask_is_f32, dp.base.mask_len = L;
-  dp.base.scale_log2 = scale * kLog2e;
-  dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
-  dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
-  const int tiles = (S + 15) / 16;
-  const int nqt = tiles >= 2 ? 2 : 1;
-  dp.n_qgroups = (tiles + nqt - 1) / nqt;
-  const long long blocks = (long long)B * N * dp.n_qgroups;
-  if (blocks >= (1ll << 31)) return false;
-  const dim3 grid((unsigned)blocks), block(256);
-  const bool m = mask != nullptr;
-#define PACE_DENSE(D_, Q_, M_) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_>), grid, block, 0, stream, dp)
-  if (H == 128) {
-    if (nqt == 2) { if (m) PACE_DENSE(128, 2, true); else PACE_DENSE(128, 2, false); }
-    else { if (m) PACE_DENSE(128, 1, true); else PACE_DENSE(128, 1, false); }
-  } else {
-    if (nqt == 2) { if (m) PACE_DENSE(64, 2, true); else PACE_DENSE(64, 2, false); }
-    else { if (m) PACE_DENSE(64, 1, true); else PACE_DENSE(64, 1, false); }
-  }
-#undef PACE_DENSE
-  return true;
 }
 
 static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, void* stream, const char* who) {
