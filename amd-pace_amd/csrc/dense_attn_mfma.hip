@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1))) void d
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
   constexpr int NW = 4;
-  constexpr int VROW = D + 8;                     // padded LDS row (elements)
+  constexpr int VROW = D + 24;                    // padded LDS row (elements): keeps the transposed reads off each other's banks
   constexpr int STAGE = 32 * VROW;                // one wave's V unit
   constexpr int MERGE_FLOATS = 2 * 16 * NQT * (D + 2);
   constexpr int LDS_BYTES = (NW * STAGE * 2 > MERGE_FLOATS * 4) ? NW * STAGE * 2 : MERGE_FLOATS * 4;
@@ -92,17 +92,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1))) void d
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
     __builtin_amdgcn_wave_barrier();
-    // ... and come back token-minor: lane (n, g) takes dim 16j + n of tokens 8g..8g+7.
+    // ... and come back token-minor: lane (n, g) takes dim 16j + n of tokens 8g..8g+7.  The LDS
+    // transpose read hands lane i of a 16-lane group element i % 4 of the 8-byte pieces that
+    // lanes 4j + i / 4 (j = 0..3) point at; with lane s of the group pointing at token
+    // 8g + s / 4, dims 16j + 4 (s % 4) .. +3, lane n receives tokens 8g .. 8g+3 of dim 16j + n,
+    // and a second read four token rows further down completes the operand.
+    typedef short tr_v4 __attribute__((ext_vector_type(4)));
+    typedef tr_v4 __attribute__((address_space(3))) * tr_ptr;
+    const uint16_t* tr_base = stage + (8 * g + (n >> 2)) * VROW + 4 * (n & 3);
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
-      u32x4 w;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t lo = stage[(8 * g + 2 * e) * VROW + 16 * j + n];
-        const uint32_t hi = stage[(8 * g + 2 * e + 1) * VROW + 16 * j + n];
-        w[e] = lo | (hi << 16);
-      }
-      buf.v[j] = w;
+      const tr_v4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 16 * j));
+      const tr_v4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 4 * VROW + 16 * j));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      buf.v[j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
     }
     __builtin_amdgcn_wave_barrier();
     const bool full = t0 + 32 <= L;

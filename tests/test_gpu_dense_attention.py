@@ -2,6 +2,7 @@
 import pytest
 import torch
 
+import pace_mi355.ops  # noqa: F401  (defines torch.ops.pace.attention)
 from helpers import assert_attention_close, seeded_kv, seeded_q
 from oracle.attention_ref import sdpa_fp32, sdpa_native
 
