@@ -82,10 +82,16 @@ struct RowState {
   int64_t mask_off[NQT]; // element offset of the row's mask line
 };
 
-template <int D, int NQT, bool HAS_MASK>
-__device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
-                                             RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
-                                             int start, bool full, int g) {
+// FULL: every token of the unit exists and is readable by every query row (no masking code at all;
+// the caller decides once per unit, wave-uniformly).
+template <int D, int NQT, bool HAS_MASK, bool FULL>
+__device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
+                                                  RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
+                                                  int start, int g) {
+  // No fused multiply-add contraction in here: which operations the compiler would fuse depends on
+  // the instantiation, and the variants of one kernel are meant to give the same bits.
+#pragma clang fp contract(off)
+  constexpr bool full = FULL;
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
 #ifdef PACE_PROBE_LOADS_ONLY
@@ -148,13 +154,14 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (
         }
     }
     if (!full || HAS_MASK) {
-      const int hi = min(st.limit[qt], tok_end - 1);
+      // token t0 + 8g + c (c = 4t + i) is readable iff lo <= c <= hi, both relative to the lane's first token
+      const int base = t0 + 8 * g;
+      const int hi = min(st.limit[qt], tok_end - 1) - base, lo = start - base;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int tok = t0 + 8 * g + 4 * t + i;
-          if (tok > hi || tok < start) s[t][i] = kNegInf;
+          if (4 * t + i > hi || 4 * t + i < lo) s[t][i] = kNegInf;
           // a NaN score can only come from a stale K row; it is replaced above
           // when out of range, and propagates (like the reference) when in range.
         }
@@ -192,6 +199,16 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (
       st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
                                                            __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
   }
+}
+
+template <int D, int NQT, bool HAS_MASK>
+__device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
+                                             RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
+                                             int start, bool full, int g) {
+  if (full)
+    compute_unit_impl<D, NQT, HAS_MASK, true>(r, qreg, st, p, t0, tok_end, start, g);
+  else
+    compute_unit_impl<D, NQT, HAS_MASK, false>(r, qreg, st, p, t0, tok_end, start, g);
 }
 
 // A sequence of `len` tokens is cut into ceil(len / part_tokens) partitions of equal size

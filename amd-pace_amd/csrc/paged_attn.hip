@@ -19,16 +19,16 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
   // K: lane (n, g) supplies token 8*(n/4) + 4*tile + n%4 of the unit, i.e. token slot
   // n % 8 of slab tile `tile` in block A (n < 8) or B; dims 32*kk + 8g .. +8 are dim
   // chunk 4*kk + g.  A 16-lane quarter (fixed g) reads 128 contiguous bytes per block.
-  const int64_t kblk = (n >= 8) ? idB : idA;
-  const uint16_t* kp = p.kpool + kblk * p.k_bs + (int64_t)kvh * p.k_hs + g * 64 + (n & 7) * 8;
+  const int64_t offA = (int64_t)idA * p.k_bs, offB = (int64_t)idB * p.k_bs;  // wave-uniform products
+  const uint16_t* kp = p.kpool + ((n >= 8) ? offB : offA) + (int64_t)kvh * p.k_hs + g * 64 + (n & 7) * 8;
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + t * (D * 8) + kk * 256);
   // V: lane (n, g) supplies dim 16j + n, tokens 8g..8g+7 of the unit: token half g & 1
   // of block A (g < 2) or B.  A 16-lane quarter reads 256 contiguous bytes.
-  const int64_t vblk = (g >= 2) ? idB : idA;
-  const uint16_t* vp = p.vpool + vblk * p.v_bs + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
+  const int64_t voffA = (int64_t)idA * p.v_bs, voffB = (int64_t)idB * p.v_bs;
+  const uint16_t* vp = p.vpool + ((g >= 2) ? voffB : voffA) + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
 #pragma unroll
   for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
 }
@@ -297,6 +297,9 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   min_limit = min(min_limit, __shfl_xor(min_limit, 2, 64));
   min_limit = min(min_limit, __shfl_xor(min_limit, 4, 64));
   min_limit = min(min_limit, __shfl_xor(min_limit, 8, 64));
+  // the same in every lane (rows do not depend on the lane quarter): make that known, so that the
+  // full / partial decision per unit is a scalar branch
+  min_limit = __builtin_amdgcn_readfirstlane(min_limit);
 
   WaveBlockIds ids;
   {
