@@ -123,9 +123,11 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
       for (int j = 0; j < MT; ++j) vreg[j] &= keep;
     }
   }
+  // All score products first: the matrix cores then work through them (and later through the
+  // previous tile's second product) while the vector unit does a tile's softmax.
+  f32x4 sc[NQT][2];
 #pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    f32x4 s[2];
+  for (int qt = 0; qt < NQT; ++qt)
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -133,8 +135,13 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
       for (int kk = 0; kk < KK; ++kk)
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[t][kk]),
                                                       __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
-      s[t] = acc * p.scale_log2;
+      sc[qt][t] = acc;
     }
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) s[t] = sc[qt][t] * p.scale_log2;
     // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
     if (HAS_MASK) {
       const int mbase = t0 + 8 * g;
