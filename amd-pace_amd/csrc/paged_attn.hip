@@ -33,51 +33,6 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
   for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
 }
 
-// Rotate one head row held in operand order: x[kk] = dims 32*kk + 8g .. +8 of the row (lane
-// quarter g).  Both members of every rotation pair sit in the same lane: dim d pairs with
-// d + D/2 (register kk + KK/2) or, interleaved, with its neighbour inside the 16 bytes.
-// Split in two so that the table loads can be issued early and consumed late.
-template <int D>
-__device__ __forceinline__ void rope_fetch_row(const RopeDev& rope, int row, int g, u32x4 (&tab)[D / 32]) {
-  constexpr int KK = D / 32;
-  const int64_t base = (int64_t)row * (D / 2);
-  if (!rope.interleaved) {
-#pragma unroll
-    for (int kk = 0; kk < KK / 2; ++kk) {
-      const int64_t col = base + 32 * kk + 8 * g;
-      tab[2 * kk] = rope_load8(rope.cos, rope.is_f32, col);
-      tab[2 * kk + 1] = rope_load8(rope.sin, rope.is_f32, col);
-    }
-  } else {
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const int64_t col = base + 16 * kk + 4 * g;
-      const u32x2 c4 = rope_load4(rope.cos, rope.is_f32, col), s4 = rope_load4(rope.sin, rope.is_f32, col);
-      tab[kk] = u32x4{c4[0], c4[1], s4[0], s4[1]};
-    }
-  }
-}
-
-template <int D>
-__device__ __forceinline__ void rope_apply_row(const RopeDev& rope, const u32x4 (&tab)[D / 32], u32x4 (&x)[D / 32]) {
-  constexpr int KK = D / 32;
-  if (!rope.interleaved) {
-#pragma unroll
-    for (int kk = 0; kk < KK / 2; ++kk) rope_rotate_halves(x[kk], x[kk + KK / 2], tab[2 * kk], tab[2 * kk + 1]);
-  } else {
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-      rope_rotate_adjacent(x[kk], u32x2{tab[kk][0], tab[kk][1]}, u32x2{tab[kk][2], tab[kk][3]});
-  }
-}
-
-template <int D>
-__device__ __forceinline__ void rotate_row_regs(const RopeDev& rope, int row, int g, u32x4 (&x)[D / 32]) {
-  u32x4 tab[D / 32];
-  rope_fetch_row<D>(rope, row, g, tab);
-  rope_apply_row<D>(rope, tab, x);
-}
-
 // The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
 // (token idx of the unit = new token idx; tokens >= n_new are zero and get masked).
 template <int D, bool ROPE>

@@ -226,3 +226,42 @@ def test_fused_append_with_sequences_of_length_zero_and_one(device):
     gk, gv = cache.gather(n_rep=1)
     K, V = model.dense(1)
     assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
+
+
+@pytest.mark.parametrize("D,S,n_rep", [(128, 64, 4), (64, 48, 4), (128, 33, 8)])
+def test_prefill_sized_launch_matches_oracle(device, D, S, n_rep):
+    """A prefill-sized launch (hundreds of query rows per KV head over the whole batch): ragged
+    lengths, a partly filled last row group, and a chunk appended on top of cached tokens."""
+    B, hkv = 16, 8
+    rng = np.random.default_rng(S)
+    lens = (rng.integers(0, 300, B) + S).tolist()   # cached tokens + the S new ones
+    lens[0], lens[1] = S, S + 1                    # nothing / one token cached before the chunk
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=S + D)
+    q = seeded_q(31, B, hkv * n_rep, S, D)
+    out = cache.attend(q.to(device))
+    ref = model.attention(q, n_rep)
+    assert_attention_close(out, ref, f"prefill-sized S={S} D={D}")
+
+
+def test_prefill_sized_launch_with_rope_rotates_queries(device):
+    from oracle import rope_ref
+    from pace_mi355.llm import PagedKVCache
+    from pace_mi355.ops import RotaryEmbedding
+    from oracle.paged_ref import RaggedCacheModel
+
+    B, hkv, n_rep, D, S = 16, 8, 4, 128, 64
+    mod = RotaryEmbedding(None, D, 256, 10000.0)
+    cache = PagedKVCache(256, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, D)
+    past = 0
+    for step in range(2):
+        k, v = seeded_kv(70 + step, B, hkv, S, D)
+        q = seeded_q(80 + step, B, hkv * n_rep, S, D)
+        pos = torch.arange(past, past + S).repeat(B, 1)
+        rope = mod(k.to(device), pos.to(device))
+        cos, sin = rope_ref.lookup(mod.cos_cache, mod.sin_cache, pos, torch.bfloat16)
+        cache.update_cache(k.to(device), v.to(device), 2, rope=rope)
+        model.append(rope_ref.rotate(k, cos, sin), v)
+        out = cache.attend(q.to(device))
+        assert_attention_close(out, model.attention(rope_ref.rotate(q, cos, sin), n_rep), f"chunk {step}")
+        past += S
