@@ -265,3 +265,17 @@ def test_prefill_sized_launch_with_rope_rotates_queries(device):
         out = cache.attend(q.to(device))
         assert_attention_close(out, model.attention(rope_ref.rotate(q, cos, sin), n_rep), f"chunk {step}")
         past += S
+
+
+def test_very_long_context_single_sequence(device):
+    """One sequence of 70 k tokens: many partitions per sequence, block ids beyond one wave's
+    register window, the merge kernel over dozens of partials."""
+    lens = [70001]
+    cache, model = _build(device, 1, 2, 4, 128, lens, seed=5)
+    q = seeded_q(6, 1, 8, 1, 128)
+    assert_attention_close(cache.attend(q.to(device)), model.attention(q, 4), "70k decode")
+    k1, v1 = seeded_kv(7, 1, 2, 3, 128)
+    q3 = seeded_q(8, 1, 8, 3, 128)
+    cache.update_cache(k1.to(device), v1.to(device), 2)   # fused 3-token verify on top
+    model.append(k1, v1)
+    assert_attention_close(cache.attend(q3.to(device)), model.attention(q3, 4), "70k verify")
