@@ -149,7 +149,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   // One slot of 16*NQT query rows per sender of the first merge round.  Kept as small as the
   // shape allows: LDS is one of the limits on how many workgroups share a compute unit.
   constexpr int MERGE_SLOTS = NWT / 2 > 0 ? NWT / 2 : 1;
-  static_assert(MERGE_SLOTS * 16 * NQT <= 64, "LDS merge buffer holds at most 64 query rows");
+  static_assert(MERGE_SLOTS * 16 * NQT <= 128, "LDS merge buffer holds at most 128 query rows");
   __shared__ float merge_buf[MERGE_SLOTS * 16 * NQT * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
 #ifdef PACE_PROBE_TIMING
@@ -460,9 +460,11 @@ static Shape shape_for(int tiles, bool fused) {
   // workgroups on a compute unit.
   // Four tiles (64 query rows, one wave per SIMD) read K/V once for up to 64 rows, which pays
   // while the launch is bound by HBM (a verify step of a wide GQA group).  Beyond 64 rows K/V
-  // are re-read per row group anyway and the launch is bound by the matrix cores, where two
-  // waves per SIMD hide the softmax arithmetic behind the other wave's products: measured on a
-  // 512-token prefill chunk, 607 TFLOP/s with two tiles against 468 with four and 450 with one.
+  // are re-read per row group anyway and the launch is bound by the matrix cores and by the rate
+  // at which operands reach them: three tiles per wave are the most that still leave two waves
+  // per SIMD (one hides the other's softmax and load latency).  Measured on a 512-token prefill
+  // chunk: 768 TFLOP/s with three tiles, 708 with two, 468 with four, 450 with one.
+  if (tiles > 4 && !fused) return Shape{3, 4, 2, 8};
   if (tiles == 2 || tiles > 4) return Shape{2, fused ? 3 : 4, 2, 8};
   return Shape{4, 2, 1, 8};
 }
@@ -532,6 +534,7 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   PACE_TRY(1, 4, 2, 8)
   PACE_TRY(1, 4, 2, 2)
   PACE_TRY(2, 4, 2, 8)
+  PACE_TRY(3, 4, 2, 8)
   PACE_TRY(2, 3, 2, 8)
   PACE_TRY(4, 2, 1, 8)
 #undef PACE_TRY
