@@ -367,7 +367,7 @@ def wl_prefill(torch, dev, args):
     return result_line(
         args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
         "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
-        {"bound": "mfma", "kernel": "paged_attn_kernel<128,2,...> (prefill chunk)", "achieved": round(tflops, 1),
+        {"bound": "mfma", "kernel": "paged_attn_kernel<128,3,...> (prefill chunk)", "achieved": round(tflops, 1),
          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5),
          "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)})
