@@ -82,34 +82,50 @@ struct RowState {
   int64_t mask_off[NQT]; // element offset of the row's mask line
 };
 
+// Additive mask values of one unit fetched ahead of time by the caller: a[qt][c] belongs to token
+// t0 + 8g + c of query tile qt's row n (-inf where the mask has no such element).
+template <int NQT>
+struct MaskRegs {
+  float a[NQT][8];
+};
+
+// First product of a unit: the scores of its 32 tokens against every query tile.  All of them are
+// issued before any softmax, so that the matrix cores work through them (and later through the
+// previous tile's second product) while the vector unit does a tile's softmax.
+template <int D, int NQT>
+__device__ __forceinline__ void score_products(const u32x4 (&k)[2][D / 32], const u32x4 (&qreg)[NQT][D / 32],
+                                               f32x4 (&sc)[NQT][2]) {
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < D / 32; ++kk)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k[t][kk]),
+                                                      __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
+      sc[qt][t] = acc;
+    }
+}
+
+// Second half of a unit: masking, online softmax and the product with V.
 // FULL: every token of the unit exists and is readable by every query row (no masking code at all;
-// the caller decides once per unit, wave-uniformly).
-template <int D, int NQT, bool HAS_MASK, bool FULL>
-__device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
-                                                  RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
-                                                  int start, int g) {
+// the caller decides once per unit, wave-uniformly).  MREG: the mask values come from `mregs`
+// instead of being loaded here.
+template <int D, int NQT, bool HAS_MASK, bool FULL, bool MREG = false>
+__device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], const u32x4 (&v)[D / 16], RowState<D, NQT>& st,
+                                                   const PagedAttnParams& p, int t0, int tok_end, int start, int g,
+                                                   const MaskRegs<NQT>& mregs = MaskRegs<NQT>{}) {
   // No fused multiply-add contraction in here: which operations the compiler would fuse depends on
   // the instantiation, and the variants of one kernel are meant to give the same bits.
 #pragma clang fp contract(off)
   constexpr bool full = FULL;
-  constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-#ifdef PACE_PROBE_LOADS_ONLY
-  {  // measurement aid: keep the loads, drop the arithmetic
-    u32x4 x = {0u, 0u, 0u, 0u};
-    for (int t = 0; t < 2; ++t)
-      for (int kk = 0; kk < KK; ++kk) x ^= r.k[t][kk];
-    for (int j = 0; j < MT; ++j) x ^= r.v[j];
-    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
-    st.l[0] = 1.f;
-    return;
-  }
-#endif
   // Zero V columns past the end of the sequence so that stale pool contents
   // (possibly non-finite bit patterns) cannot reach the accumulators.
   u32x4 vreg[MT];
 #pragma unroll
-  for (int j = 0; j < MT; ++j) vreg[j] = r.v[j];
+  for (int j = 0; j < MT; ++j) vreg[j] = v[j];
   if (!full) {
     const int nvalid = tok_end - (t0 + 8 * g);  // tokens of this lane's 8 that exist
     if (nvalid < 8) {
@@ -123,20 +139,6 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
       for (int j = 0; j < MT; ++j) vreg[j] &= keep;
     }
   }
-  // All score products first: the matrix cores then work through them (and later through the
-  // previous tile's second product) while the vector unit does a tile's softmax.
-  f32x4 sc[NQT][2];
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt)
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[t][kk]),
-                                                      __builtin_bit_cast(bf16x8, qreg[qt][kk]), acc, 0, 0, 0);
-      sc[qt][t] = acc;
-    }
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     f32x4 s[2];
@@ -151,7 +153,9 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
         for (int i = 0; i < 4; ++i) {
           const int tok = mbase + 4 * t + i;
           float add = kNegInf;
-          if (tok < p.mask_len && st.limit[qt] >= 0) {
+          if (MREG) {
+            add = mregs.a[qt][4 * t + i] * kLog2e;
+          } else if (tok < p.mask_len && st.limit[qt] >= 0) {
             if (p.mask_is_f32)
               add = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok] * kLog2e;
             else
@@ -206,6 +210,27 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
       st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
                                                            __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
   }
+}
+
+// One whole unit from registers.
+template <int D, int NQT, bool HAS_MASK, bool FULL>
+__device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
+                                                  RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
+                                                  int start, int g) {
+#ifdef PACE_PROBE_LOADS_ONLY
+  {  // measurement aid: keep the loads, drop the arithmetic
+    u32x4 x = {0u, 0u, 0u, 0u};
+    for (int t = 0; t < 2; ++t)
+      for (int kk = 0; kk < D / 32; ++kk) x ^= r.k[t][kk];
+    for (int j = 0; j < D / 16; ++j) x ^= r.v[j];
+    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
+    st.l[0] = 1.f;
+    return;
+  }
+#endif
+  f32x4 sc[NQT][2];
+  score_products<D, NQT>(r.k, qreg, sc);
+  softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, r.v, st, p, t0, tok_end, start, g);
 }
 
 template <int D, int NQT, bool HAS_MASK>

@@ -14,6 +14,19 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+// Compute units of the current device (cached per process; 256 if the query fails).
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
 int check_pool(const pace_kv_pool_t* pool, const char* who) {
   PACE_REQUIRE(pool != nullptr, "%s: pool is NULL", who);
   PACE_REQUIRE(pool->k != nullptr && pool->v != nullptr, "%s: pool has a NULL K or V pointer", who);

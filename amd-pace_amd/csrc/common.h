@@ -30,6 +30,7 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
   } while (0)
 
 int check_pool(const pace_kv_pool_t* pool, const char* who);
+int compute_units();  // of the current device
 
 // Dense bf16 attention on the matrix cores (dense_attn_mfma.hip); false = shape not handled, nothing launched.
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,

@@ -1,5 +1,7 @@
 // Dense bf16 attention on the matrix cores for head_dim 64 / 128: the fast path of the torch op
 // pace::attention (dense_attn.hip holds the general kernel and the entry point).
+#include <type_traits>
+
 #include "attn_core.h"
 
 namespace pace_kv {
@@ -21,7 +23,7 @@ struct DenseMfmaParams {
 };
 
 template <int D, int NQT, bool HAS_MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1))) void dense_attn_mfma_kernel(const DenseMfmaParams dp) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_mfma_kernel(const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
   constexpr int NW = 4;
@@ -174,6 +176,196 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1))) void d
   }
 }
 
+// ---------------------------------------------------------------------------------
+// Many query rows per head (prefill): the four waves of a workgroup own 16*NQT query rows each
+// and walk the whole L axis together.  Every 32-token unit of K and V is brought into LDS once
+// per workgroup (coalesced 16-byte chunks, the next unit travelling through registers while
+// the current one is consumed) and read back by every wave in operand order: K rows directly,
+// V token-minor through the LDS transpose read.  No merge: a row's softmax state never leaves
+// its wave.  Mask values of the next unit are fetched along with it.
+// MASK: 0 none, 1 element-wise loads (any mask dtype / alignment), 2 bf16 mask whose rows are
+// 16-byte aligned (L % 8 == 0): one 16-byte load per row and unit.
+// ---------------------------------------------------------------------------------
+constexpr int kCoopWaves = 4;
+
+template <int D, int NQT, int MASK>
+__global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_coop_kernel(
+    const DenseMfmaParams dp) {
+  constexpr int KK = D / 32;
+  constexpr int MT = D / 16;
+  constexpr int KROW = D + 8;        // padded K row: the 16 rows of one operand read fall on different banks ...
+  constexpr int KHALF = 32;          // ... together with this shift of rows 16..31
+  constexpr int VROW = D + 24;       // padded V row for the transposed reads
+  constexpr int KSTAGE = 32 * KROW + KHALF;
+  constexpr int STAGE = KSTAGE + 32 * VROW;
+  constexpr int CH = D / 8;          // 16-byte chunks per row
+  constexpr int PER_THREAD = 32 * CH / (64 * kCoopWaves);
+  constexpr bool HAS_MASK = MASK != 0;
+  static_assert(PER_THREAD >= 1 && (32 * CH) % (64 * kCoopWaves) == 0, "unit does not divide over the workgroup");
+  __shared__ __attribute__((aligned(16))) uint16_t stage[2][STAGE];
+  const PagedAttnParams& p = dp.base;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, g = lane >> 4;
+  // Workgroups are dealt to the eight XCDs in turn: keep all row groups of one (batch, head) on
+  // one XCD, so that its K / V enter a single L2.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int pair = (slot / dp.n_qgroups) * 8 + xcd, rg = slot % dp.n_qgroups;
+  if (pair >= dp.B * dp.N) return;  // uniform over the workgroup
+  const int b = pair / dp.N, head = pair % dp.N;
+  const int L = dp.L, S = dp.S;
+  const uint16_t* kbase = dp.k + (int64_t)pair * L * D;
+  const uint16_t* vbase = dp.v + (int64_t)pair * L * D;
+  const int row0 = (rg * kCoopWaves + wave) * (NQT * 16);
+  const bool wave_has_rows = row0 < S;
+
+  u32x4 qreg[NQT][KK];
+  RowState<D, NQT> st;
+  int row_s[NQT];
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int s = row0 + qt * 16 + n;
+    const bool valid = s < S;
+    row_s[qt] = s;
+    st.limit[qt] = valid ? L - 1 : -1;
+    if (HAS_MASK) {
+      const int64_t mb = dp.mB == 1 ? 0 : b, mn = dp.mN == 1 ? 0 : head, ms = dp.mS == 1 ? 0 : (valid ? s : 0);
+      st.mask_off[qt] = ((mb * dp.mN + mn) * dp.mS + ms) * (int64_t)L;
+    } else {
+      st.mask_off[qt] = 0;
+    }
+    st.m[qt] = kNegInf;
+    st.l[qt] = 0.f;
+    const uint16_t* qp = p.q + ((int64_t)pair * S + (valid ? s : 0)) * D + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  u32x4 pre_k[PER_THREAD], pre_v[PER_THREAD];
+  u32x4 pre_m[MASK == 2 ? NQT : 1], cur_m[MASK == 2 ? NQT : 1];  // raw bf16 mask values (MASK == 2)
+  MaskRegs<NQT> mnext, mcur;                                      // fp32 values (MASK == 1)
+  auto fetch = [&](int u) {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
+      const int64_t off = (int64_t)min(L - 1, 32 * u + r) * D + ch * 8;  // rows past the end are masked later
+      pre_k[i] = *reinterpret_cast<const u32x4*>(kbase + off);
+      pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
+    }
+    if (MASK == 2) {
+      const int tok = 32 * u + 8 * g;  // L % 8 == 0: the eight values exist together or not at all
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) {
+        const u32x4 none = {0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u};  // -inf pairs
+        pre_m[qt] = tok < L ? *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p.mask) + st.mask_off[qt] + tok) : none;
+      }
+    } else if (MASK == 1) {
+      const int tok = 32 * u + 8 * g;
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          float a = kNegInf;
+          if (tok + c < L) {
+            if (p.mask_is_f32)
+              a = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok + c];
+            else
+              a = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok + c]);
+          }
+          mnext.a[qt][c] = a;
+        }
+    }
+  };
+  auto park = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
+      *reinterpret_cast<u32x4*>(&stage[buf][r * KROW + (r >= 16 ? KHALF : 0) + ch * 8]) = pre_k[i];
+      *reinterpret_cast<u32x4*>(&stage[buf][KSTAGE + r * VROW + ch * 8]) = pre_v[i];
+    }
+    if (MASK == 2) {
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) cur_m[qt] = pre_m[qt];
+    } else if (MASK == 1) {
+      mcur = mnext;
+    }
+  };
+
+  typedef short tr_v4 __attribute__((ext_vector_type(4)));
+  typedef tr_v4 __attribute__((address_space(3))) * tr_ptr;
+  // One unit out of its stage: K rows in operand order for the scores; V comes back token-minor
+  // only once the score products are issued, into the registers the K rows leave.
+  auto unit = [&](int cur, int t0, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    u32x4 kop[2][KK], vop[MT];
+    // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g ..
+    const int r0 = 8 * (n >> 2) + (n & 3);
+    const uint16_t* ks = &stage[cur][r0 * KROW + (r0 >= 16 ? KHALF : 0) + 8 * g];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) kop[t][kk] = *reinterpret_cast<const u32x4*>(ks + t * 4 * KROW + kk * 32);
+    f32x4 sc[NQT][2];
+    score_products<D, NQT>(kop, qreg, sc);
+    // V: dim 16j + n of tokens 8g .. 8g+7 (see the transposed read in the kernel above)
+    const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3)];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const tr_v4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 16 * j));
+      const tr_v4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 4 * VROW + 16 * j));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      vop[j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+    }
+    if (MASK == 2) {
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          mcur.a[qt][2 * e] = bf16_bits_to_f32(cur_m[qt][e] & 0xffffu);
+          mcur.a[qt][2 * e + 1] = __uint_as_float(cur_m[qt][e] & 0xffff0000u);
+        }
+    }
+    softmax_and_output<D, NQT, HAS_MASK, FULL, HAS_MASK>(sc, vop, st, p, t0, L, 0, g, mcur);
+  };
+  // Whole units in the loop, the partial last one (if any) after it: the loop body has one shape.
+  const int whole = L / 32, units = (L + 31) / 32;
+  fetch(0);
+  park(0);
+  __syncthreads();
+  for (int u = 0; u < whole; ++u) {
+    const int cur = u & 1;
+#ifndef PROBE_NOFETCH
+    fetch(min(u + 1, units - 1));  // unconditional: no branch between a load and the wait for it
+#endif
+    if (wave_has_rows) {
+      unit(cur, 32 * u, std::true_type{});
+    }
+    park(cur ^ 1);
+    __syncthreads();
+  }
+  if (whole < units && wave_has_rows) unit(whole & 1, 32 * whole, std::false_type{});
+
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float l = st.l[qt];
+    l += xor_lanes(l, 16);
+    l += xor_lanes(l, 32);
+    if (row_s[qt] >= S) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* op = p.out + ((int64_t)pair * S + row_s[qt]) * D + 4 * g;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      u32x2 w;
+      w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
+      w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
+      *reinterpret_cast<u32x2*>(op + 16 * j) = w;
+    }
+  }
+}
+
 // Launches the dense bf16 kernel; returns false when the shape is not one it handles.
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
                        const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream) {
@@ -187,6 +379,30 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
+  if (tiles > 4) {
+    // prefill-sized: rows of a head share its K / V through LDS
+    const int mode = !mask ? 0 : ((!mask_is_f32 && L % 8 == 0 && aligned16(mask)) ? 2 : 1);
+    int cnqt = 2;
+    dp.n_qgroups = (tiles + kCoopWaves * cnqt - 1) / (kCoopWaves * cnqt);
+    // too few workgroups: halve their rows; so does the element-wise mask path at head_dim 128, whose
+    // two-tile form does not fit the register file
+    if ((long long)B * N * dp.n_qgroups < compute_units() || (mode == 1 && H == 128)) {
+      cnqt = 1;
+      dp.n_qgroups = (tiles + kCoopWaves - 1) / kCoopWaves;
+    }
+    const long long pairs8 = ((long long)B * N + 7) / 8 * 8;
+    const long long cblocks = pairs8 * dp.n_qgroups;
+    if (cblocks >= (1ll << 31)) return false;
+    const dim3 cgrid((unsigned)cblocks), cblock(64 * kCoopWaves);
+#define PACE_COOP(D_, Q_, M_) hipLaunchKernelGGL((dense_attn_coop_kernel<D_, Q_, M_>), cgrid, cblock, 0, stream, dp)
+#define PACE_COOP_M(D_, Q_) \
+  do { if (mode == 0) PACE_COOP(D_, Q_, 0); else if (mode == 1) PACE_COOP(D_, Q_, 1); else PACE_COOP(D_, Q_, 2); } while (0)
+    if (H == 128) { if (cnqt == 2) PACE_COOP_M(128, 2); else PACE_COOP_M(128, 1); }
+    else { if (cnqt == 2) PACE_COOP_M(64, 2); else PACE_COOP_M(64, 1); }
+#undef PACE_COOP_M
+#undef PACE_COOP
+    return true;
+  }
   const int nqt = tiles >= 2 ? 2 : 1;
   dp.n_qgroups = (tiles + nqt - 1) / nqt;
   const long long blocks = (long long)B * N * dp.n_qgroups;

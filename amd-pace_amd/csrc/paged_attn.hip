@@ -469,18 +469,6 @@ static Shape shape_for(int tiles, bool fused) {
   return Shape{4, 2, 1, 8};
 }
 
-static int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n = v;
-    else
-      n = 256;
-  }
-  return n;
-}
-
 // Tokens one work item may cover: each wave holds at most 128 block ids.
 static int max_partition(int nw) { return nw * 2048; }
 

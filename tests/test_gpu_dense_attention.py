@@ -49,6 +49,40 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     assert_attention_close(out, sdpa_fp32(q, k, v, m), f"mask {mshape}")
 
 
+# Prefill-sized calls (more than 64 query rows) take the kernel whose waves share K / V through
+# LDS: ragged row and key counts, every mask form it distinguishes, head counts off a multiple of 8.
+@pytest.mark.parametrize("B,N,S,H,L,mask", [
+    (1, 3, 200, 128, 333, "causal-bf16"),   # element-wise mask loads (L % 8 != 0), partial last unit
+    (2, 5, 130, 128, 264, "causal-bf16"),   # 16-byte mask loads, L % 32 != 0
+    (1, 8, 65, 64, 96, "causal-f32"),       # fp32 mask with bf16 tensors
+    (2, 2, 512, 64, 512, "rows-bf16"),      # one mask line per batch entry
+    (1, 40, 256, 128, 256, "causal-bf16"),  # enough workgroups for two tiles per wave
+    (1, 9, 100, 128, 40, None),             # no mask (C ABI; the torch op always passes one)
+])
+def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
+    from oracle.attention_ref import causal_mask_4d
+    from pace_mi355 import _native as nat
+
+    k, v = seeded_kv(11, B, N, L, H)
+    q = seeded_q(12, B, N, S, H)
+    if mask is None:
+        m = None
+    elif mask.startswith("causal"):
+        dt = torch.float32 if mask.endswith("f32") else torch.bfloat16
+        m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, dt)
+        m = m + _mask(13, (B, 1, S, L), dt) * (m == 0)  # a bias on the readable part as well
+    else:
+        m = _mask(14, (B, 1, 1, L), torch.bfloat16)
+    qd, kd, vd = q.to(device), k.to(device), v.to(device)
+    if m is not None:
+        out = torch.ops.pace.attention(qd, kd, vd, m.to(device), 0)
+    else:
+        out = torch.empty_like(qd)
+        nat.check(nat.load().pace_attn_dense(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), nat.DTYPE_BF16,
+                                             B, N, S, L, H, None, nat.DTYPE_BF16, 1, 1, 1, nat.current_stream_ptr()))
+    assert_attention_close(out, sdpa_fp32(q, k, v, m), f"prefill {B}x{N}x{S}x{H}x{L} {mask}")
+
+
 def test_dense_op_with_bmc_padded_buffers_and_finfo_min_mask(device):
     """BMC returns padded buffers and pads the mask with finfo.min (cache.py:195-222); the padded
     columns must not contribute."""
