@@ -337,9 +337,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   __syncthreads();
   for (int u = 0; u < whole; ++u) {
     const int cur = u & 1;
-#ifndef PROBE_NOFETCH
     fetch(min(u + 1, units - 1));  // unconditional: no branch between a load and the wait for it
-#endif
     if (wave_has_rows) {
       unit(cur, 32 * u, std::true_type{});
     }

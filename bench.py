@@ -373,6 +373,39 @@ def wl_prefill(torch, dev, args):
          "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)})
 
 
+def wl_dense_prefill(torch, dev, args):
+    """The reference's own op at a prefill shape: torch.ops.pace.attention on dense [B, N, L, H] K/V with
+    the additive causal [B, 1, S, L] mask that LlamaModel.forward builds (pace/llm/models/llama.py:284-310),
+    as the JIT backend calls it (pace/ops/backends/jit.py:31-47).  The mask is additive and arbitrary, so
+    every (row, key) pair is computed: 4*B*N*S*L*H flop."""
+    import pace_mi355.ops  # noqa: F401  (defines the op)
+
+    B, N, S, L, H = 8, 32, 2048, 2048, 128
+    g = torch.Generator(device=dev).manual_seed(10)
+    q, k, v = (_randn_bf16(torch, (B, N, n, H), g, dev) for n in (S, L, L))
+    mask = torch.zeros(B, 1, S, L, device=dev, dtype=torch.bfloat16)
+    ar = torch.arange(L, device=dev)
+    mask.masked_fill_(ar[None, :] > ar[:S, None] + (L - S), torch.finfo(torch.bfloat16).min)
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        torch.ops.pace.attention(q, k, v, mask, False)
+        if ev:
+            ev[1].record()
+
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    flops = 4.0 * B * N * S * L * H
+    once = 2 * (q.numel() * 2 + k.numel() + v.numel()) + B * S * L * 2  # q, out, K, V and the mask read once
+    tflops = flops / (attn_ms * 1e-3) / 1e12
+    return result_line(
+        args, "dense op at a prefill shape: batch 8, 32 heads, 2048 queries x 2048 keys, head_dim 128, additive causal mask "
+        "[B,1,S,L]; step = one torch.ops.pace.attention call (output allocation included)", once, B * S, dt,
+        {"bound": "mfma", "kernel": "dense_attn_coop_kernel<128,2,2>", "achieved": round(tflops, 1),
+         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+         "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5)})
+
+
 def wl_compact(torch, dev, args):
     import numpy as np
 
@@ -489,7 +522,7 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
 
 
 WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill,
-             "compact": wl_compact, "copy-calibration": wl_copy_calibration}
+             "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 
 def main() -> int:
