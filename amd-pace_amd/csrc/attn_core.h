@@ -49,6 +49,7 @@ struct PagedAttnParams {
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)
+  float mask_mul;     // 1 / softmax scale: additive mask values in units of the raw score products
   // Fused append: the last n_new tokens of every sequence are taken from k_new / v_new
   // (and written to the pool by this launch) instead of being read from the pool.
   const uint16_t* k_new;
@@ -76,7 +77,8 @@ struct UnitRegs {
 template <int D, int NQT>
 struct RowState {
   f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
-  float m[NQT];          // running max (log2 units)
+  float m[NQT];          // running max: of the raw score products while units are consumed,
+                         // in log2 units (x scale_log2) after finish_rows()
   float l[NQT];          // this lane's share of the running sum
   int limit[NQT];        // last readable token of the row (-1: row is padding)
   int64_t mask_off[NQT]; // element offset of the row's mask line
@@ -141,9 +143,8 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
   }
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
-    f32x4 s[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) s[t] = sc[qt][t] * p.scale_log2;
+    // Scores stay in units of the raw products; the softmax scale enters once, in the exponent.
+    f32x4 s[2] = {sc[qt][0], sc[qt][1]};
     // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
     if (HAS_MASK) {
       const int mbase = t0 + 8 * g;
@@ -152,19 +153,20 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int tok = mbase + 4 * t + i;
-          float add = kNegInf;
           if (MREG) {
-            add = mregs.a[qt][4 * t + i] * kLog2e;
+            s[t][i] = __builtin_fmaf(mregs.a[qt][4 * t + i], p.mask_mul, s[t][i]);
           } else if (tok < p.mask_len && st.limit[qt] >= 0) {
-            if (p.mask_is_f32)
-              add = static_cast<const float*>(p.mask)[st.mask_off[qt] + tok] * kLog2e;
-            else
-              add = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]) * kLog2e;
+            const float add = p.mask_is_f32 ? static_cast<const float*>(p.mask)[st.mask_off[qt] + tok]
+                                            : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]);
+            s[t][i] = __builtin_fmaf(add, p.mask_mul, s[t][i]);
+          } else {
+            s[t][i] = kNegInf;
           }
-          s[t][i] += add;
         }
     }
-    if (!full || HAS_MASK) {
+    // With mask values handed in, a whole unit needs no range check: they are -inf where the mask
+    // has no element, and rows that are padding are never written.
+    if ((!full || HAS_MASK) && !(full && MREG)) {
       // token t0 + 8g + c (c = 4t + i) is readable iff lo <= c <= hi, both relative to the lane's first token
       const int base = t0 + 8 * g;
       const int hi = min(st.limit[qt], tok_end - 1) - base, lo = start - base;
@@ -184,14 +186,15 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     const float m_old = st.m[qt];
     const float m_new = fmaxf(m_old, mx);
     const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_old - m_use);  // m_old = -inf -> 0
+    const float alpha = __builtin_amdgcn_exp2f((m_old - m_use) * p.scale_log2);  // m_old = -inf -> 0
+    const float m_neg = -(m_use * p.scale_log2);
     float psum = 0.f;
     f32x4 pr[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        pr[t][i] = __builtin_amdgcn_exp2f(s[t][i] - m_use);
+        pr[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], p.scale_log2, m_neg));
         psum += pr[t][i];
       }
     st.m[qt] = m_new;
@@ -209,6 +212,20 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     for (int j = 0; j < MT; ++j)
       st.o[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vreg[j]),
                                                            __builtin_bit_cast(bf16x8, pb), st.o[qt][j], 0, 0, 0);
+  }
+}
+
+// After the last unit: complete the row sums over the four lanes of a row and express the running
+// max in log2 units, as the merges between waves and partitions expect it.
+template <int D, int NQT>
+__device__ __forceinline__ void finish_rows(RowState<D, NQT>& st, const PagedAttnParams& p) {
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float l = st.l[qt];
+    l += xor_lanes(l, 16);
+    l += xor_lanes(l, 32);
+    st.l[qt] = l;
+    st.m[qt] *= p.scale_log2;  // -inf stays -inf: the scale is positive
   }
 }
 

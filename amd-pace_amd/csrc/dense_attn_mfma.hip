@@ -113,13 +113,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
     const bool full = t0 + 32 <= L;
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, L, 0, full, g);
   }
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    float l = st.l[qt];
-    l += xor_lanes(l, 16);
-    l += xor_lanes(l, 32);
-    st.l[qt] = l;
-  }
+  finish_rows<D, NQT>(st, p);
   __syncthreads();  // every wave is done with its V stage; the space becomes the merge buffer
   float* merge_buf = reinterpret_cast<float*>(lds_raw);
   constexpr int ROW_F = D + 2;
@@ -374,6 +368,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.base.out = static_cast<uint16_t*>(out);
   dp.base.mask = mask, dp.base.mask_is_f32 = mask_is_f32, dp.base.mask_len = L;
   dp.base.scale_log2 = scale * kLog2e;
+  dp.base.mask_mul = 1.0f / scale;
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;

@@ -304,14 +304,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
 #ifdef PACE_PROBE_TIMING
   const long long pt2 = wall_clock64();
 #endif
-  // Row sums were kept per lane; complete them over the four lanes of a row.
-#pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    float l = st.l[qt];
-    l += xor_lanes(l, 16);
-    l += xor_lanes(l, 32);
-    st.l[qt] = l;
-  }
+  finish_rows<D, NQT>(st, p);  // row sums over the lanes of a row, running max in log2 units
 
   // Pairwise merge of the waves' states through LDS (fixed order: deterministic).
   if (NWT > 1) {
@@ -547,6 +540,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
                a->max_seq_len, a->table_stride);
   PACE_REQUIRE((int64_t)a->table_stride * PACE_KV_BLOCK_TOKENS >= a->max_seq_len,
                "%s: block table row (%d blocks) cannot hold max_seq_len %d", who, a->table_stride, a->max_seq_len);
+  PACE_REQUIRE(a->scale > 0.f && a->scale < __builtin_inff(), "%s: softmax scale must be positive and finite (got %g)", who,
+               (double)a->scale);
   if (a->mask) {
     PACE_REQUIRE(a->mask_dtype == PACE_DTYPE_F32 || a->mask_dtype == PACE_DTYPE_BF16, "%s: bad mask dtype %d", who,
                  a->mask_dtype);
@@ -601,6 +596,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.causal = a->causal;
   p.part_tokens = part, p.max_parts = max_parts;
   p.scale_log2 = a->scale * kLog2e;
+  p.mask_mul = 1.0f / a->scale;
   p.part_o = nullptr, p.part_ml = nullptr;
   p.k_new = static_cast<const uint16_t*>(a->k_new), p.v_new = static_cast<const uint16_t*>(a->v_new);
   p.n_sb = a->new_stride_b, p.n_sh = a->new_stride_h, p.n_st = a->new_stride_t;

@@ -189,7 +189,7 @@ typedef struct pace_paged_attn_args {
   int32_t causal;             /* 1: query row s reads tokens <= seq_len - q_len + s    */
   int32_t max_seq_len;        /* host-side upper bound of seq_lens (sizes the grid)    */
   int32_t partition_tokens;   /* context split size per workgroup, multiple of 32; 0 = auto   */
-  float scale;                /* softmax scale, reference uses 1/sqrt(head_dim)        */
+  float scale;                /* softmax scale (> 0), reference uses 1/sqrt(head_dim)  */
   void* workspace;            /* device scratch, >= pace_paged_attn_workspace_bytes()  */
   size_t workspace_bytes;
   /* Optional fused append (NULL = off).  The last n_new (1..32) tokens of every sequence, i.e.
