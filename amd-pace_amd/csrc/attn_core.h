@@ -68,23 +68,16 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
-// Maximum of two values the compiler cannot prove canonical (matrix core results, values from
-// other lanes): fmaxf() would spend a quieting instruction on each operand first; the median with
-// +inf is the same maximum in one instruction.  A NaN operand gives an unspecified finite-or-NaN
-// result here, which is harmless: a row with a NaN score ends in NaN through the exponential
-// whatever its maximum is.
-__device__ __forceinline__ float max_raw(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, __builtin_inff()); }
-
 // Maximum over the four lanes (n, 0..3) that share query row n, left in all four.  The lane swaps
 // hand every lane the value 16 resp. 32 lanes away without a trip through LDS.
 __device__ __forceinline__ float row_max4(float v) {
   typedef unsigned v2u __attribute__((ext_vector_type(2)));
   const unsigned x = __float_as_uint(v);
   const v2u a = __builtin_amdgcn_permlane16_swap(x, x, false, false);
-  const float m1 = max_raw(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const float m1 = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
   const unsigned y = __float_as_uint(m1);
   const v2u b = __builtin_amdgcn_permlane32_swap(y, y, false, false);
-  return max_raw(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
 template <int D>
@@ -198,8 +191,8 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
           // when out of range, and propagates (like the reference) when in range.
         }
     }
-    float mx = fmaxf(fmaxf(max_raw(s[0][0], s[0][1]), max_raw(s[0][2], s[0][3])),
-                     fmaxf(max_raw(s[1][0], s[1][1]), max_raw(s[1][2], s[1][3])));
+    float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
     mx = row_max4(mx);
     const float m_old = st.m[qt];
     const float m_new = fmaxf(m_old, mx);

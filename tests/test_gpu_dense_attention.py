@@ -58,6 +58,12 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     (2, 2, 512, 64, 512, "rows-bf16"),      # one mask line per batch entry
     (1, 40, 256, 128, 256, "causal-bf16"),  # enough workgroups for two tiles per wave
     (1, 9, 100, 128, 40, None),             # no mask (C ABI; the torch op always passes one)
+    # 256 workgroups and more: two query tiles per wave
+    (2, 32, 512, 128, 72, "causal-bf16"),
+    (2, 32, 500, 64, 41, "causal-f32"),
+    (2, 32, 512, 64, 104, "causal-bf16"),
+    (2, 32, 512, 128, 50, None),
+    (1, 33, 1000, 128, 96, "heads-bf16"),   # one mask plane per head; head count off a multiple of 8
 ])
 def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     from oracle.attention_ref import causal_mask_4d
@@ -69,8 +75,14 @@ def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
         m = None
     elif mask.startswith("causal"):
         dt = torch.float32 if mask.endswith("f32") else torch.bfloat16
-        m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, dt)
+        if L >= S:
+            m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, dt)
+        else:  # more rows than keys: a banded finfo.min pattern that leaves every row something to read
+            band = (torch.arange(L)[None, :] + torch.arange(S)[:, None]) % 3 == 0
+            m = torch.zeros(B, 1, S, L, dtype=dt).masked_fill(band, torch.finfo(dt).min)
         m = m + _mask(13, (B, 1, S, L), dt) * (m == 0)  # a bias on the readable part as well
+    elif mask.startswith("heads"):
+        m = _mask(15, (B, N, S, L), torch.bfloat16)
     else:
         m = _mask(14, (B, 1, 1, L), torch.bfloat16)
     qd, kd, vd = q.to(device), k.to(device), v.to(device)
