@@ -36,8 +36,12 @@ Pinning status (what independent evidence fixes each function):
                        is **parity unpinned** by any reference test.
   * rope_ref.*         no reference test exists; complex multiplication in fp64,
                        rotation invariants, integer-bit emulation of the bf16
-                       roundings, transformers' inverse frequencies -- pinned,
-                       except the longrope row-selection rule: **parity unpinned**.
+                       roundings, transformers' inverse frequencies -- pinned.
+                       The longrope row-selection rule agrees with the installed
+                       transformers' rule on both sides of one point (largest id
+                       == original length), where the two differ and the
+                       reference is followed as written: that point is
+                       **parity unpinned**.
   * speculative_ref.*  brute force against "1 + longest common prefix" -- pinned.
   * paged_ref.*        row permutations of the pinned contiguous cache; checked
                        against ``DynamicKVCacheRef`` replay of surviving tokens.

@@ -23,8 +23,10 @@ round-to-nearest-even emulation of the bf16 steps written with integer bit
 operations, and for the scaled tables the inverse frequencies of the installed
 ``transformers.modeling_rope_utils`` (``linear``, ``dynamic``, ``llama3``,
 ``longrope``).  The ``longrope`` *row selection* of ``forward`` (offset by the
-original context length once any position exceeds it) has no such independent
-source: **parity unpinned** beyond reading the code.
+original context length once any position exceeds it) picks the factors that
+transformers' rule (``max id + 1`` exceeds the original length) picks, except
+for a batch whose largest id equals the original length; that single point
+follows the reference as written and is **parity unpinned**.
 """
 from __future__ import annotations
 

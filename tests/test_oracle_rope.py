@@ -196,3 +196,26 @@ def test_longrope_row_selection():
     assert torch.equal(rope_ref.longrope_rows(ids, 8), ids)
     ids2 = torch.tensor([[0, 1, 2], [7, 8, 9]])
     assert torch.equal(rope_ref.longrope_rows(ids2, 8), ids2 + 8)
+
+
+def test_longrope_selection_agrees_with_transformers_off_the_boundary():
+    """transformers switches to the long factors when ``max(position_ids) + 1`` exceeds the original
+    length (``dynamic_rope_update`` of modeling_rope_utils); the reference when any id exceeds it
+    (``rotary_embedding.py:381-385``).  The two rules agree except for a batch whose largest id is
+    exactly the original length: checked here on both sides of that single point, and at the point
+    the oracle follows the reference as written."""
+    D, orig, max_pos = 32, 64, 256
+    short = [1.0 + 0.01 * i for i in range(D // 2)]
+    long_ = [2.0 + 0.1 * i for i in range(D // 2)]
+    scaling = dict(rope_type="longrope", short_factor=short, long_factor=long_)
+    cos, sin, _, _ = rope_ref.cos_sin_tables(scaling, D, max_pos, 10000.0, original_max_position_embeddings=orig)
+    params = dict(rope_theta=10000.0, short_factor=short, long_factor=long_, factor=max_pos / orig,
+                  original_max_position_embeddings=orig)
+    for top in (3, orig - 1, orig + 1, max_pos - 1):
+        ids = torch.tensor([[0, 1, top]])
+        rows = rope_ref.longrope_rows(ids, orig)
+        f_hf, _ = _hf_inv_freq("longrope", params, D, max_pos, seq_len=top + 1)  # the library's choice for this batch
+        got = torch.atan2(sin[rows[0, 1]], cos[rows[0, 1]])                       # angle of position 1 = its frequency
+        torch.testing.assert_close(got, f_hf, rtol=1e-5, atol=1e-7)
+    # the one point where the rules differ: largest id == original length -> the reference stays short
+    assert torch.equal(rope_ref.longrope_rows(torch.tensor([[0, orig]]), orig), torch.tensor([[0, orig]]))
