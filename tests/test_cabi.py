@@ -87,6 +87,14 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"positions are required" in lib.pace_kv_last_error()
     assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 96, None) == -1
     assert b"head_dim 96 unsupported" in lib.pace_kv_last_error()
+    # paged attention: a scale that is not positive and finite is refused before the launch
+    pool = _native.PoolDesc(k=16, v=32, k_block_stride=4096, k_head_stride=2048, v_block_stride=4096, v_head_stride=2048,
+                            num_blocks=4, num_kv_heads=2, head_dim=128, block_size=16)
+    args = _native.PagedAttnArgs(q=16, q_stride_b=512, q_stride_h=128, q_stride_s=128, out=16, o_stride_b=512,
+                                 o_stride_h=128, o_stride_s=128, block_table=16, table_stride=4, seq_lens=16, batch=1,
+                                 num_q_heads=4, q_len=1, causal=1, max_seq_len=64, scale=0.0)
+    assert lib.pace_paged_attn_decode(ctypes.byref(pool), ctypes.byref(args), None) == -1
+    assert b"softmax scale must be positive and finite" in lib.pace_kv_last_error()
 
 
 def test_torch_op_is_defined_with_reference_schema_and_checks():
