@@ -49,7 +49,7 @@ struct PagedAttnParams {
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)
-  float mask_mul;     // 1 / softmax scale: additive mask values in units of the raw score products
+  float scale;        // softmax scale
   // Fused append: the last n_new tokens of every sequence are taken from k_new / v_new
   // (and written to the pool by this launch) instead of being read from the pool.
   const uint16_t* k_new;
@@ -65,6 +65,12 @@ struct PagedAttnParams {
 
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kLog2e = 1.4426950408889634f;
+// Additive mask values are held at -2^100: far below any score, so such a column weighs nothing
+// next to an unmasked one, yet finite, so that a row masked everywhere (finfo.min in every column)
+// still ends as the reference's uniform average instead of 0 / 0; and a power of two, so that
+// (value * log2(e)) is exact and equal values cancel exactly in the exponent.
+constexpr float kMaskFloor = -0x1p100f;
+constexpr uint32_t kMaskFloorBf16x2 = 0xf180f180u;  // the same value as a pair of bf16
 
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
@@ -89,15 +95,16 @@ struct UnitRegs {
 template <int D, int NQT>
 struct RowState {
   f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
-  float m[NQT];          // running max: of the raw score products while units are consumed,
-                         // in log2 units (x scale_log2) after finish_rows()
+  float m[NQT];          // running max while units are consumed: of the raw score products (no mask) or
+                         // of scale * product + mask (with a mask); in log2 units after finish_rows()
   float l[NQT];          // this lane's share of the running sum
   int limit[NQT];        // last readable token of the row (-1: row is padding)
   int64_t mask_off[NQT]; // element offset of the row's mask line
 };
 
 // Additive mask values of one unit fetched ahead of time by the caller: a[qt][c] belongs to token
-// t0 + 8g + c of query tile qt's row n (-inf where the mask has no such element).
+// t0 + 8g + c of query tile qt's row n, already held at kMaskFloor (anything where the mask has no
+// such element: those columns are cut off by the range check of a partial unit).
 template <int NQT>
 struct MaskRegs {
   float a[NQT][8];
@@ -155,7 +162,9 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
   }
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
-    // Scores stay in units of the raw products; the softmax scale enters once, in the exponent.
+    // Without a mask, scores stay in units of the raw products and the softmax scale enters once, in
+    // the exponent.  With one they are scale * product + mask in fp32, the reference's sum, with the
+    // mask value held at kMaskFloor.
     f32x4 s[2] = {sc[qt][0], sc[qt][1]};
     // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
     if (HAS_MASK) {
@@ -166,11 +175,11 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
         for (int i = 0; i < 4; ++i) {
           const int tok = mbase + 4 * t + i;
           if (MREG) {
-            s[t][i] = __builtin_fmaf(mregs.a[qt][4 * t + i], p.mask_mul, s[t][i]);
+            s[t][i] = __builtin_fmaf(s[t][i], p.scale, mregs.a[qt][4 * t + i]);
           } else if (tok < p.mask_len && st.limit[qt] >= 0) {
             const float add = p.mask_is_f32 ? static_cast<const float*>(p.mask)[st.mask_off[qt] + tok]
                                             : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]);
-            s[t][i] = __builtin_fmaf(add, p.mask_mul, s[t][i]);
+            s[t][i] = __builtin_fmaf(s[t][i], p.scale, fmaxf(add, kMaskFloor));
           } else {
             s[t][i] = kNegInf;
           }
@@ -197,15 +206,17 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     const float m_old = st.m[qt];
     const float m_new = fmaxf(m_old, mx);
     const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((m_old - m_use) * p.scale_log2);  // m_old = -inf -> 0
-    const float m_neg = -(m_use * p.scale_log2);
+    // exponent = (score - max) * c with c = log2(e) (masked: natural units) or scale * log2(e)
+    const float c = HAS_MASK ? kLog2e : p.scale_log2;
+    const float alpha = __builtin_amdgcn_exp2f((m_old - m_use) * c);  // m_old = -inf -> 0
+    const float m_neg = -(m_use * c);
     float psum = 0.f;
     f32x4 pr[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        pr[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], p.scale_log2, m_neg));
+        pr[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, m_neg));
         psum += pr[t][i];
       }
     st.m[qt] = m_new;
@@ -228,7 +239,7 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
 
 // After the last unit: complete the row sums over the four lanes of a row and express the running
 // max in log2 units, as the merges between waves and partitions expect it.
-template <int D, int NQT>
+template <int D, int NQT, bool HAS_MASK>
 __device__ __forceinline__ void finish_rows(RowState<D, NQT>& st, const PagedAttnParams& p) {
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
@@ -236,7 +247,7 @@ __device__ __forceinline__ void finish_rows(RowState<D, NQT>& st, const PagedAtt
     l += xor_lanes(l, 16);
     l += xor_lanes(l, 32);
     st.l[qt] = l;
-    st.m[qt] *= p.scale_log2;  // -inf stays -inf: the scale is positive
+    st.m[qt] *= HAS_MASK ? kLog2e : p.scale_log2;  // -inf stays -inf: the factor is positive
   }
 }
 

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
     const bool full = t0 + 32 <= L;
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, L, 0, full, g);
   }
-  finish_rows<D, NQT>(st, p);
+  finish_rows<D, NQT, HAS_MASK>(st, p);
   __syncthreads();  // every wave is done with its V stage; the space becomes the merge buffer
   float* merge_buf = reinterpret_cast<float*>(lds_raw);
   constexpr int ROW_F = D + 2;
@@ -181,6 +181,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
 // 16-byte aligned (L % 8 == 0): one 16-byte load per row and unit.
 // ---------------------------------------------------------------------------------
 constexpr int kCoopWaves = 4;
+
+// Unsigned minimum of two pairs of 16-bit values.  On bf16 bit patterns it holds negative values
+// at the negative value `b` (a larger pattern is a more negative number) and leaves positive
+// ones alone.
+__device__ __forceinline__ uint32_t min_u16x2(uint32_t a, uint32_t b) {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
 
 template <int D, int NQT, int MASK>
 __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_coop_kernel(
@@ -253,7 +261,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const int tok = 32 * u + 8 * g;  // L % 8 == 0: the eight values exist together or not at all
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) {
-        const u32x4 none = {0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u};  // -inf pairs
+        const u32x4 none = {0u, 0u, 0u, 0u};  // columns past the end: any value, the partial unit's range check cuts them off
         pre_m[qt] = tok < L ? *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p.mask) + st.mask_off[qt] + tok) : none;
       }
     } else if (MASK == 1) {
@@ -269,7 +277,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
             else
               a = bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok + c]);
           }
-          mnext.a[qt][c] = a;
+          mnext.a[qt][c] = fmaxf(a, kMaskFloor);
         }
     }
   };
@@ -282,7 +290,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     }
     if (MASK == 2) {
 #pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) cur_m[qt] = pre_m[qt];
+      for (int qt = 0; qt < NQT; ++qt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur_m[qt][e] = min_u16x2(pre_m[qt][e], kMaskFloorBf16x2);  // hold at the floor
     } else if (MASK == 1) {
       mcur = mnext;
     }
@@ -368,7 +378,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.base.out = static_cast<uint16_t*>(out);
   dp.base.mask = mask, dp.base.mask_is_f32 = mask_is_f32, dp.base.mask_len = L;
   dp.base.scale_log2 = scale * kLog2e;
-  dp.base.mask_mul = 1.0f / scale;
+  dp.base.scale = scale;
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;

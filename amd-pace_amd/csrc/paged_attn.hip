@@ -304,7 +304,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
 #ifdef PACE_PROBE_TIMING
   const long long pt2 = wall_clock64();
 #endif
-  finish_rows<D, NQT>(st, p);  // row sums over the lanes of a row, running max in log2 units
+  finish_rows<D, NQT, HAS_MASK>(st, p);  // row sums over the lanes of a row, running max in log2 units
 
   // Pairwise merge of the waves' states through LDS (fixed order: deterministic).
   if (NWT > 1) {
@@ -596,7 +596,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.causal = a->causal;
   p.part_tokens = part, p.max_parts = max_parts;
   p.scale_log2 = a->scale * kLog2e;
-  p.mask_mul = 1.0f / a->scale;
+  p.scale = a->scale;
   p.part_o = nullptr, p.part_ml = nullptr;
   p.k_new = static_cast<const uint16_t*>(a->k_new), p.v_new = static_cast<const uint16_t*>(a->v_new);
   p.n_sb = a->new_stride_b, p.n_sh = a->new_stride_h, p.n_st = a->new_stride_t;

@@ -64,6 +64,13 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     (2, 32, 512, 64, 104, "causal-bf16"),
     (2, 32, 512, 128, 50, None),
     (1, 33, 1000, 128, 96, "heads-bf16"),   # one mask plane per head; head count off a multiple of 8
+    # rows masked everywhere with finfo.min (the first S - L rows of a causal mask with more rows than
+    # keys; the pad rows of a left-padded batch look the same): the reference's softmax turns them into
+    # the plain average of V, in every kernel the op can take
+    (2, 32, 512, 128, 72, "causal-short-bf16"),
+    (1, 4, 100, 64, 41, "causal-short-f32"),
+    (2, 3, 20, 64, 8, "causal-short-bf16"),
+    (1, 2, 40, 128, 70, "rows-masked-bf16"),
 ])
 def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     from oracle.attention_ref import causal_mask_4d
@@ -73,9 +80,12 @@ def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     q = seeded_q(12, B, N, S, H)
     if mask is None:
         m = None
+    elif mask.startswith("rows-masked"):  # every third row masked everywhere, long enough for several waves
+        m = _mask(16, (B, 1, S, L), torch.bfloat16)
+        m[:, :, ::3, :] = torch.finfo(torch.bfloat16).min
     elif mask.startswith("causal"):
         dt = torch.float32 if mask.endswith("f32") else torch.bfloat16
-        if L >= S:
+        if L >= S or "short" in mask:
             m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, dt)
         else:  # more rows than keys: a banded finfo.min pattern that leaves every row something to read
             band = (torch.arange(L)[None, :] + torch.arange(S)[:, None]) % 3 == 0
