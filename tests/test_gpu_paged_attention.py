@@ -92,6 +92,14 @@ def test_additive_mask_path_matches_reference_semantics(device):
     rnd = torch.randn(1, 1, 1, L, generator=g)
     out = mha(q.to(device), pk, pv, attention_mask=rnd.to(device))
     assert_attention_close(out, sdpa_fp32(q, ke, ve, rnd), "random additive mask")
+    # multi-token step whose first rows see nothing but finfo.min (pad positions of a left-padded
+    # prompt): the reference's softmax makes them the plain average of V
+    S2 = 6
+    q2 = seeded_q(11, B, hkv * n_rep, S2, D)
+    m2 = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S2, L, torch.bfloat16)
+    m2[1, :, :2, :] = torch.finfo(torch.bfloat16).min
+    out = mha(q2.to(device), pk, pv, attention_mask=m2.to(device))
+    assert_attention_close(out, sdpa_fp32(q2, ke, ve, m2), "rows masked everywhere")
 
 
 def test_decode_invariant_to_physical_block_permutation(device):
