@@ -331,3 +331,91 @@ def test_plan_attention_single_round_batch_gets_even_partitions():
     # never splits below 256 tokens per partition
     _, parts, _ = st.plan_attention(np.array([300, 700]), 4736, 6144, slots=64)
     assert parts.numpy().tolist() == [1, 2]
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_cache_histories_keep_every_sequence_intact(seed):
+    """Random appends, rollbacks, evictions, compactions and beam forks driven the way PagedKVCache
+    drives them, with the pool emulated on the host (one tag per token, block copies applied as
+    planned): after every step the tokens read back through the table are each sequence's own
+    tokens in order, and the reference counts and the free list agree with the tables."""
+    from pace_mi355.llm.paged import BLOCK, PagedState
+
+    rng = np.random.default_rng(seed)
+    B, num_blocks = 4, 64
+    st = PagedState(B, 16 * BLOCK, num_blocks, torch.device("cpu"))
+    pool = np.full((num_blocks, BLOCK), -1, dtype=np.int64)
+    lens = np.zeros(B, dtype=np.int64)
+    model = [[] for _ in range(B)]
+    next_tag = 0
+
+    def copy_blocks(pairs):
+        if len(pairs):
+            assert not set(pairs[:, 0].tolist()) & set(pairs[:, 1].tolist())
+            pool[pairs[:, 1]] = pool[pairs[:, 0]]
+
+    def check():
+        refs = np.zeros(num_blocks, dtype=np.int64)
+        for b in range(B):
+            n = int(st.n_blocks[b])
+            assert n == (lens[b] + BLOCK - 1) // BLOCK or n >= (lens[b] + BLOCK - 1) // BLOCK
+            np.add.at(refs, st.table[b, :n], 1)
+            got = pool[st.table[b, :n]].reshape(-1)[: int(lens[b])].tolist()
+            assert got == model[b], f"sequence {b} reads {got[:8]}.. instead of {model[b][:8]}.."
+        assert np.array_equal(refs, st.allocator.refs)
+        free = st.allocator.free_ids()
+        assert len(set(free.tolist())) == len(free) and not refs[free].any()
+        assert len(free) + int((refs > 0).sum()) == num_blocks
+
+    for step in range(300):
+        op = rng.choice(["append", "append", "append", "truncate", "evict", "compact", "fork"])
+        if op == "append":
+            counts = rng.integers(0, 20, B)
+            need = sum(int((lens[b] + counts[b] + BLOCK - 1) // BLOCK - st.n_blocks[b]) for b in range(B)) + B  # + copies
+            if need > st.allocator.num_free or (lens + counts).max() > 16 * BLOCK:
+                continue
+            if st.tails_dirty:
+                copy_blocks(st.unshare_tails(lens))
+            st.ensure_capacity(lens + counts)
+            width = int(counts.max(initial=0))
+            if width:
+                slots = st.slots(lens, counts, width)
+                for b in range(B):
+                    for t in range(int(counts[b])):
+                        pool[slots[b, t] // BLOCK, slots[b, t] % BLOCK] = next_tag
+                        model[b].append(next_tag)
+                        next_tag += 1
+                    assert (slots[b, int(counts[b]):] == -1).all()
+            lens = lens + counts
+        elif op == "truncate":
+            remove = np.minimum(rng.integers(0, 24, B), lens)
+            lens = lens - remove
+            for b in range(B):
+                del model[b][int(lens[b]):]
+            if remove.any():
+                st.release_beyond(lens)
+                st.lengths_shrank()
+        elif op == "evict":
+            b = int(rng.integers(0, B))
+            n = int(st.n_blocks[b])
+            if n == 0:
+                continue
+            drop = sorted(set(rng.integers(0, n, rng.integers(1, 3)).tolist()))
+            keep = [t for j in range(n) if j not in drop for t in model[b][j * BLOCK:(j + 1) * BLOCK]]
+            lens = st.evict(b, drop, lens)
+            st.lengths_shrank()
+            model[b] = keep
+        elif op == "compact":
+            moves = st.plan_compaction()
+            copy_blocks(moves)
+            st.apply_moves(moves)
+            live = st.live_block_count()
+            used = np.unique(np.concatenate([st.table[b, : int(st.n_blocks[b])] for b in range(B)]))
+            assert used.size == live and (used.size == 0 or used.max() == live - 1)
+        else:
+            src = rng.integers(0, B, B).tolist()
+            st.fork(src)
+            lens = lens[src].copy()
+            model = [list(model[i]) for i in src]
+        check()
+    assert next_tag > 500  # the history really appended
