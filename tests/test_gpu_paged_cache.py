@@ -187,3 +187,58 @@ def test_manager_layers_share_block_table(device):
         assert_bits_equal(mgr[layer].key.dense(), rk, f"layer {layer} K")
         assert_bits_equal(mgr[layer].value.dense(), rv, f"layer {layer} V")
     assert mgr[0].state is mgr[1].state
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_histories_with_real_data(device, seed):
+    """A random run of uniform (fused) and ragged appends, rollbacks, evictions, compactions and beam
+    re-orderings: after every step the dense view equals the oracle's cache bit for bit, and decode
+    attention over it matches the oracle."""
+    B, H, n_rep, D = 4, 2, 4, 128
+    rng = np.random.default_rng(100 + seed)
+    cache = _paged(640, num_kv_heads=H, n_rep=n_rep, num_blocks=220)
+    model = RaggedCacheModel(B, H, D)
+    k, v = seeded_kv(400 + seed, B, H, 24, D)
+    cache.append_ragged(k.to(device), v.to(device), [24, 7, 16, 1])
+    model.append(k, v, [24, 7, 16, 1])
+    for step in range(40):
+        op = rng.choice(["uniform", "uniform", "ragged", "truncate", "evict", "compact", "reorder"])
+        if max(model.seq_lens()) > 560 and op in ("uniform", "ragged"):
+            op = "truncate"
+        if op == "uniform":  # what a decode / verify step does: held back and stored by the attention launch
+            T = int(rng.choice([1, 1, 4, 9, 33]))
+            k, v = seeded_kv(1000 * seed + 2 * step, B, H, T, D)
+            cache.update_cache(k.to(device), v.to(device), 2)
+            model.append(k, v)
+            q = seeded_q(1000 * seed + 2 * step + 1, B, H * n_rep, T, D)
+            assert_attention_close(cache.attend(q.to(device)), model.attention(q, n_rep), f"step {step} attention after {T}-token append")
+        elif op == "ragged":
+            T = int(rng.integers(1, 30))
+            counts = rng.integers(0, T + 1, size=B)
+            k, v = seeded_kv(1000 * seed + 2 * step, B, H, T, D)
+            cache.append_ragged(k.to(device), v.to(device), counts)
+            model.append(k, v, counts)
+        elif op == "truncate":
+            rem = [int(rng.integers(0, min(40, n + 1))) for n in model.seq_lens()]
+            cache.truncate(rem)
+            model.truncate(rem)
+        elif op == "evict":
+            b = int(rng.integers(0, B))
+            nb = (model.seq_lens()[b] + 15) // 16
+            if nb == 0:
+                continue
+            drop = sorted(set(rng.integers(0, nb, size=int(rng.integers(1, 4))).tolist()))
+            cache.evict_blocks(b, drop)
+            model.evict_blocks(b, drop, 16)
+        elif op == "compact":
+            cache.compact()
+        else:
+            idx = rng.integers(0, B, size=B).tolist()
+            cache.reorder(idx)
+            model.reorder(idx)
+        assert cache.lens.tolist() == model.seq_lens(), f"step {step} ({op})"
+        K, V = model.dense()
+        gk, gv = cache.gather(n_rep=1)
+        assert_bits_equal(gk, K, f"K after step {step} ({op})")
+        assert_bits_equal(gv, V, f"V after step {step} ({op})")
+    assert cache.cow_blocks_copied > 0
