@@ -7,7 +7,7 @@
 namespace pace_kv {
 
 // ---------------------------------------------------------------------------------
-// Dense bf16 attention with the same inner step: K and V are the reference's row-major
+// Up to 64 query rows per head (decode, verify).  K and V are the reference's row-major
 // [B][N][L][D] tensors.  K rows feed the first product directly (16 bytes of a row per
 // lane); V rows are staged per wave in LDS and read back token-minor for the second.
 // One workgroup of 4 waves per (batch, head, group of 16*NQT query rows); the waves split
