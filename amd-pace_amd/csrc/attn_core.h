@@ -38,6 +38,7 @@ struct PagedAttnParams {
   const void* mask;
   int32_t mask_is_f32;
   int32_t mask_len;
+  int32_t mask_vec;  // mask lines start on 16-byte boundaries (32 for fp32) and the length is a multiple of 8
   int64_t m_sb, m_ss;
   int32_t n_rep, q_len, num_q_heads;
   int32_t causal;
@@ -102,13 +103,73 @@ struct RowState {
   int64_t mask_off[NQT]; // element offset of the row's mask line
 };
 
-// Additive mask values of one unit fetched ahead of time by the caller: a[qt][c] belongs to token
-// t0 + 8g + c of query tile qt's row n, already held at kMaskFloor (anything where the mask has no
-// such element: those columns are cut off by the range check of a partial unit).
+// Unsigned minimum of two pairs of 16-bit values.  On bf16 bit patterns it holds negative values
+// at the negative value `b` (a larger pattern is a more negative number) and leaves positive
+// ones alone.
+__device__ __forceinline__ uint32_t min_u16x2(uint32_t a, uint32_t b) {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+
+// Additive mask values of one unit, fetched by the caller while the unit's K / V travel:
+// a[qt][c] belongs to token t0 + 8g + c of query tile qt's row n, held at kMaskFloor, and is -inf
+// where the mask has no such column.
 template <int NQT>
 struct MaskRegs {
   float a[NQT][8];
 };
+
+// Eight packed bf16 mask values -> MaskRegs line (held at the floor).
+__device__ __forceinline__ void mask_line_from_bf16x8(const u32x4 raw, float (&a)[8]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t w = min_u16x2(raw[e], kMaskFloorBf16x2);
+    a[2 * e] = bf16_bits_to_f32(w & 0xffffu);
+    a[2 * e + 1] = __uint_as_float(w & 0xffff0000u);
+  }
+}
+
+// Mask values of the unit at t0 for every query tile, read from p.mask (lines at mask_off[qt]).
+// ALIGNED: t0 is a multiple of 8, so that with p.mask_vec one 16-byte load serves a lane.
+template <int NQT, bool ALIGNED>
+__device__ __forceinline__ void load_mask_regs(MaskRegs<NQT>& mr, const PagedAttnParams& p, const int64_t (&mask_off)[NQT],
+                                               int t0, int g) {
+  const int base = t0 + 8 * g;
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    if (ALIGNED && p.mask_vec) {  // wave-uniform
+      const bool there = base < p.mask_len;  // the eight columns exist together or not at all
+      if (p.mask_is_f32) {
+        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+        if (there) {
+          const float* line = static_cast<const float*>(p.mask) + mask_off[qt] + base;
+          lo = *reinterpret_cast<const f32x4*>(line), hi = *reinterpret_cast<const f32x4*>(line + 4);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) mr.a[qt][c] = fmaxf(lo[c], kMaskFloor), mr.a[qt][4 + c] = fmaxf(hi[c], kMaskFloor);
+      } else {
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (there) raw = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p.mask) + mask_off[qt] + base);
+        mask_line_from_bf16x8(raw, mr.a[qt]);
+      }
+      if (!there) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) mr.a[qt][c] = kNegInf;
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        float v = kNegInf;
+        if (base + c < p.mask_len) {
+          const float x = p.mask_is_f32 ? static_cast<const float*>(p.mask)[mask_off[qt] + base + c]
+                                        : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[mask_off[qt] + base + c]);
+          v = fmaxf(x, kMaskFloor);
+        }
+        mr.a[qt][c] = v;
+      }
+    }
+  }
+}
 
 // First product of a unit: the scores of its 32 tokens against every query tile.  All of them are
 // issued before any softmax, so that the matrix cores work through them (and later through the
@@ -131,9 +192,9 @@ __device__ __forceinline__ void score_products(const u32x4 (&k)[2][D / 32], cons
 
 // Second half of a unit: masking, online softmax and the product with V.
 // FULL: every token of the unit exists and is readable by every query row (no masking code at all;
-// the caller decides once per unit, wave-uniformly).  MREG: the mask values come from `mregs`
-// instead of being loaded here.
-template <int D, int NQT, bool HAS_MASK, bool FULL, bool MREG = false>
+// the caller decides once per unit, wave-uniformly).  With HAS_MASK the unit's mask values come in
+// `mregs`.
+template <int D, int NQT, bool HAS_MASK, bool FULL>
 __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], const u32x4 (&v)[D / 16], RowState<D, NQT>& st,
                                                    const PagedAttnParams& p, int t0, int tok_end, int start, int g,
                                                    const MaskRegs<NQT>& mregs = MaskRegs<NQT>{}) {
@@ -168,26 +229,14 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     f32x4 s[2] = {sc[qt][0], sc[qt][1]};
     // lane (n, g): s[t][i] is the score of token t0 + 8g + 4t + i for query row n.
     if (HAS_MASK) {
-      const int mbase = t0 + 8 * g;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = mbase + 4 * t + i;
-          if (MREG) {
-            s[t][i] = __builtin_fmaf(s[t][i], p.scale, mregs.a[qt][4 * t + i]);
-          } else if (tok < p.mask_len && st.limit[qt] >= 0) {
-            const float add = p.mask_is_f32 ? static_cast<const float*>(p.mask)[st.mask_off[qt] + tok]
-                                            : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[st.mask_off[qt] + tok]);
-            s[t][i] = __builtin_fmaf(s[t][i], p.scale, fmaxf(add, kMaskFloor));
-          } else {
-            s[t][i] = kNegInf;
-          }
-        }
+        for (int i = 0; i < 4; ++i) s[t][i] = __builtin_fmaf(s[t][i], p.scale, mregs.a[qt][4 * t + i]);
     }
-    // With mask values handed in, a whole unit needs no range check: they are -inf where the mask
-    // has no element, and rows that are padding are never written.
-    if ((!full || HAS_MASK) && !(full && MREG)) {
+    // A whole unit needs no range check, masked or not: mask values are -inf where the mask has no
+    // column, and rows that are padding are never written.
+    if (!full) {
       // token t0 + 8g + c (c = 4t + i) is readable iff lo <= c <= hi, both relative to the lane's first token
       const int base = t0 + 8 * g;
       const int hi = min(st.limit[qt], tok_end - 1) - base, lo = start - base;
@@ -255,7 +304,7 @@ __device__ __forceinline__ void finish_rows(RowState<D, NQT>& st, const PagedAtt
 template <int D, int NQT, bool HAS_MASK, bool FULL>
 __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
                                                   RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
-                                                  int start, int g) {
+                                                  int start, int g, const MaskRegs<NQT>& mregs = MaskRegs<NQT>{}) {
 #ifdef PACE_PROBE_LOADS_ONLY
   {  // measurement aid: keep the loads, drop the arithmetic
     u32x4 x = {0u, 0u, 0u, 0u};
@@ -269,17 +318,17 @@ __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u3
 #endif
   f32x4 sc[NQT][2];
   score_products<D, NQT>(r.k, qreg, sc);
-  softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, r.v, st, p, t0, tok_end, start, g);
+  softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, r.v, st, p, t0, tok_end, start, g, mregs);
 }
 
 template <int D, int NQT, bool HAS_MASK>
 __device__ __forceinline__ void compute_unit(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
                                              RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
-                                             int start, bool full, int g) {
+                                             int start, bool full, int g, const MaskRegs<NQT>& mregs = MaskRegs<NQT>{}) {
   if (full)
-    compute_unit_impl<D, NQT, HAS_MASK, true>(r, qreg, st, p, t0, tok_end, start, g);
+    compute_unit_impl<D, NQT, HAS_MASK, true>(r, qreg, st, p, t0, tok_end, start, g, mregs);
   else
-    compute_unit_impl<D, NQT, HAS_MASK, false>(r, qreg, st, p, t0, tok_end, start, g);
+    compute_unit_impl<D, NQT, HAS_MASK, false>(r, qreg, st, p, t0, tok_end, start, g, mregs);
 }
 
 // A sequence of `len` tokens is cut into ceil(len / part_tokens) partitions of equal size

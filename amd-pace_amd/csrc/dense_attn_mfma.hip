@@ -74,8 +74,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
   const int u_begin = min(units, wave * per_wave);
   const int n_units = min(units, u_begin + per_wave) - u_begin;
   UnitRegs<D> buf;
+  MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
     const int t0 = 32 * (u_begin + uu);
+    if (HAS_MASK) load_mask_regs<NQT, true>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
     // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g.. (clamped rows are masked later).
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
     }
     __builtin_amdgcn_wave_barrier();
     const bool full = t0 + 32 <= L;
-    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, L, 0, full, g);
+    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, L, 0, full, g, mregs);
   }
   finish_rows<D, NQT, HAS_MASK>(st, p);
   __syncthreads();  // every wave is done with its V stage; the space becomes the merge buffer
@@ -181,14 +183,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
 // 16-byte aligned (L % 8 == 0): one 16-byte load per row and unit.
 // ---------------------------------------------------------------------------------
 constexpr int kCoopWaves = 4;
-
-// Unsigned minimum of two pairs of 16-bit values.  On bf16 bit patterns it holds negative values
-// at the negative value `b` (a larger pattern is a more negative number) and leaves positive
-// ones alone.
-__device__ __forceinline__ uint32_t min_u16x2(uint32_t a, uint32_t b) {
-  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-  return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
-}
 
 template <int D, int NQT, int MASK>
 __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_coop_kernel(
@@ -290,9 +284,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     }
     if (MASK == 2) {
 #pragma unroll
-      for (int qt = 0; qt < NQT; ++qt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) cur_m[qt][e] = min_u16x2(pre_m[qt][e], kMaskFloorBf16x2);  // hold at the floor
+      for (int qt = 0; qt < NQT; ++qt) cur_m[qt] = pre_m[qt];
     } else if (MASK == 1) {
       mcur = mnext;
     }
@@ -325,14 +317,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     }
     if (MASK == 2) {
 #pragma unroll
-      for (int qt = 0; qt < NQT; ++qt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          mcur.a[qt][2 * e] = bf16_bits_to_f32(cur_m[qt][e] & 0xffffu);
-          mcur.a[qt][2 * e + 1] = __uint_as_float(cur_m[qt][e] & 0xffff0000u);
-        }
+      for (int qt = 0; qt < NQT; ++qt) mask_line_from_bf16x8(cur_m[qt], mcur.a[qt]);
     }
-    softmax_and_output<D, NQT, HAS_MASK, FULL, HAS_MASK>(sc, vop, st, p, t0, L, 0, g, mcur);
+    softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, vop, st, p, t0, L, 0, g, mcur);
   };
   // Whole units in the loop, the partial last one (if any) after it: the loop body has one shape.
   const int whole = L / 32, units = (L + 31) / 32;
@@ -377,6 +364,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.base.q = static_cast<const uint16_t*>(q);
   dp.base.out = static_cast<uint16_t*>(out);
   dp.base.mask = mask, dp.base.mask_is_f32 = mask_is_f32, dp.base.mask_len = L;
+  dp.base.mask_vec = mask && L % 8 == 0 && aligned16(mask);
   dp.base.scale_log2 = scale * kLog2e;
   dp.base.scale = scale;
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
@@ -384,7 +372,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   const int tiles = (S + 15) / 16;
   if (tiles > 4) {
     // prefill-sized: rows of a head share its K / V through LDS
-    const int mode = !mask ? 0 : ((!mask_is_f32 && L % 8 == 0 && aligned16(mask)) ? 2 : 1);
+    const int mode = !mask ? 0 : ((dp.base.mask_vec && !mask_is_f32) ? 2 : 1);
     int cnqt = 2;
     dp.n_qgroups = (tiles + kCoopWaves * cnqt - 1) / (kCoopWaves * cnqt);
     // too few workgroups: halve their rows; so does the element-wise mask path at head_dim 128, whose

@@ -287,18 +287,22 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   if (FUSED) {
     if (wave == NW && n_new > 0 && part == n_parts - 1) {
       load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
+      MaskRegs<NQT> mnew;
+      if (HAS_MASK) load_mask_regs<NQT, false>(mnew, p, st.mask_off, pool_end, g);  // pool_end is any position
       if (qg == 0) write_new_tokens<D, ROPE>(p, b, kvh, pool_end, n_new, lane);
-      compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g);
+      compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g, mnew);
     }
   }
 #ifdef PACE_PROBE_TIMING
   const long long pt1 = wall_clock64();
 #endif
+  MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
     if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
-    const int t0 = tok_begin + 32 * uu;
+    const int t0 = tok_begin + 32 * uu;  // a multiple of 32: partitions and wave shares are whole units
+    if (HAS_MASK) load_mask_regs<NQT, true>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
-    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g);
+    compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
   }
 
 #ifdef PACE_PROBE_TIMING
@@ -446,8 +450,11 @@ struct Shape {
   int occ_max;  // 8: no limit; 2: with five waves per workgroup, one workgroup per compute unit
 };
 
-static Shape shape_for(int tiles, bool fused) {
+static Shape shape_for(int tiles, bool fused, bool masked = false) {
   if (tiles <= 1) return Shape{1, 4, 2, 8};
+  // An explicit mask costs eight more registers per tile (its values travel with the unit): no more
+  // than two tiles per wave then (four tiles with a mask spilled and ran at half the speed).
+  if (masked) return Shape{2, fused ? 3 : 4, 2, 8};
   // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit.
   // Four waves per workgroup (three streaming + the append wave when fused) keep two
   // workgroups on a compute unit.
@@ -498,7 +505,9 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   if (p.rope.cos) {  // never together with an explicit mask (checked by the caller)
     if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
   } else if (has_mask) {
-    if (fused) PACE_GO(true, true, false); else PACE_GO(true, false, false);
+    if constexpr (NQT <= 2) {  // shape_for() never asks for more tiles with a mask
+      if (fused) PACE_GO(true, true, false); else PACE_GO(true, false, false);
+    }
   } else {
     if (fused) PACE_GO(false, true, false); else PACE_GO(false, false, false);
   }
@@ -567,7 +576,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const int rows = a->q_len * n_rep;
   const int tiles = (rows + 15) / 16;
   const bool fused_req = a->k_new != nullptr;
-  const Shape sh = shape_for(tiles, fused_req);
+  const Shape sh = shape_for(tiles, fused_req, a->mask != nullptr);
   const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
   PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
                "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(tiles));
@@ -591,6 +600,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.table = a->block_table, p.table_stride = a->table_stride;
   p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.len_bias_dev = a->seq_len_bias_ptr, p.kv_start = a->kv_start;
   p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
+  p.mask_vec = a->mask && aligned16(a->mask) && a->mask_len % 8 == 0 &&
+               a->mask_stride_b % 8 == 0 && a->mask_stride_s % 8 == 0;
   p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
   p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;
   p.causal = a->causal;

@@ -184,12 +184,12 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-def row_groups(query_rows: int) -> int:
+def row_groups(query_rows: int, masked: bool = False) -> int:
     """Workgroups one (sequence, KV head, partition) needs for ``query_rows`` = q_len * n_rep rows:
     the library packs 16, 32, 48 or 64 rows per workgroup (one 16-row tile up to 16 rows, two for
-    17..32, four for 33..64, three beyond 64)."""
+    17..32, four for 33..64, three beyond 64; never more than two with an explicit mask)."""
     tiles = max(1, -(-int(query_rows) // 16))
-    per_group = 1 if tiles <= 1 else (2 if tiles == 2 else (4 if tiles <= 4 else 3))
+    per_group = 1 if tiles <= 1 else (2 if tiles == 2 or masked else (4 if tiles <= 4 else 3))
     return -(-tiles // per_group)
 
 

@@ -102,6 +102,37 @@ def test_additive_mask_path_matches_reference_semantics(device):
     assert_attention_close(out, sdpa_fp32(q2, ke, ve, m2), "rows masked everywhere")
 
 
+@pytest.mark.parametrize("L,mdt", [(160, torch.bfloat16), (160, torch.float32), (157, torch.bfloat16), (157, torch.float32)])
+@pytest.mark.parametrize("S", [1, 5, 12])
+def test_mask_forms_partitions_and_fused_append(device, L, mdt, S):
+    """Explicit masks through every way the kernel fetches them: whole 16-byte lines (length a multiple
+    of 8) or element by element, bf16 or fp32, with the context cut into several partitions, with two
+    query tiles per wave (12 tokens x 4 heads), and with the step's new tokens still held back, i.e.
+    read from the caller's tensors at a position that is no multiple of 8."""
+    from pace_mi355.llm import PagedKVCache
+    from pace_mi355.ops import MultiHeadAttention
+
+    B, hkv, n_rep, D = 2, 2, 4, 128
+    past = L - S
+    k, v = seeded_kv(31, B, hkv, L, D)
+    q = seeded_q(32, B, hkv * n_rep, S, D)
+    m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, mdt)
+    m[0, :, :, :9] = torch.finfo(mdt).min                      # a left-padded row of the batch
+    m = m + (torch.randn(B, 1, S, L, generator=torch.Generator().manual_seed(33)).to(mdt)) * (m == 0)
+    ref = sdpa_fp32(q, repeat_kv(k, n_rep), repeat_kv(v, n_rep), m)
+    mha = MultiHeadAttention(dtype=torch.bfloat16)
+    for fuse in (True, False):
+        cache = PagedKVCache(256, num_kv_heads=hkv, n_rep=n_rep)
+        cache.partition_tokens = 64
+        cache.fuse_append = fuse
+        cache.update_cache(k[:, :, :past].to(device), v[:, :, :past].to(device), 2)
+        cache.attend(seeded_q(34, B, hkv * n_rep, 1, D).to(device))  # flushes the prefill
+        pk, pv = cache.update_cache(k[:, :, past:].to(device), v[:, :, past:].to(device), 2)
+        assert (cache._pending is not None) == fuse
+        out = mha(q.to(device), pk, pv, attention_mask=m.to(device))
+        assert_attention_close(out, ref, f"L={L} {mdt} S={S} fused={fuse}")
+
+
 def test_decode_invariant_to_physical_block_permutation(device):
     """Same logical cache, different physical block ids (via free-list history) -> same bits out."""
     B, hkv, n_rep, D, lens = 2, 2, 4, 128, [300, 123]
