@@ -38,7 +38,6 @@ struct PagedAttnParams {
   const void* mask;
   int32_t mask_is_f32;
   int32_t mask_len;
-  int32_t mask_vec;  // mask lines start on 16-byte boundaries (32 for fp32) and the length is a multiple of 8
   int64_t m_sb, m_ss;
   int32_t n_rep, q_len, num_q_heads;
   int32_t causal;
@@ -129,32 +128,34 @@ __device__ __forceinline__ void mask_line_from_bf16x8(const u32x4 raw, float (&a
   }
 }
 
+// 16 bytes from an address that is only element-aligned (mask lines start wherever the caller's
+// row length puts them; the hardware takes unaligned multi-dword loads).
+__device__ __forceinline__ u32x4 load16_unaligned(const void* p) {
+  u32x4 r;
+  __builtin_memcpy(&r, p, 16);
+  return r;
+}
+
 // Mask values of the unit at t0 for every query tile, read from p.mask (lines at mask_off[qt]).
-// ALIGNED: t0 is a multiple of 8, so that with p.mask_vec one 16-byte load serves a lane.
-template <int NQT, bool ALIGNED>
+// A lane whose eight columns all exist takes them in one 16-byte load (two for fp32); the lanes at
+// the end of a line whose length is no multiple of 8 go element by element.
+template <int NQT>
 __device__ __forceinline__ void load_mask_regs(MaskRegs<NQT>& mr, const PagedAttnParams& p, const int64_t (&mask_off)[NQT],
                                                int t0, int g) {
   const int base = t0 + 8 * g;
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
-    if (ALIGNED && p.mask_vec) {  // wave-uniform
-      const bool there = base < p.mask_len;  // the eight columns exist together or not at all
+    if (base + 8 <= p.mask_len) {
       if (p.mask_is_f32) {
-        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
-        if (there) {
-          const float* line = static_cast<const float*>(p.mask) + mask_off[qt] + base;
-          lo = *reinterpret_cast<const f32x4*>(line), hi = *reinterpret_cast<const f32x4*>(line + 4);
+        const float* line = static_cast<const float*>(p.mask) + mask_off[qt] + base;
+        const u32x4 lo = load16_unaligned(line), hi = load16_unaligned(line + 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          mr.a[qt][c] = fmaxf(__uint_as_float(lo[c]), kMaskFloor);
+          mr.a[qt][4 + c] = fmaxf(__uint_as_float(hi[c]), kMaskFloor);
         }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) mr.a[qt][c] = fmaxf(lo[c], kMaskFloor), mr.a[qt][4 + c] = fmaxf(hi[c], kMaskFloor);
       } else {
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (there) raw = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p.mask) + mask_off[qt] + base);
-        mask_line_from_bf16x8(raw, mr.a[qt]);
-      }
-      if (!there) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) mr.a[qt][c] = kNegInf;
+        mask_line_from_bf16x8(load16_unaligned(static_cast<const uint16_t*>(p.mask) + mask_off[qt] + base), mr.a[qt]);
       }
     } else {
 #pragma unroll

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
   MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
     const int t0 = 32 * (u_begin + uu);
-    if (HAS_MASK) load_mask_regs<NQT, true>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
+    if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
     // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g.. (clamped rows are masked later).
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -179,8 +179,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
 // the current one is consumed) and read back by every wave in operand order: K rows directly,
 // V token-minor through the LDS transpose read.  No merge: a row's softmax state never leaves
 // its wave.  Mask values of the next unit are fetched along with it.
-// MASK: 0 none, 1 element-wise loads (any mask dtype / alignment), 2 bf16 mask whose rows are
-// 16-byte aligned (L % 8 == 0): one 16-byte load per row and unit.
+// MASK: 0 none, 1 fp32 mask (element-wise loads), 2 bf16 mask: one 16-byte load per row and unit
+// (unaligned where the row length makes it so).
 // ---------------------------------------------------------------------------------
 constexpr int kCoopWaves = 4;
 
@@ -252,11 +252,19 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
     }
     if (MASK == 2) {
-      const int tok = 32 * u + 8 * g;  // L % 8 == 0: the eight values exist together or not at all
+      const int tok = 32 * u + 8 * g;
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) {
-        const u32x4 none = {0u, 0u, 0u, 0u};  // columns past the end: any value, the partial unit's range check cuts them off
-        pre_m[qt] = tok < L ? *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p.mask) + st.mask_off[qt] + tok) : none;
+        const uint16_t* line = static_cast<const uint16_t*>(p.mask) + st.mask_off[qt];
+        if (tok + 8 <= L) {
+          pre_m[qt] = load16_unaligned(line + tok);
+        } else {  // the end of a line whose length is no multiple of 8 (columns past it: any value, cut off later)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t lo = tok + 2 * e < L ? line[tok + 2 * e] : 0u, hi = tok + 2 * e + 1 < L ? line[tok + 2 * e + 1] : 0u;
+            pre_m[qt][e] = lo | (hi << 16);
+          }
+        }
       }
     } else if (MASK == 1) {
       const int tok = 32 * u + 8 * g;
@@ -364,7 +372,6 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.base.q = static_cast<const uint16_t*>(q);
   dp.base.out = static_cast<uint16_t*>(out);
   dp.base.mask = mask, dp.base.mask_is_f32 = mask_is_f32, dp.base.mask_len = L;
-  dp.base.mask_vec = mask && L % 8 == 0 && aligned16(mask);
   dp.base.scale_log2 = scale * kLog2e;
   dp.base.scale = scale;
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
@@ -372,7 +379,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   const int tiles = (S + 15) / 16;
   if (tiles > 4) {
     // prefill-sized: rows of a head share its K / V through LDS
-    const int mode = !mask ? 0 : ((dp.base.mask_vec && !mask_is_f32) ? 2 : 1);
+    const int mode = !mask ? 0 : (mask_is_f32 ? 1 : 2);
     int cnqt = 2;
     dp.n_qgroups = (tiles + kCoopWaves * cnqt - 1) / (kCoopWaves * cnqt);
     // too few workgroups: halve their rows; so does the element-wise mask path at head_dim 128, whose

@@ -288,7 +288,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     if (wave == NW && n_new > 0 && part == n_parts - 1) {
       load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
       MaskRegs<NQT> mnew;
-      if (HAS_MASK) load_mask_regs<NQT, false>(mnew, p, st.mask_off, pool_end, g);  // pool_end is any position
+      if (HAS_MASK) load_mask_regs<NQT>(mnew, p, st.mask_off, pool_end, g);  // pool_end is any position
       if (qg == 0) write_new_tokens<D, ROPE>(p, b, kvh, pool_end, n_new, lane);
       compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g, mnew);
     }
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   for (int uu = 0; uu < n_units; ++uu) {
     if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const int t0 = tok_begin + 32 * uu;  // a multiple of 32: partitions and wave shares are whole units
-    if (HAS_MASK) load_mask_regs<NQT, true>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
+    if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
   }
@@ -600,8 +600,6 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.table = a->block_table, p.table_stride = a->table_stride;
   p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.len_bias_dev = a->seq_len_bias_ptr, p.kv_start = a->kv_start;
   p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
-  p.mask_vec = a->mask && aligned16(a->mask) && a->mask_len % 8 == 0 &&
-               a->mask_stride_b % 8 == 0 && a->mask_stride_s % 8 == 0;
   p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
   p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;
   p.causal = a->causal;

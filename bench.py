@@ -262,12 +262,18 @@ def wl_decode_8b(torch, dev, args):
         from pace_mi355.ops import MultiHeadAttention
 
         mha = MultiHeadAttention(dtype=torch.bfloat16)
+        # --mask: the call exactly as the reference's models make it (llama.py:151-165): K/V arrive
+        # expanded by repeat_kv, and the additive [B,1,1,L] mask of the step is passed along
+        n_rep = hq // hkv
+        ka, va = (k1.repeat_interleave(n_rep, dim=1), v1.repeat_interleave(n_rep, dim=1)) if args.mask else (k1, v1)
+        mask_all = torch.zeros(B, 1, 1, ctx + 64 + args.steps + args.warmup, device=dev, dtype=torch.bfloat16)
+        keep.extend([ka, va, mask_all])
 
         def step(ev=None):
-            pk, pv = cache.update_cache(k1, v1, 2)  # the context grows by one token per step on this path
+            pk, pv = cache.update_cache(ka, va, 2)  # the context grows by one token per step on this path
             if ev:
                 ev[0].record()
-            mha(q, pk, pv)
+            mha(q, pk, pv, attention_mask=mask_all[..., : cache.seq_len] if args.mask else None)
             if ev:
                 ev[1].record()
     else:
@@ -296,7 +302,8 @@ def wl_decode_8b(torch, dev, args):
         dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline("paged_attn_kernel<128,1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
                  {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
-        {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct")})
+        {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct"),
+         "mask": bool(args.mask and args.path == "api")})
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
@@ -536,6 +543,9 @@ def main() -> int:
                          "MultiHeadAttention")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mask", action="store_true",
+                    help="decode-8b, api path: pass repeat_kv-expanded K/V and the step's additive mask, as the reference's "
+                         "models call the cache and the attention operator")
     ap.add_argument("--rope", action="store_true",
                     help="decode-8b, direct path: q and k arrive un-rotated and the rotary embedding rides in the launch "
                          "(with --no-fuse: in the append launch)")
