@@ -172,6 +172,25 @@ __device__ __forceinline__ void load_mask_regs(MaskRegs<NQT>& mr, const PagedAtt
   }
 }
 
+// A unit can be left out altogether when it cannot change any row of the wave: every mask value
+// in it is at the floor (weight exactly 0 next to any real score) and every row has already met a
+// real score -- the upper triangle of a causal mask, which is half of a prefill.  Rows that have
+// met nothing but floor values so far still need the unit (they may end as a uniform average).
+// Wave-uniform.
+template <int D, int NQT>
+__device__ __forceinline__ bool unit_is_masked_out(const MaskRegs<NQT>& mr, const RowState<D, NQT>& st) {
+  bool out = true;
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float top = mr.a[qt][0];
+#pragma unroll
+    for (int c = 1; c < 8; ++c) top = fmaxf(top, mr.a[qt][c]);
+    // rows that are padding are never written: whatever their mask line holds does not matter
+    out = out && (st.limit[qt] < 0 || (top <= kMaskFloor && st.m[qt] > 0.5f * kMaskFloor));
+  }
+  return __all(out);
+}
+
 // First product of a unit: the scores of its 32 tokens against every query tile.  All of them are
 // issued before any softmax, so that the matrix cores work through them (and later through the
 // previous tile's second product) while the vector unit does a tile's softmax.

@@ -304,6 +304,11 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // only once the score products are issued, into the registers the K rows leave.
   auto unit = [&](int cur, int t0, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
+    if (MASK == 2) {
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) mask_line_from_bf16x8(cur_m[qt], mcur.a[qt]);
+    }
+    if (HAS_MASK && unit_is_masked_out<D, NQT>(mcur, st)) return;  // e.g. above the diagonal of a causal mask
     u32x4 kop[2][KK], vop[MT];
     // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g ..
     const int r0 = 8 * (n >> 2) + (n & 3);
@@ -322,10 +327,6 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const tr_v4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 4 * VROW + 16 * j));
       const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
       vop[j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
-    }
-    if (MASK == 2) {
-#pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) mask_line_from_bf16x8(cur_m[qt], mcur.a[qt]);
     }
     softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, vop, st, p, t0, L, 0, g, mcur);
   };

@@ -298,9 +298,11 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
 #endif
   MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
-    if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const int t0 = tok_begin + 32 * uu;  // a multiple of 32: partitions and wave shares are whole units
-    if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
+    // The mask values go first, so that they are back before the unit's K / V: the wait for those
+    // is then the only one, as without a mask.
+    if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);
+    if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
   }
