@@ -204,7 +204,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // Workgroups are dealt to the eight XCDs in turn: keep all row groups of one (batch, head) on
   // one XCD, so that its K / V enter a single L2.
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int pair = (slot / dp.n_qgroups) * 8 + xcd, rg = slot % dp.n_qgroups;
+  // Row groups from the last to the first: under a causal mask the later rows read more keys, and
+  // the longest workgroups of a head should not be the last ones to start.
+  const int pair = (slot / dp.n_qgroups) * 8 + xcd, rg = dp.n_qgroups - 1 - slot % dp.n_qgroups;
   if (pair >= dp.B * dp.N) return;  // uniform over the workgroup
   const int b = pair / dp.N, head = pair % dp.N;
   const int L = dp.L, S = dp.S;
@@ -330,8 +332,73 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     }
     softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, vop, st, p, t0, L, 0, g, mcur);
   };
+  // Units past the last one that matters to any row of the workgroup are not walked at all: with a
+  // bf16 mask every wave first looks from the end of its rows' mask lines backwards for the last
+  // value above the floor (several units per round trip), until each of its rows has shown one; a
+  // row that shows none (masked everywhere: it ends as the average of V) keeps every unit.  What lies
+  // past the workgroup's last such unit weighs exactly 0 for rows that have all met a real score by
+  // then: the upper triangle of a causal mask, half of a prefill.
+  int units = (L + 31) / 32;
+  if (MASK == 2) {
+    __shared__ int last_needed[kCoopWaves];
+    constexpr int ROUND = 4;  // units looked at per round trip (16 measured slower: the volume counts, not the trips)
+    int mine = -1;            // last unit in which this lane's columns of a (real) row hold a value above the floor
+    bool shown[NQT];
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) shown[qt] = false;
+    bool open_rows = wave_has_rows;
+    for (int top = units - 1; top >= 0 && open_rows; top -= ROUND) {
+      u32x4 raw[ROUND][NQT];
+#pragma unroll
+      for (int r = 0; r < ROUND; ++r) {
+        const int tok = 32 * max(top - r, 0) + 8 * g;
+#pragma unroll
+        for (int qt = 0; qt < NQT; ++qt) {
+          const uint16_t* line = static_cast<const uint16_t*>(p.mask) + st.mask_off[qt];
+          if (tok + 8 <= L) {
+            raw[r][qt] = load16_unaligned(line + tok);
+          } else {  // columns that do not exist count as masked
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t lo = tok + 2 * e < L ? line[tok + 2 * e] : 0xffffu, hi = tok + 2 * e + 1 < L ? line[tok + 2 * e + 1] : 0xffffu;
+              raw[r][qt][e] = lo | (hi << 16);
+            }
+          }
+        }
+      }
+      bool all_shown = true;
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) {
+        int row_last = -1;
+#pragma unroll
+        for (int r = ROUND - 1; r >= 0; --r) {  // ascending unit index: the largest hit wins
+          const uint32_t w = min_u16x2(min_u16x2(raw[r][qt][0], raw[r][qt][1]), min_u16x2(raw[r][qt][2], raw[r][qt][3]));
+          const bool above = min(w & 0xffffu, w >> 16) < (kMaskFloorBf16x2 & 0xffffu);
+          if (above && top - r >= 0 && st.limit[qt] >= 0) row_last = max(row_last, top - r);
+        }
+        mine = max(mine, row_last);
+        // the row's four lanes (n, 0..3) look at different columns: it has shown a value if any of them has
+        int any = row_last >= 0 || shown[qt];
+        any |= __shfl_xor(any, 16, 64);
+        any |= __shfl_xor(any, 32, 64);
+        shown[qt] = any != 0;
+        all_shown = all_shown && (st.limit[qt] < 0 || shown[qt]);
+      }
+      open_rows = !__all(all_shown);
+    }
+    int wave_last = open_rows ? units - 1 : mine;  // a row never showed a value: keep everything
+#pragma unroll
+    for (int off = 1; off < 64; off *= 2) wave_last = max(wave_last, __shfl_xor(wave_last, off, 64));
+    if (!wave_has_rows) wave_last = -1;
+    if (lane == 0) last_needed[wave] = wave_last;
+    __syncthreads();
+    int wg_last = last_needed[0];
+#pragma unroll
+    for (int w = 1; w < kCoopWaves; ++w) wg_last = max(wg_last, last_needed[w]);
+    units = __builtin_amdgcn_readfirstlane(min(units, wg_last + 1));
+  }
   // Whole units in the loop, the partial last one (if any) after it: the loop body has one shape.
-  const int whole = L / 32, units = (L + 31) / 32;
+  const int whole = min(L / 32, units);
   fetch(0);
   park(0);
   __syncthreads();
