@@ -133,6 +133,45 @@ def test_mask_forms_partitions_and_fused_append(device, L, mdt, S):
         assert_attention_close(out, ref, f"L={L} {mdt} S={S} fused={fuse}")
 
 
+@pytest.mark.parametrize("kind", ["causal", "left-padded", "row-masked-everywhere", "window", "real-only-past-the-end"])
+def test_prefill_sized_masked_launch_leaves_out_only_what_weighs_nothing(device, kind):
+    """More than 64 query rows per KV head with an explicit mask: the kernel looks over the mask and
+    does not walk the units at the end of a wave's share that it rules out -- unless a row has no
+    readable real value anywhere (it must end as the average of V).  Results must not depend on it."""
+    from pace_mi355.llm import PagedKVCache
+
+    B, hkv, n_rep, D, L, S = 2, 2, 4, 128, 700, 300
+    k, v = seeded_kv(41, B, hkv, L, D)
+    q = seeded_q(42, B, hkv * n_rep, S, D)
+    dt = torch.bfloat16
+    m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, dt)
+    cols = torch.arange(L)
+    Lm = L
+    if kind == "left-padded":
+        m[1, :, :, :150] = torch.finfo(dt).min           # 150 pad columns: the forward look has to go past them
+    elif kind == "row-masked-everywhere":
+        m[0, :, 17, :] = torch.finfo(dt).min             # one row with nothing to read: nothing may be left out around it
+    elif kind == "window":                               # sliding window: masked units on both sides of a band
+        rows = torch.arange(S)[:, None] + (L - S)
+        m = torch.zeros(B, 1, S, L, dtype=dt).masked_fill((cols[None, :] > rows) | (cols[None, :] < rows - 100), torch.finfo(dt).min)
+    elif kind == "real-only-past-the-end":               # mask wider than the cache: zeros beyond the sequence must not count
+        Lm = L + 64
+        wide = torch.full((B, 1, S, Lm), torch.finfo(dt).min, dtype=dt)
+        wide[..., :L] = m
+        wide[0, :, 5, :] = torch.finfo(dt).min
+        wide[0, :, 5, L:] = 0.0                           # row 5 of sequence 0 reads nothing it has: average of V
+        m = wide
+    bias = torch.randn(B, 1, S, Lm, generator=torch.Generator().manual_seed(43)).to(dt)
+    m = m + bias * (m == 0)
+    ref = sdpa_fp32(q, repeat_kv(k, n_rep), repeat_kv(v, n_rep), m[..., :L].contiguous())
+    for partition in (0, 128):
+        cache = PagedKVCache(L + 64, num_kv_heads=hkv, n_rep=n_rep)
+        cache.partition_tokens = partition
+        cache.update_cache(k.to(device), v.to(device), 2)
+        out = cache.attend(q.to(device), m.to(device))
+        assert_attention_close(out, ref, f"{kind} partition={partition}")
+
+
 def test_decode_invariant_to_physical_block_permutation(device):
     """Same logical cache, different physical block ids (via free-list history) -> same bits out."""
     B, hkv, n_rep, D, lens = 2, 2, 4, 128, [300, 123]
