@@ -58,6 +58,10 @@ struct PagedAttnParams {
   int32_t n_new;
   float* part_o;      // [B][Hq][S][max_parts][D]
   float* part_ml;     // [B][Hq][S][max_parts][2]  (running max in log2 units, sum)
+  // Optional, prefill-sized launches with an explicit mask: per (sequence, query token) the last
+  // column the row can read whose mask value is above the floor, -1 if there is none (written by
+  // mask_row_last_kernel just before the attention launch).
+  const int32_t* row_last;
   // Optional rotary embedding (rope.cos == NULL: off): q rows are rotated as they are loaded,
   // the fused append's new keys before they are used and stored.  rotary_dim == D here.
   RopeDev rope;

@@ -192,13 +192,6 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   // needed, which halves the work of a prefill chunk (whole units are skipped, not masked).
   const int last_row = min(R, (qg + 1) * NQT * 16) - 1;
   const int group_end = (p.causal && last_row >= 0) ? len - S + last_row / p.n_rep + 1 : len;
-  const int tok_end = min(min(pool_end, part_begin + P), group_end);
-  // This wave's share of the partition's 32-token units.
-  const int part_units = max(0, (tok_end - part_begin + 31) / 32);
-  const int per_wave = (part_units + NW - 1) / NW;
-  const int u_begin = min(part_units, wave * per_wave);  // the extra wave (wave == NW) gets none
-  const int n_units = min(part_units, u_begin + per_wave) - u_begin;
-  const int tok_begin = part_begin + 32 * u_begin;
 
   // Query rows of this wave (B operand of the first product) and per-row limits.
   u32x4 qreg[NQT][KK];
@@ -255,6 +248,33 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   // the same in every lane (rows do not depend on the lane quarter): make that known, so that the
   // full / partial decision per unit is a scalar branch
   min_limit = __builtin_amdgcn_readfirstlane(min_limit);
+
+  int tok_end = min(min(pool_end, part_begin + P), group_end);
+  if (HAS_MASK && p.row_last) {
+    // Explicit mask on a prefill-sized launch: nothing past the last column any row of the group can
+    // use is needed (the diagonal of a causal mask) -- provided every row has a real score somewhere,
+    // so that the columns left out weigh exactly 0; a row masked everywhere must end as the average of
+    // V and keeps every column.  All waves of the workgroup hold the same rows and decide alike.
+    int last = -1;
+    bool real = true;
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      if (st.limit[qt] >= 0) {
+        const int v = p.row_last[(int64_t)b * S + row_s[qt]];
+        last = max(last, v);
+        real = real && v >= 0;
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o *= 2) last = max(last, __shfl_xor(last, o, 64));
+    if (__all(real)) tok_end = min(tok_end, __builtin_amdgcn_readfirstlane(last) + 1);
+  }
+  // This wave's share of the partition's 32-token units.
+  const int part_units = max(0, (tok_end - part_begin + 31) / 32);
+  const int per_wave = (part_units + NW - 1) / NW;
+  const int u_begin = min(part_units, wave * per_wave);  // the extra wave (wave == NW) gets none
+  const int n_units = min(part_units, u_begin + per_wave) - u_begin;
+  const int tok_begin = part_begin + 32 * u_begin;
 
   WaveBlockIds ids;
   {
@@ -409,6 +429,48 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     }
   }
 #endif
+}
+
+// One wave per (sequence, query token): the last column of the row's mask line, among those the
+// row can read ([kv_start, len) and inside the mask), that holds a value above the floor; -1 if none.
+// With it a workgroup knows where its rows stop needing the context -- the diagonal of a causal mask
+// -- and whether every row has a real score at all, without walking the mask itself.
+__global__ __launch_bounds__(64) void mask_row_last_kernel(const PagedAttnParams p, int32_t* out) {
+  const int row = blockIdx.x, S = p.q_len, b = row / S, s = row % S, lane = threadIdx.x;
+  const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
+  const int start = p.kv_start ? p.kv_start[b] : 0;
+  const int end = min(len, p.mask_len);
+  const int64_t off = (int64_t)b * p.m_sb + (int64_t)s * p.m_ss;
+  int last = -1;
+  for (int c0 = start + 8 * lane; c0 < end; c0 += 8 * 64) {
+    float a[8];
+    if (c0 + 8 <= end) {
+      if (p.mask_is_f32) {
+        const float* line = static_cast<const float*>(p.mask) + off + c0;
+        const u32x4 lo = load16_unaligned(line), hi = load16_unaligned(line + 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] = __uint_as_float(lo[c]), a[4 + c] = __uint_as_float(hi[c]);
+      } else {
+        const u32x4 raw = load16_unaligned(static_cast<const uint16_t*>(p.mask) + off + c0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[2 * e] = bf16_bits_to_f32(raw[e] & 0xffffu), a[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        a[c] = kNegInf;
+        if (c0 + c < end)
+          a[c] = p.mask_is_f32 ? static_cast<const float*>(p.mask)[off + c0 + c]
+                               : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[off + c0 + c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (a[c] > kMaskFloor) last = c0 + c;  // ascending: the largest column wins (NaN compares false: treated as masked)
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o *= 2) last = max(last, __shfl_xor(last, o, 64));
+  if (lane == 0) out[row] = last;
 }
 
 // Merge the partitions of one query row: out = sum_p 2^(m_p - M) o_p / sum_p 2^(m_p - M) l_p.
@@ -624,6 +686,17 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     p.part_o = static_cast<float*>(a->workspace);
     p.part_ml = p.part_o + rows_total * max_parts * pool->head_dim;
   }
+  p.row_last = nullptr;
+  int32_t* row_last = nullptr;
+  if (a->mask && rows > 64) {
+    // room behind the partials for one int per (sequence, query token)?  (pace_paged_attn_workspace_bytes*
+    // asks for it; a caller that sized its workspace otherwise simply goes without)
+    const size_t part_bytes = max_parts > 1 ? (size_t)a->batch * a->num_q_heads * a->q_len * max_parts * (pool->head_dim + 2) * sizeof(float) : 0;
+    const size_t at = (part_bytes + 15) & ~(size_t)15;
+    if (a->workspace && aligned16(a->workspace) && a->workspace_bytes >= at + (size_t)a->batch * a->q_len * sizeof(int32_t))
+      row_last = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + at);
+    p.row_last = row_last;
+  }
   p.num_kv_heads = pool->num_kv_heads;
   p.items = nullptr;
   p.seq_parts = a->seq_parts;
@@ -645,6 +718,11 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     launch_shape_sel.occ_max = 2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
+  if (row_last) {
+    PACE_REQUIRE((long long)a->batch * a->q_len < (1ll << 31), "%s: too many query rows", who);
+    hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
+    PACE_HIP_CHECK(hipGetLastError());
+  }
   const bool ok = pool->head_dim == 128 ? launch_shape<128>(launch_shape_sel, p, has_mask, s) : launch_shape<64>(launch_shape_sel, p, has_mask, s);
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   PACE_HIP_CHECK(hipGetLastError());
@@ -682,20 +760,29 @@ extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q
   return resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, q_len * (num_q_heads / num_kv_heads));
 }
 
+// Partials of every (row, partition) when a sequence is cut into several partitions, then (16-byte
+// aligned) one int per (sequence, query token) for launches of more than 64 query rows per KV head:
+// the per-row summary of an explicit mask (mask_row_last_kernel).
+static size_t workspace_need(int batch, int num_q_heads, int q_len, int head_dim, int max_parts, int rows) {
+  size_t need = max_parts > 1 ? (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float) : 0;
+  if (rows > 64) need = ((need + 15) & ~(size_t)15) + (size_t)batch * q_len * sizeof(int32_t);
+  return need;
+}
+
 extern "C" size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
                                                   int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {
   if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
   const int rows = q_len * (num_q_heads / num_kv_heads);
   const int part = resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, rows);
   const int max_parts = (max_seq_len + part - 1) / part;
-  if (max_parts <= 1) return 0;
-  return (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float);
+  return workspace_need(batch, num_q_heads, q_len, head_dim, max_parts, rows);
 }
 
 extern "C" size_t pace_paged_attn_workspace_bytes_for_parts(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
                                                             int32_t max_parts) {
-  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_parts <= 1) return 0;
-  return (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float);
+  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_parts < 1) return 0;
+  // rows per KV head are not known here: room for the per-row mask summary whenever the launch could be prefill-sized
+  return workspace_need(batch, num_q_heads, q_len, head_dim, max_parts, q_len * num_q_heads);
 }
 
 extern "C" int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {

@@ -238,7 +238,11 @@ int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int
                                          int32_t max_seq_len, int32_t partition_tokens,
                                          int32_t num_kv_heads);
 
-/* Scratch bytes the two entry points below need for these sizes (0 = none). */
+/* Scratch bytes the two entry points below need for these sizes (0 = none): the partial results
+ * of sequences cut into several partitions and, for launches of more than 64 query rows per KV
+ * head, one int32 per (sequence, query token) in which a launch with an explicit mask keeps a
+ * summary of the mask (the last column each row can use).  The partials are required; a workspace
+ * without room for the summary is accepted and the launch simply walks every column. */
 size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len,
                                        int32_t head_dim, int32_t max_seq_len,
                                        int32_t partition_tokens, int32_t num_kv_heads);
