@@ -172,6 +172,27 @@ def test_prefill_sized_masked_launch_leaves_out_only_what_weighs_nothing(device,
         assert_attention_close(out, ref, f"{kind} partition={partition}")
 
 
+def test_masked_prefill_without_room_for_the_mask_summary(device):
+    """The per-row mask summary is optional: a workspace without room for it (here: none at all) makes
+    the launch walk every column, with the same result."""
+    from pace_mi355.llm import PagedKVCache
+
+    B, hkv, n_rep, D, L, S = 2, 2, 4, 128, 400, 200
+    k, v = seeded_kv(51, B, hkv, L, D)
+    q = seeded_q(52, B, hkv * n_rep, S, D)
+    m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, torch.bfloat16)
+    ref = sdpa_fp32(q, repeat_kv(k, n_rep), repeat_kv(v, n_rep), m)
+    cache = PagedKVCache(L + 64, num_kv_heads=hkv, n_rep=n_rep)
+    cache.partition_tokens = 1024  # one partition per sequence: the partials need no workspace
+    cache.update_cache(k.to(device), v.to(device), 2)
+    with_summary = cache.attend(q.to(device), m.to(device))
+    plan = cache._plan
+    cache._plan = lambda *a: plan(*a)[:4] + (0,)  # same cut, no workspace
+    without = cache.attend(q.to(device), m.to(device))
+    assert_attention_close(with_summary, ref, "with the summary")
+    assert_attention_close(without, ref, "without the summary")
+
+
 def test_decode_invariant_to_physical_block_permutation(device):
     """Same logical cache, different physical block ids (via free-list history) -> same bits out."""
     B, hkv, n_rep, D, lens = 2, 2, 4, 128, [300, 123]
