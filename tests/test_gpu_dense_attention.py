@@ -1,4 +1,5 @@
 """GPU parity: torch.ops.pace.attention (dense op of the reference) against the oracle."""
+import numpy as np
 import pytest
 import torch
 
@@ -137,3 +138,47 @@ def test_operator_without_mask_and_noncontiguous_inputs(device):
     qt = q.transpose(1, 2).contiguous().transpose(1, 2)  # [B,H,S,D] view over [B,S,H,D] storage
     out2 = mha(qt.to(device), k.to(device), v.to(device))
     assert torch.allclose(out2.cpu(), sdpa_fp32(q, k, v), atol=1e-5, rtol=1e-5)
+
+
+def _random_mask(rng, kind, B, N, S, L, dt):
+    """Additive masks of the forms the kernels tell apart; finfo.min marks what is masked."""
+    lo = torch.finfo(dt).min
+    cols, rows = torch.arange(L)[None, :], torch.arange(S)[:, None]
+    heads = N if kind == "per-head" else 1
+    m = torch.zeros(B, heads, S, L, dtype=dt)
+    if kind in ("causal", "causal-left-padded", "per-head"):
+        m = m.masked_fill(cols > rows + (L - S), lo)          # S > L: the first rows read nothing at all
+    if kind == "causal-left-padded":
+        for b in range(B):
+            m[b, :, :, : int(rng.integers(0, max(1, L // 2)))] = lo
+    if kind == "window":
+        m = m.masked_fill((cols > rows + (L - S)) | (cols < rows + (L - S) - 40), lo)
+    if kind == "rows-masked":
+        m[:, :, :: int(rng.integers(2, 6)), :] = lo
+    if kind == "key-padding":                                  # [B,1,1,L]
+        m = torch.zeros(B, 1, 1, L, dtype=dt)
+        for b in range(B):
+            m[b, :, :, int(rng.integers(1, L + 1)):] = lo
+    bias = torch.randn(m.shape, generator=torch.Generator().manual_seed(int(rng.integers(1 << 30)))).to(dt)
+    return m + bias * (m == 0)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_dense_op_random_shapes_and_masks(device, seed):
+    """Seeded sweep over shapes and mask forms, in the spirit of the reference's property test
+    (tests/ops/test_sdpa.py:83-127): every kernel the op can take, ragged sizes, masks that leave
+    whole stretches (and sometimes whole rows) unreadable."""
+    rng = np.random.default_rng(1000 + seed)
+    kinds = ["random", "causal", "causal-left-padded", "window", "rows-masked", "per-head", "key-padding"]
+    for case in range(8):
+        B, N = int(rng.integers(1, 4)), int(rng.integers(1, 10))
+        S = int(rng.choice([1, 3, 8, 17, 40, 64, 65, 100, 130, 260]))
+        L = int(rng.choice([1, 7, 31, 32, 33, 64, 100, 129, 256, 300]))
+        H = int(rng.choice([64, 128, 128, 80]))
+        dt = torch.bfloat16
+        mdt = torch.bfloat16 if rng.random() < 0.7 else torch.float32
+        kind = kinds[int(rng.integers(len(kinds)))]
+        q, (k, v) = seeded_q(seed * 100 + case, B, N, S, H), seeded_kv(seed * 100 + case + 50, B, N, L, H)
+        m = _random_mask(rng, kind, B, N, S, L, mdt) if kind != "random" else _mask(case, (B, 1, S, L), mdt)
+        out = torch.ops.pace.attention(q.to(device), k.to(device), v.to(device), m.to(device), 0)
+        assert_attention_close(out, sdpa_fp32(q, k, v, m), f"seed {seed} case {case}: B{B} N{N} S{S} L{L} H{H} {kind} {mdt}")

@@ -378,3 +378,58 @@ def test_very_long_context_single_sequence(device):
     cache.update_cache(k1.to(device), v1.to(device), 2)   # fused 3-token verify on top
     model.append(k1, v1)
     assert_attention_close(cache.attend(q3.to(device)), model.attention(q3, 4), "70k verify")
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_paged_attention_random_batches_masks_and_partitions(device, seed):
+    """Seeded sweep: ragged lengths, query lengths on both sides of the kernel's tile limits, forced
+    partition sizes, with and without an explicit mask (random bias, causal, left padding), with the
+    step's tokens held back for the attention launch or appended first."""
+    from pace_mi355.llm import PagedKVCache
+
+    rng = np.random.default_rng(2000 + seed)
+    for case in range(6):
+        B = int(rng.integers(1, 5))
+        hkv, n_rep, D = int(rng.choice([1, 2, 4])), int(rng.choice([1, 4, 8])), int(rng.choice([64, 128]))
+        S = int(rng.choice([1, 2, 5, 8, 16, 24, 70]))
+        past = rng.integers(0, 400, size=B)
+        uniform = rng.random() < 0.5
+        if uniform:
+            past[:] = past[0]
+        lens = (past + S).tolist()
+        Lmax = max(lens)
+        tag = f"seed {seed} case {case}: B{B} hkv{hkv} rep{n_rep} D{D} S{S} lens{lens}"
+        k, v = seeded_kv(seed * 100 + case, B, hkv, Lmax, D)
+        q = seeded_q(seed * 100 + case + 50, B, hkv * n_rep, S, D)
+        cache = PagedKVCache(Lmax + 64, num_kv_heads=hkv, n_rep=n_rep)
+        cache.partition_tokens = int(rng.choice([0, 32, 128]))
+        cache.fuse_append = bool(rng.random() < 0.5)
+        model = RaggedCacheModel(B, hkv, D)
+        if past.max() > 0:
+            cache.append_ragged(k[:, :, : past.max()].to(device), v[:, :, : past.max()].to(device), past.tolist())
+            model.append(k[:, :, : past.max()], v[:, :, : past.max()], past.tolist())
+        kn, vn = seeded_kv(seed * 100 + case + 70, B, hkv, S, D)
+        cache.update_cache(kn.to(device), vn.to(device), 2)
+        model.append(kn, vn)
+        kind = str(rng.choice(["none", "bias", "causal", "left-padded"]))
+        if kind == "none" or not uniform:  # an explicit mask addresses columns by position: equal lengths only
+            out = cache.attend(q.to(device))
+            ref = model.attention(q, n_rep)
+        else:
+            L = lens[0]
+            mdt = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+            m = torch.zeros(B, 1, S, L, dtype=mdt)
+            if kind != "bias":
+                m = causal_mask_4d(torch.ones(B, L, dtype=torch.long), S, L, mdt)
+            if kind == "left-padded" and L > S + 2:
+                for b in range(B):
+                    m[b, :, :, : int(rng.integers(0, L - S))] = torch.finfo(mdt).min
+            m = m + torch.randn(m.shape, generator=torch.Generator().manual_seed(case)).to(mdt) * (m == 0)
+            out = cache.attend(q.to(device), m.to(device))
+            K, V = model.dense(n_rep)
+            ref = sdpa_fp32(q, K, V, m)
+            tag += f" mask {kind} {mdt}"
+        assert_attention_close(out, ref, tag)
+        gk, gv = cache.gather(n_rep=1)
+        Kd, Vd = model.dense()
+        assert torch.equal(gk.cpu(), Kd) and torch.equal(gv.cpu(), Vd), tag
