@@ -96,7 +96,7 @@ class FixedStep:
     """Direct C-ABI calls with metadata frozen at "T new tokens on top of the prefilled cache":
     the new tokens land on the same positions every step, so each step moves the same bytes."""
 
-    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True, rope=None):
+    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True, rope=None, mask=None):
         import numpy as np
         from pace_mi355 import _native as nat
 
@@ -118,6 +118,10 @@ class FixedStep:
                                                            self.out.stride(2))
         a.block_table, a.table_stride, a.seq_lens = self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr()
         a.kv_start, a.mask, a.causal = None, None, 1
+        if mask is not None:  # additive bf16 [B,1,S,L]: the mask alone decides what a row reads
+            self.mask = mask
+            a.mask, a.mask_dtype, a.mask_len, a.causal = mask.data_ptr(), nat.DTYPE_BF16, mask.shape[3], 0
+            a.mask_stride_b, a.mask_stride_s = mask.stride(0), mask.stride(2)
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         if partition == 0 and max_len > 1.5 * float(lens_after.mean()):  # same rule as PagedKVCache.attend
             partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
@@ -365,7 +369,13 @@ def wl_prefill(torch, dev, args):
     g = torch.Generator(device=dev).manual_seed(9)
     kd, vd = _randn_bf16(torch, (B, hkv, S, D), g, dev), _randn_bf16(torch, (B, hkv, S, D), g, dev)
     q = _randn_bf16(torch, (B, hq, S, D), g, dev)
-    step = FixedStep(torch, cache, q, kd, vd, args.partition, fused=False)
+    mask = None
+    if args.mask:  # the additive causal mask the reference's models pass along (llama.py:292-299), as a tensor
+        ctx = past + S
+        ar = torch.arange(ctx, device=dev)
+        mask = torch.zeros(B, 1, S, ctx, device=dev, dtype=torch.bfloat16)
+        mask.masked_fill_(ar[None, :] > ar[:S, None] + past, torch.finfo(torch.bfloat16).min)
+    step = FixedStep(torch, cache, q, kd, vd, args.partition, fused=False, mask=mask)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     # causal: row s of the chunk reads past + s + 1 tokens
     flops = 4.0 * B * hq * D * sum(past + s + 1 for s in range(S))
@@ -374,10 +384,11 @@ def wl_prefill(torch, dev, args):
     return result_line(
         args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
         "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
-        {"bound": "mfma", "kernel": "paged_attn_kernel<128,3,...> (prefill chunk)", "achieved": round(tflops, 1),
+        {"bound": "mfma", "kernel": "paged_attn_kernel<128,2,true,...> (prefill chunk, explicit mask)" if args.mask else "paged_attn_kernel<128,3,...> (prefill chunk)", "achieved": round(tflops, 1),
          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5),
-         "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)})
+         "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)},
+        {"mask": bool(args.mask)})
 
 
 def wl_dense_prefill(torch, dev, args):
@@ -550,7 +561,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--mask", action="store_true",
                     help="decode-8b, api path: pass repeat_kv-expanded K/V and the step's additive mask, as the reference's "
-                         "models call the cache and the attention operator")
+                         "models call the cache and the attention operator; prefill: pass the causal mask as a tensor")
     ap.add_argument("--rope", action="store_true",
                     help="decode-8b, direct path: q and k arrive un-rotated and the rotary embedding rides in the launch "
                          "(with --no-fuse: in the append launch)")
