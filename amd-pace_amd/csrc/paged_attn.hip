@@ -11,11 +11,21 @@
 
 namespace pace_kv {
 
+// 16 bytes of the cache.  ONCE (a kernel template argument: with both forms behind a run-time branch
+// the compiler merges the two arms and the hint is lost): nothing will read them again in this launch
+// (one group of query rows per sequence and KV head), so they are fetched non-temporally and leave the caches to what is
+// re-used; the decode step runs 10 % faster for it (186 -> 169 us).  With several row groups
+// (prefill) the later ones find K / V in L2 and the plain load is the faster one (778 vs 623 TFLOP/s).
+template <bool ONCE>
+__device__ __forceinline__ u32x4 load_kv16(const uint16_t* p) {
+  if (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return *reinterpret_cast<const u32x4*>(p);
+}
+
 // Issue the 16-byte loads of one 32-token unit.  ids: pool block ids of the
 // unit's two blocks (wave-uniform).
-template <int D>
-__device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n,
-                                          int g) {
+template <int D, bool ONCE>
+__device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n, int g) {
   // K: lane (n, g) supplies token 8*(n/4) + 4*tile + n%4 of the unit, i.e. token slot
   // n % 8 of slab tile `tile` in block A (n < 8) or B; dims 32*kk + 8g .. +8 are dim
   // chunk 4*kk + g.  A 16-lane quarter (fixed g) reads 128 contiguous bytes per block.
@@ -24,13 +34,13 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + t * (D * 8) + kk * 256);
+    for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = load_kv16<ONCE>(kp + t * (D * 8) + kk * 256);
   // V: lane (n, g) supplies dim 16j + n, tokens 8g..8g+7 of the unit: token half g & 1
   // of block A (g < 2) or B.  A 16-lane quarter reads 256 contiguous bytes.
   const int64_t voffA = (int64_t)idA * p.v_bs, voffB = (int64_t)idB * p.v_bs;
   const uint16_t* vp = p.vpool + ((g >= 2) ? voffB : voffA) + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
 #pragma unroll
-  for (int j = 0; j < D / 16; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(vp + j * 256);
+  for (int j = 0; j < D / 16; ++j) r.v[j] = load_kv16<ONCE>(vp + j * 256);
 }
 
 // The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
@@ -140,7 +150,7 @@ struct WaveBlockIds {
 // more wave per workgroup handles the step's new tokens (attends to them from the caller's
 // buffers and stores them into the pool), so that its dependent round trips overlap with the
 // streaming waves.  With ROPE, query rows and the new keys are rotated on their way in.
-template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED, bool ROPE>
+template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED, bool ROPE, bool ONCE>
 __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC_MAX))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
@@ -295,7 +305,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     // rotation is written out in both arms: after a join the wait for the (older) table loads
     // would have to assume the worst and cover the unit's loads as well.
     if (n_units > 0) {
-      load_unit<D>(buf, p, kvh, ids.get(0), ids.get(1), n, g);
+      load_unit<D, ONCE>(buf, p, kvh, ids.get(0), ids.get(1), n, g);
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);  // padding rows stay zero
       asm volatile("; query rows rotated, first unit in flight");  // keeps the two arms from being merged
@@ -322,7 +332,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     // The mask values go first, so that they are back before the unit's K / V: the wait for those
     // is then the only one, as without a mask.
     if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);
-    if (!ROPE || uu > 0) load_unit<D>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
+    if (!ROPE || uu > 0) load_unit<D, ONCE>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
   }
@@ -564,8 +574,18 @@ template <int D, int NQT, int NW, int OCC, int OCC_MAX>
 static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   const bool fused = p.n_new > 0;
   const unsigned blocks = (unsigned)p.total_items;
-#define PACE_GO(M_, F_, R_) \
-  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+  // K / V are read once per launch when one group of query rows covers a sequence's rows: always with one
+  // or four tiles per wave, never with three, either way with two.
+#define PACE_GO1(M_, F_, R_, O_) \
+  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_, O_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+#define PACE_GO(M_, F_, R_)                                                              \
+  do {                                                                                   \
+    if constexpr (NQT == 2) {                                                            \
+      if (p.n_qgroups == 1) PACE_GO1(M_, F_, R_, true); else PACE_GO1(M_, F_, R_, false); \
+    } else {                                                                             \
+      PACE_GO1(M_, F_, R_, NQT != 3);                                                    \
+    }                                                                                    \
+  } while (0)
   if (p.rope.cos) {  // never together with an explicit mask (checked by the caller)
     if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
   } else if (has_mask) {
@@ -575,6 +595,7 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   } else {
     if (fused) PACE_GO(false, true, false); else PACE_GO(false, false, false);
   }
+#undef PACE_GO1
 #undef PACE_GO
 }
 
