@@ -43,6 +43,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
+// Streaming accesses: 16 bytes that this launch touches once.  Fetched / stored non-temporally they
+// do not displace what the caches hold for re-use; on this GPU a pure stream runs about 10 % faster.
+__device__ __forceinline__ u32x4 load16_stream(const void* p) { return __builtin_nontemporal_load(static_cast<const u32x4*>(p)); }
+__device__ __forceinline__ void store16_stream(void* p, u32x4 v) { __builtin_nontemporal_store(v, static_cast<u32x4*>(p)); }
+
 // Element offsets inside one (block, head) slab of 16 tokens x D dims.
 // K slab  [tile 2][dim chunk D/8][token slot 8][dim 8]   with token -> (tile, slot):
 //         tile = (tok >> 2) & 1,  slot = ((tok >> 3) << 2) | (tok & 3)

@@ -22,7 +22,8 @@ struct DenseMfmaParams {
   int32_t n_qgroups;
 };
 
-template <int D, int NQT, bool HAS_MASK>
+// ONCE: one group of query rows per (batch, head), so K / V are read once and fetched non-temporally.
+template <int D, int NQT, bool HAS_MASK, bool ONCE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_mfma_kernel(const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
       const int tok = min(L - 1, t0 + 8 * (n >> 2) + 4 * t + (n & 3));
       const uint16_t* kp = kbase + (int64_t)tok * D + 8 * g;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = *reinterpret_cast<const u32x4*>(kp + kk * 32);
+      for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = ONCE ? load16_stream(kp + kk * 32) : *reinterpret_cast<const u32x4*>(kp + kk * 32);
     }
     // V: the unit's 32 rows go to this wave's LDS stage (coalesced 16-byte chunks) ...
     constexpr int CH = D / 8;  // chunks per row
@@ -92,7 +93,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void d
     for (int i = 0; i < 32 * CH / 64; ++i) {
       const int c = i * 64 + lane, r = c / CH, ch = c % CH;
       const int tok = min(L - 1, t0 + r);
-      *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = *reinterpret_cast<const u32x4*>(vbase + (int64_t)tok * D + ch * 8);
+      const uint16_t* vp = vbase + (int64_t)tok * D + ch * 8;
+      *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = ONCE ? load16_stream(vp) : *reinterpret_cast<const u32x4*>(vp);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
     __builtin_amdgcn_wave_barrier();
@@ -475,7 +477,9 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   if (blocks >= (1ll << 31)) return false;
   const dim3 grid((unsigned)blocks), block(256);
   const bool m = mask != nullptr;
-#define PACE_DENSE(D_, Q_, M_) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_>), grid, block, 0, stream, dp)
+  const bool once = dp.n_qgroups == 1;
+#define PACE_DENSE1(D_, Q_, M_, O_) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_>), grid, block, 0, stream, dp)
+#define PACE_DENSE(D_, Q_, M_) do { if (once) PACE_DENSE1(D_, Q_, M_, true); else PACE_DENSE1(D_, Q_, M_, false); } while (0)
   if (H == 128) {
     if (nqt == 2) { if (m) PACE_DENSE(128, 2, true); else PACE_DENSE(128, 2, false); }
     else { if (m) PACE_DENSE(128, 1, true); else PACE_DENSE(128, 1, false); }
@@ -483,6 +487,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
     if (nqt == 2) { if (m) PACE_DENSE(64, 2, true); else PACE_DENSE(64, 2, false); }
     else { if (m) PACE_DENSE(64, 1, true); else PACE_DENSE(64, 1, false); }
   }
+#undef PACE_DENSE1
 #undef PACE_DENSE
   return true;
 }

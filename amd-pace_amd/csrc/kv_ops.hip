@@ -96,20 +96,20 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
       int ca, cb;
       rope_chunk_pair(rope, ci, ca, cb);
       const int64_t src = (int64_t)t * st;
-      u32x4 ka = *reinterpret_cast<const u32x4*>(kin + src + ca * 8);
-      u32x4 kb = *reinterpret_cast<const u32x4*>(kin + src + cb * 8);
+      u32x4 ka = load16_stream(kin + src + ca * 8);
+      u32x4 kb = load16_stream(kin + src + cb * 8);
       rope_rotate_chunks(rope, rope_row(rope, b, t, (int)(pos0 + t)), ci, ka, kb);
       *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ca * 8]) = ka;
       *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + cb * 8]) = kb;
-      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ca * 8]) = *reinterpret_cast<const u32x4*>(vin + src + ca * 8);
-      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + cb * 8]) = *reinterpret_cast<const u32x4*>(vin + src + cb * 8);
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ca * 8]) = load16_stream(vin + src + ca * 8);
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + cb * 8]) = load16_stream(vin + src + cb * 8);
     }
   } else {
     for (int c = threadIdx.x; c < n_here * CHUNKS; c += 256) {
       const int r = c / CHUNKS, ch = c % CHUNKS;
       const int64_t src = (int64_t)(t_lo + r) * st + ch * 8;
-      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = *reinterpret_cast<const u32x4*>(kin + src);
-      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = *reinterpret_cast<const u32x4*>(vin + src);
+      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = load16_stream(kin + src);
+      *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = load16_stream(vin + src);
     }
   }
   __syncthreads();
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
     const int tile = c / (CHUNKS * 8), chunk = (c / 8) % CHUNKS, slot = c % 8;
     const int tok = ((slot >> 2) << 3) | (tile << 2) | (slot & 3);
     if (tok >= off_lo && tok < off_lo + n_here)
-      *reinterpret_cast<u32x4*>(kslab + c * 8) = *reinterpret_cast<const u32x4*>(&ks[tok * D + chunk * 8]);
+      store16_stream(kslab + c * 8, *reinterpret_cast<const u32x4*>(&ks[tok * D + chunk * 8]));
   }
   // V: slab chunk c = (dim tile, token half, dim) holds tokens 8*half..+7 of one dim.
   for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         w[e] = (uint32_t)vs[(8 * half + 2 * e) * (D + 8) + dim] | ((uint32_t)vs[(8 * half + 2 * e + 1) * (D + 8) + dim] << 16);
-      *reinterpret_cast<u32x4*>(vslab + c * 8) = w;
+      store16_stream(vslab + c * 8, w);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
   const uint16_t* vsrc = reinterpret_cast<const uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
   if (live) {
     for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x)
-      *reinterpret_cast<u32x4*>(&vt[c * 8]) = *reinterpret_cast<const u32x4*>(vsrc + c * 8);
+      *reinterpret_cast<u32x4*>(&vt[c * 8]) = load16_stream(vsrc + c * 8);
   }
   __syncthreads();
   for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x) {
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
     if (t >= out_len) continue;
     u32x4 kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
     if (t < len) {
-      kv = *reinterpret_cast<const u32x4*>(ksrc + k_slab_offset<D>(tok, chunk * 8));
+      kv = load16_stream(ksrc + k_slab_offset<D>(tok, chunk * 8));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const uint32_t lo = vt[v_slab_offset<D>(tok, chunk * 8 + 2 * e)];
@@ -187,8 +187,8 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
     }
     for (int r = 0; r < n_rep; ++r) {
       const int64_t o = (int64_t)b * osb + (int64_t)(h * n_rep + r) * osh + (int64_t)t * D + chunk * 8;
-      *reinterpret_cast<u32x4*>(k_out + o) = kv;
-      *reinterpret_cast<u32x4*>(v_out + o) = vv;
+      store16_stream(k_out + o, kv);
+      store16_stream(v_out + o, vv);
     }
   }
 }
@@ -210,10 +210,10 @@ __global__ __launch_bounds__(256) void kv_copy_blocks_kernel(pace_kv_pool_t src,
   u32x4* kd = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dst.k) + d * dst.k_block_stride + h * dst.k_head_stride);
   u32x4* vd = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dst.v) + d * dst.v_block_stride + h * dst.v_head_stride);
   for (int c = threadIdx.x; c < slab_chunks; c += blockDim.x) {
-    const u32x4 a = ks[c];
-    const u32x4 bq = vs[c];
-    kd[c] = a;
-    vd[c] = bq;
+    const u32x4 a = load16_stream(ks + c);
+    const u32x4 bq = load16_stream(vs + c);
+    store16_stream(kd + c, a);
+    store16_stream(vd + c, bq);
   }
 }
 
