@@ -146,16 +146,17 @@ struct WaveBlockIds {
 // NW waves per workgroup split the partition's units among themselves and merge their
 // softmax states through LDS.  OCC is the least number of waves that must fit on one SIMD
 // (caps the register budget) and OCC_MAX the most that may share it; latency is hidden by
-// the other resident waves, each wave keeps one unit (16 KiB) in flight.  With FUSED, one
-// more wave per workgroup handles the step's new tokens (attends to them from the caller's
-// buffers and stores them into the pool), so that its dependent round trips overlap with the
-// streaming waves.  With ROPE, query rows and the new keys are rotated on their way in.
+// the other resident waves, each wave keeps one unit (16 KiB) in flight.  With FUSED, the last
+// wave of a sequence's last partition also takes the step's new tokens as one more unit (attends
+// to them from the caller's buffers and stores them into the pool); a workgroup of its own shape
+// for that (a fifth wave) measured 4 % slower on the decode step than this.  With ROPE, query rows
+// and the new keys are rotated on their way in.
 template <int D, int NQT, bool HAS_MASK, int NW, int OCC, int OCC_MAX, bool FUSED, bool ROPE, bool ONCE>
-__global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_waves_per_eu(OCC, OCC_MAX))) void paged_attn_kernel(
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OCC_MAX))) void paged_attn_kernel(
     const PagedAttnParams p) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-  constexpr int NWT = NW + (FUSED ? 1 : 0);  // waves per work item
+  constexpr int NWT = NW;  // waves per work item
   // One slot of 16*NQT query rows per sender of the first merge round.  Kept as small as the
   // shape allows: LDS is one of the limits on how many workgroups share a compute unit.
   constexpr int MERGE_SLOTS = NWT / 2 > 0 ? NWT / 2 : 1;
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
   // This wave's share of the partition's 32-token units.
   const int part_units = max(0, (tok_end - part_begin + 31) / 32);
   const int per_wave = (part_units + NW - 1) / NW;
-  const int u_begin = min(part_units, wave * per_wave);  // the extra wave (wave == NW) gets none
+  const int u_begin = min(part_units, wave * per_wave);
   const int n_units = min(part_units, u_begin + per_wave) - u_begin;
   const int tok_begin = part_begin + 32 * u_begin;
 
@@ -314,15 +315,6 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
       for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
     }
   }
-  if (FUSED) {
-    if (wave == NW && n_new > 0 && part == n_parts - 1) {
-      load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
-      MaskRegs<NQT> mnew;
-      if (HAS_MASK) load_mask_regs<NQT>(mnew, p, st.mask_off, pool_end, g);  // pool_end is any position
-      if (qg == 0) write_new_tokens<D, ROPE>(p, b, kvh, pool_end, n_new, lane);
-      compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g, mnew);
-    }
-  }
 #ifdef PACE_PROBE_TIMING
   const long long pt1 = wall_clock64();
 #endif
@@ -335,6 +327,17 @@ __global__ __launch_bounds__(64 * (NW + (FUSED ? 1 : 0))) __attribute__((amdgpu_
     if (!ROPE || uu > 0) load_unit<D, ONCE>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
+  }
+  if (FUSED) {
+    // The step's new tokens: the last wave of the sequence's last partition takes them after its
+    // share of the pool (attends to them from the caller's buffers and stores them into the pool).
+    if (wave == NW - 1 && n_new > 0 && part == n_parts - 1) {
+      load_new_unit<D, ROPE>(buf, p, b, kvh, pool_end, n_new, n, g);
+      MaskRegs<NQT> mnew;
+      if (HAS_MASK) load_mask_regs<NQT>(mnew, p, st.mask_off, pool_end, g);  // pool_end is any position
+      if (qg == 0) write_new_tokens<D, ROPE>(p, b, kvh, pool_end, n_new, lane);
+      compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, pool_end, len, start, false, g, mnew);
+    }
   }
 
 #ifdef PACE_PROBE_TIMING
@@ -521,32 +524,32 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
 // Launch shape per query-tile count: waves per workgroup and unit buffers per wave.
 struct Shape {
   int nqt, nw, occ;
-  int occ_max;  // 8: no limit; 2: with five waves per workgroup, one workgroup per compute unit
+  int occ_max;  // most waves per SIMD (8: no limit)
 };
 
-static Shape shape_for(int tiles, bool fused, bool masked = false) {
+// A launch with the append fused in has the shape of one without.
+static Shape shape_for(int tiles, bool masked = false) {
   if (tiles <= 1) return Shape{1, 4, 2, 8};
   // An explicit mask costs eight more registers per tile (its values travel with the unit): no more
   // than two tiles per wave then (four tiles with a mask spilled and ran at half the speed).
-  if (masked) return Shape{2, fused ? 3 : 4, 2, 8};
-  // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit.
-  // Four waves per workgroup (three streaming + the append wave when fused) keep two
-  // workgroups on a compute unit.
+  if (masked) return Shape{2, 4, 2, 8};
+  // Two query tiles need about 230 registers: two waves per SIMD, eight per compute unit, that is
+  // two workgroups of four waves.
   // Four tiles (64 query rows, one wave per SIMD) read K/V once for up to 64 rows, which pays
   // while the launch is bound by HBM (a verify step of a wide GQA group).  Beyond 64 rows K/V
   // are re-read per row group anyway and the launch is bound by the matrix cores and by the rate
   // at which operands reach them: three tiles per wave are the most that still leave two waves
   // per SIMD (one hides the other's softmax and load latency).  Measured on a 512-token prefill
   // chunk: 768 TFLOP/s with three tiles, 708 with two, 468 with four, 450 with one.
-  if (tiles > 4 && !fused) return Shape{3, 4, 2, 8};
-  if (tiles == 2 || tiles > 4) return Shape{2, fused ? 3 : 4, 2, 8};
+  if (tiles > 4) return Shape{3, 4, 2, 8};
+  if (tiles == 2) return Shape{2, 4, 2, 8};
   return Shape{4, 2, 1, 8};
 }
 
 // Tokens one work item may cover: each wave holds at most 128 block ids.
 static int max_partition(int nw) { return nw * 2048; }
 
-// Largest partition any shape of this tile count can take (fused or not), so that one
+// Largest partition any shape of this tile count can take (with a mask or without), so that one
 // resolved value is valid for every launch of the same problem size.
 static int partition_cap(int tiles) {
   const Shape a = shape_for(tiles, false), b = shape_for(tiles, true);
@@ -555,7 +558,7 @@ static int partition_cap(int tiles) {
 
 static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
   const int tiles = (rows + 15) / 16;
-  const Shape sh = shape_for(tiles, false);
+  const Shape sh = shape_for(tiles);
   const int granule = 128;
   if (requested > 0) return requested;
   // Enough workgroups to give every compute unit (256) two of them; a batch that
@@ -577,7 +580,7 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   // K / V are read once per launch when one group of query rows covers a sequence's rows: always with one
   // or four tiles per wave, never with three, either way with two.
 #define PACE_GO1(M_, F_, R_, O_) \
-  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_, O_>), dim3(blocks), dim3(64 * (NW + (F_ ? 1 : 0))), 0, s, p)
+  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_, O_>), dim3(blocks), dim3(64 * NW), 0, s, p)
 #define PACE_GO(M_, F_, R_)                                                              \
   do {                                                                                   \
     if constexpr (NQT == 2) {                                                            \
@@ -607,10 +610,8 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
     return true;                                                                    \
   }
   PACE_TRY(1, 4, 2, 8)
-  PACE_TRY(1, 4, 2, 2)
   PACE_TRY(2, 4, 2, 8)
   PACE_TRY(3, 4, 2, 8)
-  PACE_TRY(2, 3, 2, 8)
   PACE_TRY(4, 2, 1, 8)
 #undef PACE_TRY
   return false;
@@ -660,8 +661,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
   const int tiles = (rows + 15) / 16;
-  const bool fused_req = a->k_new != nullptr;
-  const Shape sh = shape_for(tiles, fused_req, a->mask != nullptr);
+  const Shape sh = shape_for(tiles, a->mask != nullptr);
   const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
   PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
                "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(tiles));
@@ -729,14 +729,6 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   }
   p.total_items = pairs * pool->num_kv_heads * p.n_qgroups;
   PACE_REQUIRE(p.total_items < (1ll << 31), "%s: grid too large", who);
-  Shape launch_shape_sel = sh;
-  // Two rounds of one workgroup per compute unit beat one round of two: when two workgroups
-  // share a compute unit, the waves placed second on each SIMD fall behind and leave a long
-  // under-filled tail.  Applies to the fused decode shape (five waves per workgroup, so that
-  // a two-waves-per-SIMD limit means one workgroup per compute unit).
-  if (sh.nqt == 1 && sh.nw == 4 && p.n_new > 0 && p.total_items > compute_units() &&
-      p.total_items <= 2ll * compute_units())
-    launch_shape_sel.occ_max = 2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
   if (row_last) {
@@ -744,7 +736,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
     PACE_HIP_CHECK(hipGetLastError());
   }
-  const bool ok = pool->head_dim == 128 ? launch_shape<128>(launch_shape_sel, p, has_mask, s) : launch_shape<64>(launch_shape_sel, p, has_mask, s);
+  const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, has_mask, s) : launch_shape<64>(sh, p, has_mask, s);
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {

@@ -39,7 +39,7 @@ METRIC = "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, scaled by the
 # same counters on the copy-calibration workload (figures and commands: profiles/decode_8b_paged_attn_kernel.txt).
-MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_069_100_000}
+MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_075_000_000}
 
 
 def kv_token_bytes(kv_heads, head_dim):
