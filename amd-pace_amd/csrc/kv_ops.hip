@@ -240,6 +240,8 @@ int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void*
                      n_tokens, dest, rope ? *rope : none)
   if (pool->head_dim == 128) {
     if (rope) PACE_BLOCK_APPEND(128, true); else PACE_BLOCK_APPEND(128, false);
+  } else if (pool->head_dim == 256) {
+    if (rope) PACE_BLOCK_APPEND(256, true); else PACE_BLOCK_APPEND(256, false);
   } else {
     if (rope) PACE_BLOCK_APPEND(64, true); else PACE_BLOCK_APPEND(64, false);
   }
@@ -277,6 +279,8 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
                      n_tokens, (int32_t)rows, dest)
   if (pool->head_dim == 128) {
     if (paged) PACE_LAUNCH_APPEND(128, true); else PACE_LAUNCH_APPEND(128, false);
+  } else if (pool->head_dim == 256) {
+    if (paged) PACE_LAUNCH_APPEND(256, true); else PACE_LAUNCH_APPEND(256, false);
   } else {
     if (paged) PACE_LAUNCH_APPEND(64, true); else PACE_LAUNCH_APPEND(64, false);
   }
@@ -325,6 +329,9 @@ extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_t
   uint16_t* vo = static_cast<uint16_t*>(v_out);
   if (pool->head_dim == 128)
     hipLaunchKernelGGL(kv_gather_kernel<128>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias,
+                       n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
+  else if (pool->head_dim == 256)
+    hipLaunchKernelGGL(kv_gather_kernel<256>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias,
                        n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
   else
     hipLaunchKernelGGL(kv_gather_kernel<64>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias, n_rep,

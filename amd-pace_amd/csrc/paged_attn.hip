@@ -25,7 +25,7 @@ __device__ __forceinline__ u32x4 load_kv16(const uint16_t* p) {
 // Issue the 16-byte loads of one 32-token unit.  ids: pool block ids of the
 // unit's two blocks (wave-uniform).
 template <int D, bool ONCE>
-__device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n, int g) {
+__device__ __forceinline__ void load_unit_k(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n, int g) {
   // K: lane (n, g) supplies token 8*(n/4) + 4*tile + n%4 of the unit, i.e. token slot
   // n % 8 of slab tile `tile` in block A (n < 8) or B; dims 32*kk + 8g .. +8 are dim
   // chunk 4*kk + g.  A 16-lane quarter (fixed g) reads 128 contiguous bytes per block.
@@ -35,12 +35,20 @@ __device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams&
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int kk = 0; kk < D / 32; ++kk) r.k[t][kk] = load_kv16<ONCE>(kp + t * (D * 8) + kk * 256);
+}
+template <int D, bool ONCE>
+__device__ __forceinline__ void load_unit_v(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n, int g) {
   // V: lane (n, g) supplies dim 16j + n, tokens 8g..8g+7 of the unit: token half g & 1
   // of block A (g < 2) or B.  A 16-lane quarter reads 256 contiguous bytes.
   const int64_t voffA = (int64_t)idA * p.v_bs, voffB = (int64_t)idB * p.v_bs;
   const uint16_t* vp = p.vpool + ((g >= 2) ? voffB : voffA) + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8;
 #pragma unroll
   for (int j = 0; j < D / 16; ++j) r.v[j] = load_kv16<ONCE>(vp + j * 256);
+}
+template <int D, bool ONCE>
+__device__ __forceinline__ void load_unit(UnitRegs<D>& r, const PagedAttnParams& p, int kvh, int idA, int idB, int n, int g) {
+  load_unit_k<D, ONCE>(r, p, kvh, idA, idB, n, g);
+  load_unit_v<D, ONCE>(r, p, kvh, idA, idB, n, g);
 }
 
 // The "unit" made of the step's new tokens, read straight from the caller's [T][D] rows
@@ -514,10 +522,12 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + threadIdx.x * PER;
-  if (PER == 2) {
-    *reinterpret_cast<uint32_t*>(op) = pack_bf16x2(acc[0] * inv, acc[PER - 1] * inv);
-  } else {
+  if (PER == 1) {
     op[0] = (uint16_t)f32_to_bf16_bits(acc[0] * inv);
+  } else {
+#pragma unroll
+    for (int e = 0; e < PER; e += 2)
+      *reinterpret_cast<uint32_t*>(op + e) = pack_bf16x2(acc[e] * inv, acc[e + (PER > 1 ? 1 : 0)] * inv);
   }
 }
 
@@ -528,7 +538,13 @@ struct Shape {
 };
 
 // A launch with the append fused in has the shape of one without.
-static Shape shape_for(int tiles, bool masked = false) {
+static Shape shape_for(int head_dim, int tiles, bool masked = false) {
+  if (head_dim == 256) {
+    // One unit is 32 KiB in 128 registers and a query tile's output 64 more: one wave per SIMD (it may
+    // then use all 512 registers), and two tiles at most.  Two tiles' merge slots leave room in LDS for two
+    // waves per workgroup only.
+    return tiles <= 1 ? Shape{1, 2, 1, 8} : Shape{2, 2, 1, 8};
+  }
   if (tiles <= 1) return Shape{1, 4, 2, 8};
   // An explicit mask costs eight more registers per tile (its values travel with the unit): no more
   // than two tiles per wave then (four tiles with a mask spilled and ran at half the speed).
@@ -551,25 +567,27 @@ static int max_partition(int nw) { return nw * 2048; }
 
 // Largest partition any shape of this tile count can take (with a mask or without), so that one
 // resolved value is valid for every launch of the same problem size.
-static int partition_cap(int tiles) {
-  const Shape a = shape_for(tiles, false), b = shape_for(tiles, true);
+static int partition_cap(int head_dim, int tiles) {
+  const Shape a = shape_for(head_dim, tiles, false), b = shape_for(head_dim, tiles, true);
   return max_partition(a.nw < b.nw ? a.nw : b.nw);
 }
 
-static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows) {
+static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t batch, int32_t num_kv_heads, int32_t rows,
+                             int32_t head_dim) {
   const int tiles = (rows + 15) / 16;
-  const Shape sh = shape_for(tiles);
+  const Shape sh = shape_for(head_dim, tiles);
   const int granule = 128;
   if (requested > 0) return requested;
-  // Enough workgroups to give every compute unit (256) two of them; a batch that
-  // already does so is not split at all.
+  // Enough workgroups to fill every compute unit (256) with as many as fit (4 * occ waves each); a batch
+  // that already does so is not split at all.
   const int64_t groups = (int64_t)batch * num_kv_heads * ((tiles + sh.nqt - 1) / sh.nqt);
-  int64_t parts = (512 + groups - 1) / groups;
+  const int64_t slots = 256 * 4 * sh.occ / sh.nw;
+  int64_t parts = (slots + groups - 1) / groups;
   if (parts < 1) parts = 1;
   int64_t per = ((int64_t)max_seq_len + parts - 1) / parts;
   per = (per + granule - 1) / granule * granule;
   if (per < granule) per = granule;
-  if (per > partition_cap(tiles)) per = partition_cap(tiles);
+  if (per > partition_cap(head_dim, tiles)) per = partition_cap(head_dim, tiles);
   return (int)per;
 }
 
@@ -609,10 +627,15 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
     launch<D, NQT_, NW_, OCC_, MAX_>(p, has_mask, s);                               \
     return true;                                                                    \
   }
-  PACE_TRY(1, 4, 2, 8)
-  PACE_TRY(2, 4, 2, 8)
-  PACE_TRY(3, 4, 2, 8)
-  PACE_TRY(4, 2, 1, 8)
+  if constexpr (D == 256) {
+    PACE_TRY(1, 2, 1, 8)
+    PACE_TRY(2, 2, 1, 8)
+  } else {
+    PACE_TRY(1, 4, 2, 8)
+    PACE_TRY(2, 4, 2, 8)
+    PACE_TRY(3, 4, 2, 8)
+    PACE_TRY(4, 2, 1, 8)
+  }
 #undef PACE_TRY
   return false;
 }
@@ -661,10 +684,10 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;
   const int tiles = (rows + 15) / 16;
-  const Shape sh = shape_for(tiles, a->mask != nullptr);
-  const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows);
+  const Shape sh = shape_for(pool->head_dim, tiles, a->mask != nullptr);
+  const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows, pool->head_dim);
   PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
-               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(tiles));
+               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(pool->head_dim, tiles));
   int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
   if (a->seq_parts) {
     PACE_REQUIRE(a->work_items != nullptr && a->max_parts >= 1,
@@ -736,7 +759,9 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
     PACE_HIP_CHECK(hipGetLastError());
   }
-  const bool ok = pool->head_dim == 128 ? launch_shape<128>(sh, p, has_mask, s) : launch_shape<64>(sh, p, has_mask, s);
+  const bool ok = pool->head_dim == 128   ? launch_shape<128>(sh, p, has_mask, s)
+                  : pool->head_dim == 256 ? launch_shape<256>(sh, p, has_mask, s)
+                                          : launch_shape<64>(sh, p, has_mask, s);
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
@@ -744,6 +769,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     PACE_REQUIRE(rows_total < ((size_t)1 << 31), "%s: too many query rows", who);
     if (pool->head_dim == 128)
       hipLaunchKernelGGL(paged_attn_merge_kernel<128>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+    else if (pool->head_dim == 256)
+      hipLaunchKernelGGL(paged_attn_merge_kernel<256>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
     else
       hipLaunchKernelGGL(paged_attn_merge_kernel<64>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
     PACE_HIP_CHECK(hipGetLastError());
@@ -767,10 +794,11 @@ extern "C" int pace_probe_read(long long* host, unsigned int* n, int reset) {
 }
 #endif
 
-extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t max_seq_len,
-                                                    int32_t partition_tokens, int32_t num_kv_heads) {
-  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
-  return resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, q_len * (num_q_heads / num_kv_heads));
+extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
+                                                    int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {
+  if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
+  return resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, q_len * (num_q_heads / num_kv_heads),
+                           head_dim);
 }
 
 // Partials of every (row, partition) when a sequence is cut into several partitions, then (16-byte
@@ -786,7 +814,7 @@ extern "C" size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_h
                                                   int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {
   if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_seq_len <= 0 || num_kv_heads <= 0) return 0;
   const int rows = q_len * (num_q_heads / num_kv_heads);
-  const int part = resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, rows);
+  const int part = resolve_partition(partition_tokens, max_seq_len, batch, num_kv_heads, rows, head_dim);
   const int max_parts = (max_seq_len + part - 1) / part;
   return workspace_need(batch, num_q_heads, q_len, head_dim, max_parts, rows);
 }

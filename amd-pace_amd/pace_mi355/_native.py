@@ -162,7 +162,7 @@ def load() -> ctypes.CDLL:
         + [c_void_p, c_int32, c_void_p, c_int32, c_void_p]
     )
     lib.pace_paged_attn_partition_tokens.restype = c_int32
-    lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 6
+    lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 7
     lib.pace_paged_attn_workspace_bytes.restype = c_size_t
     lib.pace_paged_attn_workspace_bytes.argtypes = [c_int32] * 7
     lib.pace_paged_attn_workspace_bytes_for_parts.restype = c_size_t
@@ -184,13 +184,22 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-def row_groups(query_rows: int, masked: bool = False) -> int:
+def row_groups(query_rows: int, masked: bool = False, head_dim: int = 128) -> int:
     """Workgroups one (sequence, KV head, partition) needs for ``query_rows`` = q_len * n_rep rows:
     the library packs 16, 32, 48 or 64 rows per workgroup (one 16-row tile up to 16 rows, two for
-    17..32, four for 33..64, three beyond 64; never more than two with an explicit mask)."""
+    17..32, four for 33..64, three beyond 64; never more than two with an explicit mask or with
+    head_dim 256)."""
     tiles = max(1, -(-int(query_rows) // 16))
-    per_group = 1 if tiles <= 1 else (2 if tiles == 2 or masked else (4 if tiles <= 4 else 3))
+    two_at_most = masked or head_dim == 256
+    per_group = 1 if tiles <= 1 else (2 if tiles == 2 or two_at_most else (4 if tiles <= 4 else 3))
     return -(-tiles // per_group)
+
+
+def workgroup_slots(query_rows: int, head_dim: int = 128) -> int:
+    """Workgroups of one attention launch that are resident at the same time on the 256 compute
+    units: two per unit, except one with head_dim 256 and a single 16-row tile (one wave per SIMD,
+    four waves per workgroup)."""
+    return 512
 
 
 def check(rc: int) -> None:

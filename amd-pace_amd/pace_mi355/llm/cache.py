@@ -436,7 +436,7 @@ class PagedKVCache(KVCacheBase):
         if self._uniform:
             key = (B, hq, S, D, want, -(-max_len // 128))
             if key != self._plan_key:
-                part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
+                part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, max_len, want, self.num_kv_heads))
                 max_parts = max(1, -(-max_len // part)) if part else 1
                 ws = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, -(-max_len // 128) * 128, part, self.num_kv_heads))
                 self._plan_key, self._plan_val = key, (None, None, part, max_parts, ws)
@@ -447,12 +447,14 @@ class PagedKVCache(KVCacheBase):
             mean = float(self.lens.mean())
             if max_len > 1.5 * mean:
                 want = max(1024, (int(mean) + 127) // 128 * 128)
-        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, want, self.num_kv_heads))
+        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, max_len, want, self.num_kv_heads))
         items = parts = None
         max_parts = 1
         if part:
-            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, self.num_kv_heads))
-            slots = max(1, 512 // (self.num_kv_heads * nat.row_groups(S * (hq // self.num_kv_heads))))
+            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, 1 << 30, 0, self.num_kv_heads))
+            rows = S * (hq // self.num_kv_heads)
+            groups = self.num_kv_heads * nat.row_groups(rows, head_dim=self.head_dim)
+            slots = max(1, nat.workgroup_slots(rows, self.head_dim) // groups)
             items, parts, max_parts = self.state.plan_attention(self.lens, part, cap, slots)
         if parts is not None:
             ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))

@@ -14,6 +14,9 @@ Other workloads (same JSON shape, `config.workload` names them):
   ragged    batch 256, contexts log-uniform in [128, 16384], pool 1.3x live tokens:
             append + decode per step; gather timed beside it
   verify    batch 32, contexts U[1024, 8192], 8 draft tokens appended + causal 8-query attention
+  prefill / dense-prefill   a 512-token chunk over 3584 cached tokens through the paged path; the dense
+            op on 2048 x 2048 with the additive causal mask (roofline against the matrix-core peak)
+  decode-gptj   the headline step at GPT-J-6B's attention shape (16 heads of 256, batch 64 x 2048)
   compact   Llama-3-70B-shape KV, batch 8, context 32768: evict 40% of the blocks, then time the
             compaction copy and the decode over the compacted cache
   copy-calibration   block copy of a known byte count, used to scale the HBM byte counters
@@ -125,9 +128,10 @@ class FixedStep:
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         if partition == 0 and max_len > 1.5 * float(lens_after.mean()):  # same rule as PagedKVCache.attend
             partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
-        part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, max_len, partition, cache.num_kv_heads))
-        cap = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, 1 << 30, 0, cache.num_kv_heads))
-        slots = max(1, 512 // (cache.num_kv_heads * nat.row_groups(S * (hq // cache.num_kv_heads))))
+        part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, cache.head_dim, max_len, partition, cache.num_kv_heads))
+        cap = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, cache.head_dim, 1 << 30, 0, cache.num_kv_heads))
+        rows = S * (hq // cache.num_kv_heads)
+        slots = max(1, nat.workgroup_slots(rows, cache.head_dim) // (cache.num_kv_heads * nat.row_groups(rows, head_dim=cache.head_dim)))
         # ragged batches: compact longest-first work list; single-round launches: evened-out partition counts
         self.items, self.parts, max_parts = cache.state.plan_attention(lens_after, part, cap, slots)
         a.max_seq_len, a.partition_tokens, a.scale = max_len, part, 1.0 / math.sqrt(D)
@@ -254,7 +258,22 @@ def result_line(args, workload, step_bytes, tokens_per_step, dt, roof, extra_cfg
 
 # ---- workloads ---------------------------------------------------------------------------------
 def wl_decode_8b(torch, dev, args):
-    B, ctx, hq, hkv, D = 64, 4096, 32, 8, 128
+    return _wl_decode(torch, dev, args, (64, 4096, 32, 8, 128),
+                      "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, head_dim 128, "
+                      "KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
+                      MEASURED_TRAFFIC_BYTES["decode-8b"], with_cpu=True)
+
+
+def wl_decode_gptj(torch, dev, args):
+    """The same step at GPT-J-6B's attention shape (16 heads of 256, no GQA): the same bytes per step
+    as the headline with half the context."""
+    return _wl_decode(torch, dev, args, (64, 2048, 16, 16, 256),
+                      "GPT-J-6B-shape single-layer decode: batch 64, context 2048 (+1 appended), 16 Q / 16 KV heads, head_dim 256, "
+                      "KV block 16, seeded random physical block permutation, 1-token append + decode", None, with_cpu=False)
+
+
+def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
+    B, ctx, hq, hkv, D = shape
     cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute,
                         headroom=64 + args.steps + args.warmup)
     cache.partition_tokens = args.partition
@@ -300,15 +319,12 @@ def wl_decode_8b(torch, dev, args):
     fused = args.path == "direct" and not args.no_fuse or args.path == "api"
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
     line = result_line(
-        args,
-        "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, head_dim 128, "
-        "KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
-        dec + append_bytes(B, 1, hkv, D), B, dt,
-        roofline("paged_attn_kernel<128,1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
-                 {"traffic": MEASURED_TRAFFIC_BYTES["decode-8b"]}),
+        args, label, dec + append_bytes(B, 1, hkv, D), B, dt,
+        roofline(f"paged_attn_kernel<{D},1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
+                 {"traffic": traffic}),
         {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct"),
          "mask": bool(args.mask and args.path == "api")})
-    if not args.no_cpu_baseline:
+    if with_cpu and not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
 
@@ -544,7 +560,7 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
     }
 
 
-WORKLOADS = {"decode-8b": wl_decode_8b, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill,
+WORKLOADS = {"decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill,
              "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 

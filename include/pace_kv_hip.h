@@ -57,7 +57,7 @@ typedef struct pace_kv_pool {
   int64_t v_head_stride;
   int32_t num_blocks;
   int32_t num_kv_heads;
-  int32_t head_dim;       /* 64 or 128                                       */
+  int32_t head_dim;       /* 64, 128 or 256                                  */
   int32_t block_size;     /* must be PACE_KV_BLOCK_TOKENS                    */
 } pace_kv_pool_t;
 
@@ -235,8 +235,8 @@ typedef struct pace_paged_attn_args {
 /* The context split size (tokens per workgroup) the library uses for these sizes when
  * partition_tokens is 0; a sequence of n tokens is cut into ceil(n / split) equal partitions. */
 int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len,
-                                         int32_t max_seq_len, int32_t partition_tokens,
-                                         int32_t num_kv_heads);
+                                         int32_t head_dim, int32_t max_seq_len,
+                                         int32_t partition_tokens, int32_t num_kv_heads);
 
 /* Scratch bytes the two entry points below need for these sizes (0 = none): the partial results
  * of sequences cut into several partitions and, for launches of more than 64 query rows per KV
