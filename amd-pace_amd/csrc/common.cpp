@@ -32,8 +32,7 @@ int check_pool(const pace_kv_pool_t* pool, const char* who) {
   PACE_REQUIRE(pool->k != nullptr && pool->v != nullptr, "%s: pool has a NULL K or V pointer", who);
   PACE_REQUIRE(pool->block_size == PACE_KV_BLOCK_TOKENS, "%s: block_size %d unsupported (must be %d)", who,
                pool->block_size, PACE_KV_BLOCK_TOKENS);
-  PACE_REQUIRE(pool->head_dim == 64 || pool->head_dim == 128 || pool->head_dim == 256,
-               "%s: head_dim %d unsupported (64, 128 or 256)", who, pool->head_dim);
+  PACE_REQUIRE(head_dim_supported(pool->head_dim), "%s: head_dim %d unsupported (64, 96, 128 or 256)", who, pool->head_dim);
   PACE_REQUIRE(pool->num_blocks > 0 && pool->num_kv_heads > 0, "%s: empty pool (%d blocks, %d heads)", who,
                pool->num_blocks, pool->num_kv_heads);
   const int64_t slab = (int64_t)pool->block_size * pool->head_dim;

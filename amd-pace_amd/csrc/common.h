@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "pace_kv_hip.h"
 
 namespace pace_kv {
@@ -91,5 +93,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
+
+// Head sizes the pool kernels are built for.  Calls f(std::integral_constant<int, D>) for the one that
+// matches; false if none does (check_pool() has then already refused the pool).
+template <class F>
+inline bool for_head_dim(int head_dim, F&& f) {
+  switch (head_dim) {
+    case 64: f(std::integral_constant<int, 64>{}); return true;
+    case 96: f(std::integral_constant<int, 96>{}); return true;
+    case 128: f(std::integral_constant<int, 128>{}); return true;
+    case 256: f(std::integral_constant<int, 256>{}); return true;
+    default: return false;
+  }
+}
+inline bool head_dim_supported(int head_dim) { return head_dim == 64 || head_dim == 96 || head_dim == 128 || head_dim == 256; }
 
 }  // namespace pace_kv

@@ -238,13 +238,10 @@ int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void*
 #define PACE_BLOCK_APPEND(DIM, R_)                                                                                        \
   hipLaunchKernelGGL((kv_append_block_kernel<DIM, R_>), grid, dim3(256), 0, stream, *pool, kq, vq, stride_b, stride_h, stride_t, \
                      n_tokens, dest, rope ? *rope : none)
-  if (pool->head_dim == 128) {
-    if (rope) PACE_BLOCK_APPEND(128, true); else PACE_BLOCK_APPEND(128, false);
-  } else if (pool->head_dim == 256) {
-    if (rope) PACE_BLOCK_APPEND(256, true); else PACE_BLOCK_APPEND(256, false);
-  } else {
-    if (rope) PACE_BLOCK_APPEND(64, true); else PACE_BLOCK_APPEND(64, false);
-  }
+  for_head_dim(pool->head_dim, [&](auto d) {
+    constexpr int DIM = decltype(d)::value;
+    if (rope) PACE_BLOCK_APPEND(DIM, true); else PACE_BLOCK_APPEND(DIM, false);
+  });
 #undef PACE_BLOCK_APPEND
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
@@ -277,13 +274,10 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
 #define PACE_LAUNCH_APPEND(DIM, PG)                                                                                  \
   hipLaunchKernelGGL((kv_append_kernel<DIM, PG>), dim3(grid), dim3(256), 0, s, *pool, k, v, stride_b, stride_h, stride_t, \
                      n_tokens, (int32_t)rows, dest)
-  if (pool->head_dim == 128) {
-    if (paged) PACE_LAUNCH_APPEND(128, true); else PACE_LAUNCH_APPEND(128, false);
-  } else if (pool->head_dim == 256) {
-    if (paged) PACE_LAUNCH_APPEND(256, true); else PACE_LAUNCH_APPEND(256, false);
-  } else {
-    if (paged) PACE_LAUNCH_APPEND(64, true); else PACE_LAUNCH_APPEND(64, false);
-  }
+  for_head_dim(pool->head_dim, [&](auto d) {
+    constexpr int DIM = decltype(d)::value;
+    if (paged) PACE_LAUNCH_APPEND(DIM, true); else PACE_LAUNCH_APPEND(DIM, false);
+  });
 #undef PACE_LAUNCH_APPEND
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
@@ -327,15 +321,10 @@ extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_t
   hipStream_t s = static_cast<hipStream_t>(stream);
   uint16_t* ko = static_cast<uint16_t*>(k_out);
   uint16_t* vo = static_cast<uint16_t*>(v_out);
-  if (pool->head_dim == 128)
-    hipLaunchKernelGGL(kv_gather_kernel<128>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias,
-                       n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
-  else if (pool->head_dim == 256)
-    hipLaunchKernelGGL(kv_gather_kernel<256>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias,
-                       n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
-  else
-    hipLaunchKernelGGL(kv_gather_kernel<64>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias, n_rep,
-                       ko, vo, out_stride_b, out_stride_h, out_len);
+  for_head_dim(pool->head_dim, [&](auto d) {
+    hipLaunchKernelGGL(kv_gather_kernel<decltype(d)::value>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens,
+                       seq_len_bias, n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
+  });
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }

@@ -509,26 +509,29 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   float M = kNegInf;
   for (int i = 0; i < n_parts; ++i) M = fmaxf(M, ml[2 * i]);
   const float m_use = (M == kNegInf) ? 0.f : M;
-  constexpr int PER = D / 64;  // dims per lane
-  float acc[PER];
+  constexpr int PASSES = (D + 127) / 128;  // a lane owns the dim pairs 2 * lane + 128 * pass that exist
+  float acc[PASSES][2];
 #pragma unroll
-  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+  for (int e = 0; e < PASSES; ++e) acc[e][0] = acc[e][1] = 0.f;
   float L = 0.f;
+  const int d0 = 2 * threadIdx.x;
   for (int i = 0; i < n_parts; ++i) {
     const float w = __builtin_amdgcn_exp2f(ml[2 * i] - m_use);
     L += w * ml[2 * i + 1];
 #pragma unroll
-    for (int e = 0; e < PER; ++e) acc[e] += w * po[(int64_t)i * D + threadIdx.x * PER + e];
+    for (int e = 0; e < PASSES; ++e) {
+      if (d0 + 128 * e < D) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(po + (int64_t)i * D + d0 + 128 * e);
+        acc[e][0] += w * __uint_as_float(v[0]);
+        acc[e][1] += w * __uint_as_float(v[1]);
+      }
+    }
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + threadIdx.x * PER;
-  if (PER == 1) {
-    op[0] = (uint16_t)f32_to_bf16_bits(acc[0] * inv);
-  } else {
+  uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + d0;
 #pragma unroll
-    for (int e = 0; e < PER; e += 2)
-      *reinterpret_cast<uint32_t*>(op + e) = pack_bf16x2(acc[e] * inv, acc[e + (PER > 1 ? 1 : 0)] * inv);
-  }
+  for (int e = 0; e < PASSES; ++e)
+    if (d0 + 128 * e < D) *reinterpret_cast<uint32_t*>(op + 128 * e) = pack_bf16x2(acc[e][0] * inv, acc[e][1] * inv);
 }
 
 // Launch shape per query-tile count: waves per workgroup and unit buffers per wave.
@@ -608,7 +611,10 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
     }                                                                                    \
   } while (0)
   if (p.rope.cos) {  // never together with an explicit mask (checked by the caller)
-    if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
+    // (head sizes whose halves fall inside a 32-dim operand step have no in-register rotation: refused by the caller)
+    if constexpr (D % 64 == 0) {
+      if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
+    }
   } else if (has_mask) {
     if constexpr (NQT <= 2) {  // shape_for() never asks for more tiles with a mask
       if (fused) PACE_GO(true, true, false); else PACE_GO(true, false, false);
@@ -677,6 +683,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     if (int rc = make_rope_dev(a->rope, pool->head_dim, false, who, &rope_dev)) return rc;
     PACE_REQUIRE(rope_dev.rot == pool->head_dim, "%s: rotary_dim %d must equal head_dim %d when rope rides in the attention launch",
                  who, rope_dev.rot, pool->head_dim);
+    PACE_REQUIRE(pool->head_dim % 64 == 0, "%s: rope cannot ride in the attention launch with head_dim %d (rotate with pace_rope_* first)",
+                 who, pool->head_dim);
     PACE_REQUIRE(a->mask == nullptr, "%s: rope in the attention launch cannot be combined with an explicit mask", who);
     PACE_REQUIRE(!a->k_new || a->n_new == a->q_len, "%s: with rope, the fused append takes n_new == q_len (got %d, %d)", who,
                  a->n_new, a->q_len);
@@ -759,20 +767,16 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
     PACE_HIP_CHECK(hipGetLastError());
   }
-  const bool ok = pool->head_dim == 128   ? launch_shape<128>(sh, p, has_mask, s)
-                  : pool->head_dim == 256 ? launch_shape<256>(sh, p, has_mask, s)
-                                          : launch_shape<64>(sh, p, has_mask, s);
+  bool ok = false;
+  for_head_dim(pool->head_dim, [&](auto d) { ok = launch_shape<decltype(d)::value>(sh, p, has_mask, s); });
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
     PACE_REQUIRE(rows_total < ((size_t)1 << 31), "%s: too many query rows", who);
-    if (pool->head_dim == 128)
-      hipLaunchKernelGGL(paged_attn_merge_kernel<128>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
-    else if (pool->head_dim == 256)
-      hipLaunchKernelGGL(paged_attn_merge_kernel<256>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
-    else
-      hipLaunchKernelGGL(paged_attn_merge_kernel<64>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+    for_head_dim(pool->head_dim, [&](auto d) {
+      hipLaunchKernelGGL(paged_attn_merge_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+    });
     PACE_HIP_CHECK(hipGetLastError());
   }
   return PACE_KV_OK;

@@ -104,12 +104,7 @@ static int launch_rows(RopeRowsParams& p, int head_dim, int batch, void* stream,
   p.total = total;
   const unsigned grid = (unsigned)((total + 255) / 256);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (head_dim == 128)
-    hipLaunchKernelGGL(rope_rows_kernel<128>, dim3(grid), dim3(256), 0, s, p);
-  else if (head_dim == 256)
-    hipLaunchKernelGGL(rope_rows_kernel<256>, dim3(grid), dim3(256), 0, s, p);
-  else
-    hipLaunchKernelGGL(rope_rows_kernel<64>, dim3(grid), dim3(256), 0, s, p);
+  for_head_dim(head_dim, [&](auto d) { hipLaunchKernelGGL(rope_rows_kernel<decltype(d)::value>, dim3(grid), dim3(256), 0, s, p); });
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }
@@ -132,8 +127,7 @@ extern "C" int pace_rope_apply(const pace_rope_t* rope, const void* q, void* q_o
                                int64_t k_stride_h, int64_t k_stride_t, int32_t num_k_heads, int32_t batch, int32_t n_tokens,
                                int32_t head_dim, void* stream) {
   const char* who = "pace_rope_apply";
-  PACE_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "%s: head_dim %d unsupported (64, 128 or 256)", who,
-               head_dim);
+  PACE_REQUIRE(head_dim_supported(head_dim), "%s: head_dim %d unsupported (64, 96, 128 or 256)", who, head_dim);
   PACE_REQUIRE(batch >= 0 && n_tokens >= 0, "%s: negative batch (%d) or n_tokens (%d)", who, batch, n_tokens);
   RopeRowsParams p = {};
   if (int rc = make_rope_dev(rope, head_dim, true, who, &p.rope)) return rc;

@@ -483,7 +483,7 @@ class PagedKVCache(KVCacheBase):
             if tuple(rope.rows.shape) != (B, S):
                 raise RuntimeError(f"rope rows {tuple(rope.rows.shape)} do not match the query [B={B}, S={S}]")
             rope_desc = rope.desc()
-            if attention_mask is not None or rope_desc.rotary_dim != D:
+            if attention_mask is not None or rope_desc.rotary_dim != D or D % 64:
                 # cases the attention launch does not fold in: rotate the queries (and a held-back append) first
                 self._flush()
                 query, _ = rope(query, None)

@@ -12,7 +12,7 @@ rotation can run
                                                                      -> ``pace_rope_append_paged``
   * folded into the attention launch together with the append (decode / verify steps).
 
-bf16 device tensors with head_dim 64, 128 or 256 only; anything else raises (there is
+bf16 device tensors with head_dim 64, 96, 128 or 256 only; anything else raises (there is
 no second implementation).
 """
 from __future__ import annotations
@@ -82,8 +82,8 @@ def _check_rows(x: torch.Tensor, name: str) -> None:
     if not x.is_cuda or x.dtype != torch.bfloat16 or x.dim() != 4:
         raise NotImplementedError(f"rotary embedding runs on bf16 device tensors [B, H, S, D]; {name} is "
                                   f"{x.dtype} {tuple(x.shape)} on {x.device}")
-    if x.shape[-1] not in (64, 128, 256):
-        raise NotImplementedError(f"rotary embedding supports head_dim 64, 128 or 256, got {x.shape[-1]}")
+    if x.shape[-1] not in (64, 96, 128, 256):
+        raise NotImplementedError(f"rotary embedding supports head_dim 64, 96, 128 or 256, got {x.shape[-1]}")
 
 
 def _strided(x: torch.Tensor) -> torch.Tensor:

@@ -57,7 +57,7 @@ typedef struct pace_kv_pool {
   int64_t v_head_stride;
   int32_t num_blocks;
   int32_t num_kv_heads;
-  int32_t head_dim;       /* 64, 128 or 256                                  */
+  int32_t head_dim;       /* 64, 96, 128 or 256                              */
   int32_t block_size;     /* must be PACE_KV_BLOCK_TOKENS                    */
 } pace_kv_pool_t;
 

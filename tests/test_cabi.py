@@ -69,10 +69,10 @@ def test_argument_errors_are_reported_without_a_gpu():
                            num_blocks=4, num_kv_heads=2, head_dim=128, block_size=32)
     rc = lib.pace_kv_append(ctypes.byref(bad), 16, 16, 8, 8, 8, 1, 1, 16, None)
     assert rc == -1 and b"block_size 32 unsupported" in lib.pace_kv_last_error()
-    bad.block_size, bad.head_dim = 16, 96
+    bad.block_size, bad.head_dim = 16, 80
     assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 0, 1, 1, 16, 16, 8, 8, 16, None) == -1
-    assert b"head_dim 96 unsupported" in lib.pace_kv_last_error()
-    with pytest.raises(_native.NativeError, match="head_dim 96"):
+    assert b"head_dim 80 unsupported" in lib.pace_kv_last_error()
+    with pytest.raises(_native.NativeError, match="head_dim 80"):
         _native.check(-1)
     assert lib.pace_attn_dense(16, 16, 16, 16, 1, 1, 1, 1, 1, 300, None, 0, 1, 1, 1, None) == -1
     assert b"head_dim 300 unsupported" in lib.pace_kv_last_error()
@@ -85,8 +85,8 @@ def test_argument_errors_are_reported_without_a_gpu():
     rope.rotary_dim, rope.positions = 64, None
     assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 64, None) == -1
     assert b"positions are required" in lib.pace_kv_last_error()
-    assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 96, None) == -1
-    assert b"head_dim 96 unsupported" in lib.pace_kv_last_error()
+    assert lib.pace_rope_apply(ctypes.byref(rope), *rows, *rows, 1, 1, 80, None) == -1
+    assert b"head_dim 80 unsupported" in lib.pace_kv_last_error()
     # paged attention: a scale that is not positive and finite is refused before the launch
     pool = _native.PoolDesc(k=16, v=32, k_block_stride=4096, k_head_stride=2048, v_block_stride=4096, v_head_stride=2048,
                             num_blocks=4, num_kv_heads=2, head_dim=128, block_size=16)

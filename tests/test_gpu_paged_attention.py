@@ -37,6 +37,9 @@ def _build(device, B, hkv, n_rep, D, lens, seed, partition=0, num_blocks=None, s
         (3, 4, 1, 256, [700, 31, 1500], 256),         # head_dim 256 (GPT-J's heads), MHA, several partitions
         (2, 2, 4, 256, [129, 4100], 0),               # head_dim 256 with a GQA group
         (2, 1, 20, 256, [95, 300], 128),              # head_dim 256, two query tiles
+        (3, 4, 1, 96, [700, 31, 1500], 256),          # head_dim 96 (Phi-3-mini's heads), several partitions
+        (2, 2, 4, 96, [129, 4100], 0),                # head_dim 96 with a GQA group
+        (2, 1, 40, 96, [95, 300], 128),               # head_dim 96, three query tiles
     ],
 )
 def test_decode_matches_oracle(device, B, hkv, n_rep, D, lens, partition):
@@ -223,7 +226,8 @@ def test_decode_invariant_to_physical_block_permutation(device):
 @pytest.mark.parametrize("T,S,lens,partition,D", [(1, 1, [40, 200, 1029, 16], 0, 128), (1, 1, [4096, 17], 512, 128),
                                                   (8, 8, [31, 700], 256, 128), (9, 9, [100, 64], 0, 128), (16, 1, [5, 48], 0, 128),
                                                   (32, 32, [33, 500], 0, 128), (1, 1, [40, 200, 1029, 16], 0, 256),
-                                                  (5, 5, [31, 700], 256, 256), (1, 1, [77, 130], 0, 64)])
+                                                  (5, 5, [31, 700], 256, 256), (1, 1, [77, 130], 0, 64),
+                                                  (1, 1, [77, 1300], 0, 96), (7, 7, [40, 600], 256, 96)])
 def test_fused_append_equals_append_then_attend(device, T, S, lens, partition, D):
     """update_cache holds the new tokens back and the attention launch both reads them from the
     caller's tensors and stores them: same attention result as append-then-attend (to tolerance, the
@@ -332,7 +336,7 @@ def test_fused_append_with_sequences_of_length_zero_and_one(device):
     assert torch.equal(gk.cpu(), K) and torch.equal(gv.cpu(), V)
 
 
-@pytest.mark.parametrize("D,S,n_rep", [(128, 64, 4), (64, 48, 4), (128, 33, 8), (256, 24, 2)])
+@pytest.mark.parametrize("D,S,n_rep", [(128, 64, 4), (64, 48, 4), (128, 33, 8), (256, 24, 2), (96, 40, 4)])
 def test_prefill_sized_launch_matches_oracle(device, D, S, n_rep):
     """A prefill-sized launch (hundreds of query rows per KV head over the whole batch): ragged
     lengths, a partly filled last row group, and a chunk appended on top of cached tokens."""
@@ -395,7 +399,7 @@ def test_paged_attention_random_batches_masks_and_partitions(device, seed):
     rng = np.random.default_rng(2000 + seed)
     for case in range(6):
         B = int(rng.integers(1, 5))
-        hkv, n_rep, D = int(rng.choice([1, 2, 4])), int(rng.choice([1, 4, 8])), int(rng.choice([64, 128, 128, 256]))
+        hkv, n_rep, D = int(rng.choice([1, 2, 4])), int(rng.choice([1, 4, 8])), int(rng.choice([64, 96, 128, 128, 256]))
         S = int(rng.choice([1, 2, 5, 8, 16, 24, 70]))
         past = rng.integers(0, 400, size=B)
         uniform = rng.random() < 0.5

@@ -29,7 +29,7 @@ def _oracle_rotate(x, module, position_ids, neox=True):
 
 @pytest.mark.parametrize("D,neox,partial", [(128, True, 1.0), (128, False, 1.0), (64, True, 1.0), (64, False, 1.0),
                                             (128, True, 0.5), (64, False, 0.5), (128, False, 0.25),
-                                            (256, False, 0.25), (256, True, 1.0)])
+                                            (256, False, 0.25), (256, True, 1.0), (96, True, 1.0), (96, False, 0.5)])
 def test_dense_rope_is_bit_exact(device, D, neox, partial):
     B, Hq, Hk, S = 3, 8, 2, 19
     mod = _module(D, partial_rotary_factor=partial)
@@ -92,7 +92,7 @@ def test_fp32_tables_are_rounded_like_the_reference(device):
 
 
 @pytest.mark.parametrize("D,neox,steps", [(128, True, [5, 1, 1, 40, 1]), (64, False, [17, 3, 1]), (128, False, [1, 1, 16, 33]),
-                                          (256, False, [5, 1, 16, 9])])
+                                          (256, False, [5, 1, 16, 9]), (96, True, [5, 1, 16, 9])])
 def test_rope_append_fills_the_pool_like_rope_then_update_cache(device, D, neox, steps):
     """rope(k) then update_cache (llama.py:147-158) == one rotate-and-append launch, bit for bit."""
     from pace_mi355.llm import PagedKVCache
@@ -165,7 +165,7 @@ def _reference_step(q, k, v, mod, pos, ref_cache, n_rep, neox=True):
 
 
 @pytest.mark.parametrize("D,neox,S", [(128, True, 1), (128, False, 1), (64, True, 1), (128, True, 8), (64, False, 5), (128, True, 20),
-                                      (256, True, 1), (256, False, 4)])
+                                      (256, True, 1), (256, False, 4), (96, True, 1), (96, False, 3)])
 def test_one_launch_step_rope_append_attention(device, D, neox, S):
     """update_cache(raw k, v, rope) + attention(raw q): one launch per step; pool bit-exact,
     attention within tolerance, and identical to rotating in a launch of its own."""
@@ -195,7 +195,10 @@ def test_one_launch_step_rope_append_attention(device, D, neox, S):
         q_rot, k_rot = rope(qd, kd)
         kk2, vv2 = split.update_cache(k_rot, vd, 2)
         got2 = attn(q_rot, kk2, vv2)
-        assert_bits_equal(got, got2, f"step {i}: fused launch vs separate launches")
+        if D % 64 == 0:
+            assert_bits_equal(got, got2, f"step {i}: fused launch vs separate launches")
+        else:  # no in-launch rotation for this head size: the first path appends before it attends, the second fuses the append
+            assert_attention_close(got2, want, f"step {i} separate launches")
         past += T
         kg, vg = fused.gather(n_rep=1)
         assert_bits_equal(kg, ref.key, f"pool K after step {i}")
