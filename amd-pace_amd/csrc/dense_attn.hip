@@ -2,14 +2,23 @@
 // pace::attention for arbitrary head_dim, fp32 or bf16 tensors and an arbitrary
 // additive mask broadcast from [mB][mN][mS][L].
 //
-// One 256-thread workgroup owns 16 query rows of one (batch, head) and streams
-// the keys / values in chunks through LDS with an online softmax, so the
-// [S][L] score matrix is never materialised.  fp32 arithmetic throughout.
-#include "common.h"
+// General kernel (fp32 tensors, head sizes the bf16 kernels are not built for): fp32 arithmetic on
+// the matrix cores (v_mfma_f32_16x16x4_f32), online softmax, the [S][L] score matrix never
+// materialised.  A wave owns 16 query rows of one (batch, head) and walks its share of the keys in
+// 16-token tiles; with lane = (n, g), n = lane % 16, g = lane / 16:
+//   S^T tile = K[16 tokens x HP dims] * Q^T[HP dims x 16 rows], HP/4 steps of 4 dims: in step s lane
+//       (n, g) supplies dim g*HP/4 + s of K row n (A operand) and of Q row n (B operand) -- any
+//       assignment of dims to steps gives the same sum, this one lets a lane read its dims of a row
+//       as one contiguous run; the result leaves lane (n, g) with tokens 4g..4g+3 of query row n;
+//   O^T tile = V^T[16 dims x 16 tokens] * P^T[16 tokens x 16 rows], 4 steps: in step i lane (n, g)
+//       supplies V[token 4g+i][dim 16j+n] and its own probability of token 4g+i,
+// so probabilities never leave their lane and the state of query row n lives in lanes (n, 0..3).
+// The four waves of a workgroup take four row groups, or split the keys of fewer row groups among
+// themselves (few query rows: decode) and merge through LDS.  Operands come straight from global
+// memory: at 32 cycles per matrix instruction their traffic is far from any limit.
+#include "attn_core.h"
 
 namespace pace_kv {
-
-constexpr int kRows = 16;
 
 template <typename T>
 __device__ __forceinline__ float load_f32(const T* p);
@@ -20,6 +29,18 @@ __device__ __forceinline__ float load_f32<float>(const float* p) {
 template <>
 __device__ __forceinline__ float load_f32<uint16_t>(const uint16_t* p) {
   return bf16_bits_to_f32(*p);
+}
+
+// Four consecutive elements as fp32 (p 16- resp. 8-byte aligned).
+__device__ __forceinline__ f32x4 load4_f32(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 load4_f32(const uint16_t* p) {
+  const u32x2 w = *reinterpret_cast<const u32x2*>(p);
+  return f32x4{bf16_bits_to_f32(w[0] & 0xffffu), __uint_as_float(w[0] & 0xffff0000u), bf16_bits_to_f32(w[1] & 0xffffu),
+               __uint_as_float(w[1] & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4_out(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void store4_out(uint16_t* p, f32x4 v) {
+  *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
 }
 __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_out(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
@@ -32,104 +53,153 @@ struct DenseParams {
   const void* mask;
   int32_t B, N, S, L, H;
   int32_t mB, mN, mS;
-  int32_t TL;  // tokens per chunk
+  int32_t l_split;  // waves of a workgroup that share one row group and split its keys: 1, 2 or 4
   float scale;
 };
 
-template <typename T, typename MT>
-__global__ __launch_bounds__(256) void attn_dense_kernel(const DenseParams p) {
-  extern __shared__ float smem[];
-  const int H = p.H, L = p.L, TL = p.TL;
-  float* qs = smem;                        // [kRows][H]
-  float* kv = qs + kRows * H;              // [TL][H + 1]
-  float* sc = kv + TL * (H + 1);           // [kRows][TL + 1]
-  float* row_m = sc + kRows * (TL + 1);    // [kRows]
-  float* row_l = row_m + kRows;            // [kRows]
-  float* row_a = row_l + kRows;            // [kRows]
-  const int tid = threadIdx.x;
-  const int s0 = blockIdx.x * kRows, n = blockIdx.y, b = blockIdx.z;
-  const int rows = min(kRows, p.S - s0);
-  const T* q = static_cast<const T*>(p.q) + (((int64_t)b * p.N + n) * p.S + s0) * H;
-  const T* k = static_cast<const T*>(p.k) + ((int64_t)b * p.N + n) * (int64_t)L * H;
-  const T* v = static_cast<const T*>(p.v) + ((int64_t)b * p.N + n) * (int64_t)L * H;
-  T* out = static_cast<T*>(p.out) + (((int64_t)b * p.N + n) * p.S + s0) * H;
-  const MT* mask = static_cast<const MT*>(p.mask);
-  const int64_t m_b = p.mB == 1 ? 0 : b, m_n = p.mN == 1 ? 0 : n;
-
-  for (int i = tid; i < kRows * H; i += 256) qs[i] = (i / H) < rows ? load_f32<T>(q + i) : 0.f;
-  if (tid < kRows) {
-    row_m[tid] = -__builtin_inff();
-    row_l[tid] = 0.f;
+// HP: head size rounded up to the next size built (dims >= H read as zero).  VEC: H is a multiple
+// of 4, so a lane's run of a row can be read four elements at a time.
+template <typename T, typename MT, int HP, bool VEC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_kernel(
+    const DenseParams p) {
+  constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
+  constexpr int MTL = HP / 16;  // 16-dim output tiles
+  constexpr int ROW_F = HP + 2;
+  __shared__ float merge_buf[2 * 16 * ROW_F];
+  const int H = p.H, L = p.L, S = p.S;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
+  const int split = p.l_split;
+  const int head = blockIdx.y, b = blockIdx.z;
+  const int rowgroup = blockIdx.x * (4 / split) + wave / split, ls = wave % split;
+  const int row = rowgroup * 16 + n;
+  const bool valid = row < S;
+  const int64_t pair = (int64_t)b * p.N + head;
+  const T* qrow = static_cast<const T*>(p.q) + (pair * S + (valid ? row : 0)) * H;
+  const T* kbase = static_cast<const T*>(p.k) + pair * (int64_t)L * H;
+  const T* vbase = static_cast<const T*>(p.v) + pair * (int64_t)L * H;
+  const MT* mrow = nullptr;
+  if (p.mask) {
+    const int64_t mb = p.mB == 1 ? 0 : b, mn = p.mN == 1 ? 0 : head, ms = p.mS == 1 ? 0 : (valid ? row : 0);
+    mrow = static_cast<const MT*>(p.mask) + ((mb * p.mN + mn) * p.mS + ms) * (int64_t)L;
   }
-  // Output ownership: thread (r, c) = (tid / 16, tid % 16) accumulates dims c, c+16, ...
-  const int r_own = tid >> 4, c_own = tid & 15;
-  constexpr int kMaxOwn = 16;  // H <= 256
-  float acc[kMaxOwn];
+  // This lane's dims of a row for the first product: d0 .. d0 + KS - 1.
+  const int d0 = g * KS;
+  auto load_run = [&](const T* r, float (&x)[KS]) {
 #pragma unroll
-  for (int i = 0; i < kMaxOwn; ++i) acc[i] = 0.f;
-  __syncthreads();
+    for (int s4 = 0; s4 < KS; s4 += 4) {
+      const int d = d0 + s4;
+      if (VEC && d + 4 <= H) {
+        const f32x4 t = load4_f32(r + d);
+        x[s4] = t[0], x[s4 + 1] = t[1], x[s4 + 2] = t[2], x[s4 + 3] = t[3];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[s4 + e] = (d + e < H) ? load_f32<T>(r + d + e) : 0.f;
+      }
+    }
+  };
+  float qf[KS];
+  load_run(qrow, qf);
+  if (!valid) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = 0.f;
+  }
+  f32x4 o[MTL];
+#pragma unroll
+  for (int j = 0; j < MTL; ++j) o[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = kNegInf, l_run = 0.f;
 
-  for (int l0 = 0; l0 < L; l0 += TL) {
-    const int nt = min(TL, L - l0);
-    for (int i = tid; i < nt * H; i += 256) kv[(i / H) * (H + 1) + (i % H)] = load_f32<T>(k + (int64_t)l0 * H + i);
-    __syncthreads();
-    for (int idx = tid; idx < kRows * TL; idx += 256) {
-      const int r = idx / TL, t = idx % TL;
-      float val = -__builtin_inff();
-      if (r < rows && t < nt) {
-        float dot = 0.f;
-        const float* qr = qs + r * H;
-        const float* kr = kv + t * (H + 1);
-        for (int h = 0; h < H; ++h) dot += qr[h] * kr[h];
-        val = dot * p.scale;
-        if (mask) {
-          const int64_t m_s = p.mS == 1 ? 0 : (s0 + r);
-          val += load_f32<MT>(mask + ((m_b * p.mN + m_n) * p.mS + m_s) * (int64_t)L + l0 + t);
-        }
-      }
-      sc[r * (TL + 1) + t] = val;
-    }
-    __syncthreads();
-    for (int i = tid; i < nt * H; i += 256) kv[(i / H) * (H + 1) + (i % H)] = load_f32<T>(v + (int64_t)l0 * H + i);
-    if (tid < kRows) {
-      float* sr = sc + tid * (TL + 1);
-      float mx = row_m[tid];
-      for (int t = 0; t < nt; ++t) mx = fmaxf(mx, sr[t]);
-      const float m_use = (mx == -__builtin_inff()) ? 0.f : mx;
-      const float alpha = expf(row_m[tid] - m_use);
-      float sum = 0.f;
-      for (int t = 0; t < nt; ++t) {
-        const float e = expf(sr[t] - m_use);
-        sr[t] = e;
-        sum += e;
-      }
-      row_m[tid] = mx;
-      row_l[tid] = row_l[tid] * alpha + sum;
-      row_a[tid] = alpha;
-    }
-    __syncthreads();
-    {
-      const float alpha = row_a[r_own];
-      const float* pr = sc + r_own * (TL + 1);
+  // This wave's share of the 16-token tiles.
+  const int tiles = (L + 15) / 16, per = (tiles + split - 1) / split;
+  const int tile_lo = min(tiles, ls * per), tile_hi = min(tiles, tile_lo + per);
+  const bool has_rows = rowgroup * 16 < S;  // wave-uniform
+  for (int tile = tile_lo; has_rows && tile < tile_hi; ++tile) {
+    const int t0 = tile * 16;
+    float kf[KS];
+    load_run(kbase + (int64_t)min(L - 1, t0 + n) * H, kf);  // rows past the end are masked below
+    float vf[MTL][4];
 #pragma unroll
-      for (int i = 0; i < kMaxOwn; ++i) {
-        const int d = c_own + 16 * i;
-        if (d < H) {
-          float a = acc[i] * alpha;
-          for (int t = 0; t < nt; ++t) a += pr[t] * kv[t * (H + 1) + d];
-          acc[i] = a;
-        }
-      }
+    for (int i = 0; i < 4; ++i) {
+      const T* vr = vbase + (int64_t)min(L - 1, t0 + 4 * g + i) * H + n;
+#pragma unroll
+      for (int j = 0; j < MTL; ++j) vf[j][i] = (16 * j + n < H) ? load_f32<T>(vr + 16 * j) : 0.f;
+    }
+    float mv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + 4 * g + i;
+      mv[i] = (mrow && t < L) ? load_f32<MT>(mrow + t) : 0.f;
+    }
+    f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], sc, 0, 0, 0);
+    float val[4], mx = kNegInf;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      val[i] = (t0 + 4 * g + i < L) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
+      mx = fmaxf(mx, val[i]);
+    }
+    mx = row_max4(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = expf(m_run - m_use);
+    float pr[4], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = expf(val[i] - m_use);
+      sum += pr[i];
+    }
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int j = 0; j < MTL; ++j) {
+      o[j] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j][i], pr[i], o[j], 0, 0, 0);
+    }
+  }
+  // row sum over the four lanes of a row
+  l_run += xor_lanes(l_run, 16);
+  l_run += xor_lanes(l_run, 32);
+
+  // Merge the key shares of a row group (fixed order: deterministic).  Every wave passes the same barriers.
+  for (int stride = 1; stride < split; stride *= 2) {
+    const bool sender = (ls & (2 * stride - 1)) == stride;
+    const bool receiver = (ls & (2 * stride - 1)) == 0 && ls + stride < split;
+    float* slot = merge_buf + (wave / (2 * stride)) * 16 * ROW_F + n * ROW_F;
+    if (sender) {
+#pragma unroll
+      for (int j = 0; j < MTL; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) slot[16 * j + 4 * g + c] = o[j][c];
+      if (g == 0) slot[HP] = m_run, slot[HP + 1] = l_run;
+    }
+    __syncthreads();
+    if (receiver) {
+      const float m_b = slot[HP], l_b = slot[HP + 1];
+      const float m_new = fmaxf(m_run, m_b);
+      const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+      const float wa = expf(m_run - m_use), wb = expf(m_b - m_use);
+#pragma unroll
+      for (int j = 0; j < MTL; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o[j][c] = o[j][c] * wa + slot[16 * j + 4 * g + c] * wb;
+      l_run = l_run * wa + l_b * wb;
+      m_run = m_new;
     }
     __syncthreads();
   }
-  if (r_own < rows) {
-    const float l = row_l[r_own];
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+  if (ls != 0 || !valid) return;
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  T* orow = static_cast<T*>(p.out) + (pair * S + row) * H;
 #pragma unroll
-    for (int i = 0; i < kMaxOwn; ++i) {
-      const int d = c_own + 16 * i;
-      if (d < H) store_out(out + (int64_t)r_own * H + d, acc[i] * inv);
+  for (int j = 0; j < MTL; ++j) {
+    const int d = 16 * j + 4 * g;
+    if (VEC && d + 4 <= H) {
+      store4_out(orow + d, o[j] * inv);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (d + c < H) store_out(orow + d + c, o[j][c] * inv);
     }
   }
 }
@@ -155,8 +225,8 @@ extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void
   }
   PACE_REQUIRE(B <= 65535 && N <= 65535, "pace_attn_dense: batch / heads exceed grid limits");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // bf16 with head_dim 64 / 128 runs on the matrix cores; everything else (fp32, other head
-  // sizes) takes the general kernel below.
+  // bf16 with head_dim 64 / 96 / 128 / 256 runs on the bf16 matrix-core kernels; everything else (fp32,
+  // other head sizes) takes the general kernel below.
   if (qkv_dtype == PACE_DTYPE_BF16 &&
       launch_dense_mfma(q, k, v, out, B, N, S, L, H, mask, mask_dtype == PACE_DTYPE_F32, mB, mN, mS,
                         1.0f / sqrtf((float)H), s)) {
@@ -167,20 +237,34 @@ extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void
   p.q = q, p.k = k, p.v = v, p.out = out, p.mask = mask;
   p.B = B, p.N = N, p.S = S, p.L = L, p.H = H;
   p.mB = mB, p.mN = mN, p.mS = mS;
-  p.TL = H > 128 ? 32 : 64;
   p.scale = 1.0f / sqrtf((float)H);
-  const size_t smem = ((size_t)kRows * H + (size_t)p.TL * (H + 1) + (size_t)kRows * (p.TL + 1) + 3 * kRows) * sizeof(float);
-  dim3 grid((S + kRows - 1) / kRows, N, B);
+  // Few query rows: the four waves of a workgroup split the keys of one row group (or of two).
+  p.l_split = S <= 16 ? 4 : (S <= 32 ? 2 : 1);
+  const int rowgroups = (S + 15) / 16, per_wg = 4 / p.l_split;
+  dim3 grid((rowgroups + per_wg - 1) / per_wg, N, B);
   const bool f32 = qkv_dtype == PACE_DTYPE_F32;
   const bool mf32 = mask_dtype == PACE_DTYPE_F32;
-  if (f32 && mf32)
-    hipLaunchKernelGGL((attn_dense_kernel<float, float>), grid, dim3(256), smem, s, p);
-  else if (f32)
-    hipLaunchKernelGGL((attn_dense_kernel<float, uint16_t>), grid, dim3(256), smem, s, p);
-  else if (mf32)
-    hipLaunchKernelGGL((attn_dense_kernel<uint16_t, float>), grid, dim3(256), smem, s, p);
-  else
-    hipLaunchKernelGGL((attn_dense_kernel<uint16_t, uint16_t>), grid, dim3(256), smem, s, p);
+  // vector accesses need rows that start on a 16-byte (fp32) / 8-byte (bf16) boundary
+  const size_t row_align = f32 ? 16 : 8;
+  const bool vec = H % 4 == 0 && ((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % row_align == 0;
+#define PACE_DENSE_GO(T_, MT_, HP_) \
+  do { \
+    if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true>), grid, dim3(256), 0, s, p); \
+    else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false>), grid, dim3(256), 0, s, p); \
+  } while (0)
+#define PACE_DENSE_HP(T_, MT_) \
+  do { \
+    if (H <= 32) PACE_DENSE_GO(T_, MT_, 32); \
+    else if (H <= 64) PACE_DENSE_GO(T_, MT_, 64); \
+    else if (H <= 128) PACE_DENSE_GO(T_, MT_, 128); \
+    else PACE_DENSE_GO(T_, MT_, 256); \
+  } while (0)
+  if (f32 && mf32) PACE_DENSE_HP(float, float);
+  else if (f32) PACE_DENSE_HP(float, uint16_t);
+  else if (mf32) PACE_DENSE_HP(uint16_t, float);
+  else PACE_DENSE_HP(uint16_t, uint16_t);
+#undef PACE_DENSE_HP
+#undef PACE_DENSE_GO
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }

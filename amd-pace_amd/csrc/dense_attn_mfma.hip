@@ -1,4 +1,4 @@
-// Dense bf16 attention on the matrix cores for head_dim 64 / 128: the fast path of the torch op
+// Dense bf16 attention on the matrix cores for head_dim 64 / 96 / 128 / 256: the fast path of the torch op
 // pace::attention (dense_attn.hip holds the general kernel and the entry point).
 #include <type_traits>
 
@@ -23,14 +23,20 @@ struct DenseMfmaParams {
 };
 
 // ONCE: one group of query rows per (batch, head), so K / V are read once and fetched non-temporally.
+// Waves per workgroup: four; two with head_dim 256, where a wave has a SIMD (and its 512 registers) to itself
+// and the V stages of four would not fit the LDS a workgroup may have.
+template <int D>
+constexpr int dense_split_waves() { return D > 128 ? 2 : 4; }
+
 template <int D, int NQT, bool HAS_MASK, bool ONCE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_mfma_kernel(const DenseMfmaParams dp) {
+__global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : 2))) void dense_attn_mfma_kernel(
+    const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
-  constexpr int NW = 4;
+  constexpr int NW = dense_split_waves<D>();
   constexpr int VROW = D + 24;                    // padded LDS row (elements): keeps the transposed reads off each other's banks
   constexpr int STAGE = 32 * VROW;                // one wave's V unit
-  constexpr int MERGE_FLOATS = 2 * 16 * NQT * (D + 2);
+  constexpr int MERGE_FLOATS = (NW / 2) * 16 * NQT * (D + 2);
   constexpr int LDS_BYTES = (NW * STAGE * 2 > MERGE_FLOATS * 4) ? NW * STAGE * 2 : MERGE_FLOATS * 4;
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[LDS_BYTES];
   const PagedAttnParams& p = dp.base;
@@ -436,7 +442,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 // Launches the dense bf16 kernel; returns false when the shape is not one it handles.
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
                        const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream) {
-  if ((H != 64 && H != 128) || L < 1) return false;
+  if ((H != 64 && H != 96 && H != 128 && H != 256) || L < 1) return false;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(out) & 7u)) return false;
   DenseMfmaParams dp = {};
   dp.base.q = static_cast<const uint16_t*>(q);
@@ -447,7 +453,8 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
-  if (tiles > 4) {
+  const bool coop_built = H == 64 || H == 128;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
+  if (tiles > 4 && coop_built) {
     // prefill-sized: rows of a head share its K / V through LDS
     const int mode = !mask ? 0 : (mask_is_f32 ? 1 : 2);
     int cnqt = 2;
@@ -471,22 +478,25 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
 #undef PACE_COOP
     return true;
   }
-  const int nqt = tiles >= 2 ? 2 : 1;
+  const int nqt = (tiles >= 2 && H != 256) ? 2 : 1;  // two tiles of head_dim 256 do not fit the register file
   dp.n_qgroups = (tiles + nqt - 1) / nqt;
   const long long blocks = (long long)B * N * dp.n_qgroups;
   if (blocks >= (1ll << 31)) return false;
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks), block(H > 128 ? 128 : 256);
   const bool m = mask != nullptr;
   const bool once = dp.n_qgroups == 1;
 #define PACE_DENSE1(D_, Q_, M_, O_) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_>), grid, block, 0, stream, dp)
 #define PACE_DENSE(D_, Q_, M_) do { if (once) PACE_DENSE1(D_, Q_, M_, true); else PACE_DENSE1(D_, Q_, M_, false); } while (0)
-  if (H == 128) {
-    if (nqt == 2) { if (m) PACE_DENSE(128, 2, true); else PACE_DENSE(128, 2, false); }
-    else { if (m) PACE_DENSE(128, 1, true); else PACE_DENSE(128, 1, false); }
-  } else {
-    if (nqt == 2) { if (m) PACE_DENSE(64, 2, true); else PACE_DENSE(64, 2, false); }
-    else { if (m) PACE_DENSE(64, 1, true); else PACE_DENSE(64, 1, false); }
-  }
+  for_head_dim(H, [&](auto d) {
+    constexpr int DIM = decltype(d)::value;
+    if constexpr (DIM != 256) {
+      if (nqt == 2) {
+        if (m) PACE_DENSE(DIM, 2, true); else PACE_DENSE(DIM, 2, false);
+        return;
+      }
+    }
+    if (m) PACE_DENSE(DIM, 1, true); else PACE_DENSE(DIM, 1, false);
+  });
 #undef PACE_DENSE1
 #undef PACE_DENSE
   return true;

@@ -19,6 +19,7 @@ def _mask(seed, shape, dtype):
 CASES = [
     (1, 1, 1, 1, 1), (1, 16, 128, 64, 512), (32, 1, 1, 128, 2048), (2, 32, 512, 128, 1), (3, 2, 17, 1, 33),
     (2, 16, 1, 64, 2048), (96, 1, 1, 64, 1), (1, 1, 128, 128, 512), (2, 3, 5, 80, 70), (1, 2, 33, 256, 40),
+    (2, 4, 1, 96, 700), (1, 3, 100, 96, 333), (2, 2, 1, 256, 900), (1, 2, 70, 256, 130), (1, 2, 9, 100, 50),
 ]
 
 
@@ -174,7 +175,7 @@ def test_dense_op_random_shapes_and_masks(device, seed):
         B, N = int(rng.integers(1, 4)), int(rng.integers(1, 10))
         S = int(rng.choice([1, 3, 8, 17, 40, 64, 65, 100, 130, 260]))
         L = int(rng.choice([1, 7, 31, 32, 33, 64, 100, 129, 256, 300]))
-        H = int(rng.choice([64, 128, 128, 80]))
+        H = int(rng.choice([64, 128, 128, 80, 96, 256]))
         dt = torch.bfloat16
         mdt = torch.bfloat16 if rng.random() < 0.7 else torch.float32
         kind = kinds[int(rng.integers(len(kinds)))]
