@@ -17,6 +17,7 @@ Other workloads (same JSON shape, `config.workload` names them):
   prefill / dense-prefill   a 512-token chunk over 3584 cached tokens through the paged path; the dense
             op on 2048 x 2048 with the additive causal mask (roofline against the matrix-core peak)
   decode-gptj   the headline step at GPT-J-6B's attention shape (16 heads of 256, batch 64 x 2048)
+  dense-f32     the dense op on fp32 tensors (the general kernel; roofline against the fp32 matrix-core peak)
   compact   Llama-3-70B-shape KV, batch 8, context 32768: evict 40% of the blocks, then time the
             compaction copy and the decode over the compacted cache
   copy-calibration   block copy of a known byte count, used to scale the HBM byte counters
@@ -38,6 +39,7 @@ for _p in (REPO, os.path.join(REPO, "amd-pace_amd")):
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix-core peak, published
+MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X fp32 matrix-core peak, published
 METRIC = "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 1 GPU"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, scaled by the
@@ -445,6 +447,35 @@ def wl_dense_prefill(torch, dev, args):
          "tflops_if_all_pairs_counted": round(all_pairs / (attn_ms * 1e-3) / 1e12, 1)})
 
 
+def wl_dense_f32(torch, dev, args):
+    """The reference's own op on fp32 tensors (its tests' dtype, tests/ops/test_sdpa.py:83-127): the general
+    kernel, fp32 arithmetic on the matrix cores.  Mask [B,1,1,L] as in the reference's test."""
+    import pace_mi355.ops  # noqa: F401  (defines the op)
+
+    B, N, S, L, H = 8, 32, 512, 512, 128
+    g = torch.Generator(device=dev).manual_seed(11)
+    q, k, v = (torch.randn(B, N, n, H, generator=g, device=dev) for n in (S, L, L))
+    mask = torch.randn(B, 1, 1, L, generator=g, device=dev)
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        torch.ops.pace.attention(q, k, v, mask, False)
+        if ev:
+            ev[1].record()
+
+    dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
+    flops = 4.0 * B * N * S * L * H
+    once = 4 * (2 * q.numel() + k.numel() + v.numel()) + 4 * mask.numel()
+    tflops = flops / (attn_ms * 1e-3) / 1e12
+    return result_line(
+        args, "dense op on fp32 tensors: batch 8, 32 heads, 512 queries x 512 keys, head_dim 128, additive mask [B,1,1,L]; "
+        "step = one torch.ops.pace.attention call (output allocation included)", once, B * S, dt,
+        {"bound": "mfma", "kernel": "attn_dense_kernel<float,float,128,true>", "achieved": round(tflops, 1),
+         "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_F32_PEAK_TFLOPS, 4), "traffic": None,
+         "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5)}, extra={"dtype": "f32"})
+
+
 def wl_compact(torch, dev, args):
     import numpy as np
 
@@ -560,7 +591,7 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
     }
 
 
-WORKLOADS = {"decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill,
+WORKLOADS = {"decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32,
              "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 
