@@ -23,12 +23,10 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("B,N,S,H,L", CASES)
+# use_KQ selects an experimental path of the same function in the reference: two shapes suffice for it
+@pytest.mark.parametrize("B,N,S,H,L,use_kq", [c + (False,) for c in CASES] + [CASES[1] + (True,), CASES[4] + (True,)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("use_kq", [False, True])
 def test_dense_op_matches_oracle(device, B, N, S, H, L, dtype, use_kq):
-    if use_kq and (B, N, S, H, L) not in (CASES[1], CASES[4]):
-        pytest.skip("use_KQ selects an experimental path of the same function; two shapes suffice")
     k, v = seeded_kv(1, B, N, L, H, dtype)
     q = seeded_q(2, B, N, S, H, dtype)
     m = _mask(3, (B, 1, 1, L), dtype)  # the reference test's mask: random additive bias of shape (B,1,1,L)
