@@ -310,6 +310,8 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 
   typedef short tr_v4 __attribute__((ext_vector_type(4)));
   typedef tr_v4 __attribute__((address_space(3))) * tr_ptr;
+  int opaque_zero;
+  asm volatile("s_mov_b32 %0, 0" : "=s"(opaque_zero));
   // One unit out of its stage: K rows in operand order for the scores; V comes back token-minor
   // only once the score products are issued, into the registers the K rows leave.
   auto unit = [&](int cur, int t0, auto full_tag) {
@@ -329,8 +331,15 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       for (int kk = 0; kk < KK; ++kk) kop[t][kk] = *reinterpret_cast<const u32x4*>(ks + t * 4 * KROW + kk * 32);
     f32x4 sc[NQT][2];
     score_products<D, NQT>(kop, qreg, sc);
+    // The V reads below land in registers the score products have just been issued from.  Nothing holds an LDS
+    // read back until a matrix instruction in flight has fetched its operands (one that waits in the pipeline for
+    // the accumulator of the instruction before it fetches them late), and now and then a V value arrived first:
+    // one tile's scores came out slightly wrong, differently from run to run.  So the address of the V reads is
+    // made to depend on the last score product's result (an "and" with a zero the compiler cannot see through):
+    // reading that result waits for the instruction, and the ones issued before it, to complete.
+    const int done = __builtin_amdgcn_readfirstlane(__float_as_int(sc[NQT - 1][1][3])) & opaque_zero;
     // V: dim 16j + n of tokens 8g .. 8g+7 (see the transposed read in the kernel above)
-    const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3)];
+    const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3) + done];
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       const tr_v4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 16 * j));
