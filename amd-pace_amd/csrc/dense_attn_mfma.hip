@@ -335,9 +335,12 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     // read back until a matrix instruction in flight has fetched its operands (one that waits in the pipeline for
     // the accumulator of the instruction before it fetches them late), and now and then a V value arrived first:
     // one tile's scores came out slightly wrong, differently from run to run.  So the address of the V reads is
-    // made to depend on the last score product's result (an "and" with a zero the compiler cannot see through):
-    // reading that result waits for the instruction, and the ones issued before it, to complete.
-    const int done = __builtin_amdgcn_readfirstlane(__float_as_int(sc[NQT - 1][1][3])) & opaque_zero;
+    // made to depend on every score tile's result (an "and" with a zero the compiler cannot see through):
+    // reading the results waits for the instructions to complete, in whatever order the compiler issued them.
+    int all_scores = 0;
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) all_scores |= __float_as_int(sc[qt][0][3]) | __float_as_int(sc[qt][1][3]);
+    const int done = __builtin_amdgcn_readfirstlane(all_scores) & opaque_zero;
     // V: dim 16j + n of tokens 8g .. 8g+7 (see the transposed read in the kernel above)
     const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3) + done];
 #pragma unroll
