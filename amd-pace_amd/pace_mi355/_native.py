@@ -15,6 +15,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
 ABI_VERSION = 8
+HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
 EXPORTED_SYMBOLS = (
     "pace_kv_last_error",

@@ -99,7 +99,7 @@ class PagedKVView:
     @property
     def shape(self) -> Tuple[int, int, int, int]:
         c = self.cache
-        return (c.batch, c.num_kv_heads * c.n_rep, int(c.lens.max(initial=0)), c.head_dim)
+        return (c.batch, c.num_kv_heads * c.n_rep, int(c.lens.max(initial=0)), c.model_dim)
 
     def size(self, dim: int) -> int:
         return self.shape[dim]
@@ -145,7 +145,8 @@ class PagedKVCache(KVCacheBase):
         self.batch = 0
         self.num_kv_heads = 0
         self.n_rep = 1
-        self.head_dim = 0
+        self.head_dim = 0   # head size of the pool: one the kernels are built for
+        self.model_dim = 0  # head size of the caller's tensors (smaller where it is not such a size: zero-padded)
         self.partition_tokens = 0  # 0: let the library choose
         # Appends of up to 32 tokens are held back until the attention call that follows, which
         # reads them from the caller's tensors and stores them into the pool in the same launch;
@@ -184,7 +185,12 @@ class PagedKVCache(KVCacheBase):
             hkv = h_in
         if h_in % hkv:
             raise RuntimeError(f"{h_in} input heads cannot be reduced to {hkv} KV heads")
-        self.batch, self.num_kv_heads, self.head_dim = int(B), hkv, int(D)
+        self.batch, self.num_kv_heads, self.model_dim = int(B), hkv, int(D)
+        # e.g. 80 (OPT-2.7B) is kept in slabs of 96: zero dims change neither a score nor an output
+        self.head_dim = next((d for d in nat.HEAD_DIMS if d >= D), 0)
+        if not self.head_dim:
+            raise RuntimeError(f"head_dim {D} unsupported (at most {nat.HEAD_DIMS[-1]})")
+        D = self.head_dim
         self.n_rep = int(self._cfg_n_rep) if self._cfg_n_rep is not None else h_in // hkv
         if "state" not in self._shared:
             self._shared["state"] = PagedState(B, self.max_seq_length, self._cfg_num_blocks, key_states.device)
@@ -261,10 +267,14 @@ class PagedKVCache(KVCacheBase):
         B, h_in, T, D = k.shape
         if rope is not None and (counts is not None or tuple(rope.rows.shape) != (B, T)):
             raise RuntimeError("rope rows must be [B, T] and cannot be combined with per-sequence counts")
-        if B != self.batch or D != self.head_dim or h_in % self.num_kv_heads:
+        if B != self.batch or D != self.model_dim or h_in % self.num_kv_heads:
             raise RuntimeError(f"update of shape {tuple(k.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={D}]")
         if v.shape != k.shape:
             raise RuntimeError("key_states and value_states differ in shape")
+        if self.head_dim != self.model_dim:
+            if rope is not None:
+                raise NotImplementedError("rotary embedding with a zero-padded head size")
+            k, v = (torch.nn.functional.pad(t, (0, self.head_dim - self.model_dim)) for t in (k, v))
         if k.stride(3) != 1 or v.stride(3) != 1 or k.stride() != v.stride() or any(s % 8 for s in k.stride()[:3]):
             k, v = k.contiguous(), v.contiguous()
         head_step = h_in // self.num_kv_heads  # de-duplicate a repeat_kv-expanded input
@@ -412,6 +422,7 @@ class PagedKVCache(KVCacheBase):
         n_rep = self.n_rep if n_rep is None else int(n_rep)
         L = int(self.lens.max(initial=0)) if pad_to is None else int(pad_to)
         shape = (self.batch, self.num_kv_heads * n_rep, L, self.head_dim)
+        padded = self.head_dim != self.model_dim
         k = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
         v = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
         if L:
@@ -423,6 +434,8 @@ class PagedKVCache(KVCacheBase):
                     k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, nat.current_stream_ptr(),
                 )
             )
+        if padded:
+            k, v = k[..., : self.model_dim].contiguous(), v[..., : self.model_dim].contiguous()
         return k, v
 
     def _plan(self, B: int, hq: int, S: int, D: int, max_len: int):
@@ -473,8 +486,10 @@ class PagedKVCache(KVCacheBase):
         if query.dim() != 4 or query.dtype != torch.bfloat16 or not query.is_cuda:
             raise RuntimeError("paged attention expects a bf16 device tensor [B, Hq, S, D]")
         B, hq, S, D = query.shape
-        if B != self.batch or D != self.head_dim or hq % self.num_kv_heads:
-            raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.head_dim}]")
+        if B != self.batch or D != self.model_dim or hq % self.num_kv_heads:
+            raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.model_dim}]")
+        if self.head_dim != self.model_dim:
+            query, D = torch.nn.functional.pad(query, (0, self.head_dim - self.model_dim)), self.head_dim
         if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
             query = query.contiguous()
         rope, self._query_rope = self._query_rope, None
@@ -524,7 +539,7 @@ class PagedKVCache(KVCacheBase):
             a.work_items, a.n_work_items = items.data_ptr(), items.shape[0]
         if parts is not None:
             a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
-        a.scale = 1.0 / math.sqrt(D)
+        a.scale = 1.0 / math.sqrt(self.model_dim)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes
         if rope_desc is not None:
@@ -538,7 +553,7 @@ class PagedKVCache(KVCacheBase):
             a.new_stride_b, a.new_stride_h, a.new_stride_t = k.stride(0), k.stride(1) * head_step, k.stride(2)
         fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
         nat.check(fn(ctypes.byref(self._desc), ctypes.byref(a), nat.current_stream_ptr()))
-        return out
+        return out if self.head_dim == self.model_dim else out[..., : self.model_dim].contiguous()
 
 
 class KVCacheManager:

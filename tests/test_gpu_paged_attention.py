@@ -40,6 +40,7 @@ def _build(device, B, hkv, n_rep, D, lens, seed, partition=0, num_blocks=None, s
         (3, 4, 1, 96, [700, 31, 1500], 256),          # head_dim 96 (Phi-3-mini's heads), several partitions
         (2, 2, 4, 96, [129, 4100], 0),                # head_dim 96 with a GQA group
         (2, 1, 40, 96, [95, 300], 128),               # head_dim 96, three query tiles
+        (3, 4, 1, 80, [700, 31, 1500], 256),          # head_dim 80 (OPT-2.7B's heads): kept zero-padded in slabs of 96
     ],
 )
 def test_decode_matches_oracle(device, B, hkv, n_rep, D, lens, partition):
@@ -227,7 +228,7 @@ def test_decode_invariant_to_physical_block_permutation(device):
                                                   (8, 8, [31, 700], 256, 128), (9, 9, [100, 64], 0, 128), (16, 1, [5, 48], 0, 128),
                                                   (32, 32, [33, 500], 0, 128), (1, 1, [40, 200, 1029, 16], 0, 256),
                                                   (5, 5, [31, 700], 256, 256), (1, 1, [77, 130], 0, 64),
-                                                  (1, 1, [77, 1300], 0, 96), (7, 7, [40, 600], 256, 96)])
+                                                  (1, 1, [77, 1300], 0, 96), (7, 7, [40, 600], 256, 96), (1, 1, [77, 300], 0, 80)])
 def test_fused_append_equals_append_then_attend(device, T, S, lens, partition, D):
     """update_cache holds the new tokens back and the attention launch both reads them from the
     caller's tensors and stores them: same attention result as append-then-attend (to tolerance, the

@@ -17,7 +17,7 @@ def _paged(max_len, **kw):
     return PagedKVCache(max_len, **kw)
 
 
-@pytest.mark.parametrize("hkv,n_rep,dim", [(8, 4, 128), (2, 1, 64), (4, 8, 128), (4, 1, 256), (2, 4, 96)])
+@pytest.mark.parametrize("hkv,n_rep,dim", [(8, 4, 128), (2, 1, 64), (4, 8, 128), (4, 1, 256), (2, 4, 96), (2, 2, 80)])
 def test_append_matches_reference_dynamic_cache(device, hkv, n_rep, dim):
     """Feed the same GQA-expanded stream to the reference's DynamicKVCache restatement
     and to the paged cache; gather(expand) must equal the reference tensors bit for bit."""
