@@ -250,3 +250,19 @@ def test_longrope_rows_follow_the_reference_switch(device):
         qo, _ = rope(q.to(device), None)
         cos, sin = rope_ref.lookup(mod.cos_cache, mod.sin_cache, rows, torch.bfloat16)
         assert_bits_equal(qo, rope_ref.rotate_longrope_form(q, cos, sin, 64), "longrope")
+
+
+def test_rope_with_a_zero_padded_head_size_is_refused(device):
+    """Head sizes the kernels are not built for are kept zero-padded by PagedKVCache; the rotation has no such
+    path and must say so instead of rotating padded rows."""
+    from pace_mi355.llm import PagedKVCache
+
+    B, hkv, D, T = 2, 2, 80, 5
+    k, v = seeded_kv(1, B, hkv, T, D)
+    cache = PagedKVCache(64, num_kv_heads=hkv, n_rep=1)
+    mod = _module(64, rows=64)
+    rope = mod(k.to(device)[..., :64], torch.arange(T).repeat(B, 1).to(device))
+    with pytest.raises(NotImplementedError, match="zero-padded head size"):
+        cache.update_cache(k.to(device), v.to(device), 2, rope=rope)
+    pk, pv = cache.update_cache(k.to(device), v.to(device), 2)  # without rotation it is stored and read back as given
+    assert_bits_equal(pk.dense(), k, "K of head size 80")
