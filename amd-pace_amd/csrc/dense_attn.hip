@@ -59,7 +59,10 @@ struct DenseParams {
 
 // HP: head size rounded up to the next size built (dims >= H read as zero).  VEC: H is a multiple
 // of 4, so a lane's run of a row can be read four elements at a time.
-template <typename T, typename MT, int HP, bool VEC>
+// AHEAD: the operands of the next tile are fetched while this one is computed (a second set of registers: one
+// wave per SIMD at head size 128).  It pays where the launch is bound by memory (few query rows: +8 % on an fp32
+// decode step) and costs 10 % where it is bound by the matrix cores, so the launcher picks.
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_kernel(
     const DenseParams p) {
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
@@ -112,22 +115,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   const int tiles = (L + 15) / 16, per = (tiles + split - 1) / split;
   const int tile_lo = min(tiles, ls * per), tile_hi = min(tiles, tile_lo + per);
   const bool has_rows = rowgroup * 16 < S;  // wave-uniform
-  for (int tile = tile_lo; has_rows && tile < tile_hi; ++tile) {
+  float kf[KS], vf[MTL][4], mv[4];
+  auto fetch = [&](int tile, float (&kx)[KS], float (&vx)[MTL][4], float (&mx4)[4]) {
     const int t0 = tile * 16;
-    float kf[KS];
-    load_run(kbase + (int64_t)min(L - 1, t0 + n) * H, kf);  // rows past the end are masked below
-    float vf[MTL][4];
+    load_run(kbase + (int64_t)min(L - 1, t0 + n) * H, kx);  // rows past the end are masked below
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const T* vr = vbase + (int64_t)min(L - 1, t0 + 4 * g + i) * H + n;
 #pragma unroll
-      for (int j = 0; j < MTL; ++j) vf[j][i] = (16 * j + n < H) ? load_f32<T>(vr + 16 * j) : 0.f;
+      for (int j = 0; j < MTL; ++j) vx[j][i] = (16 * j + n < H) ? load_f32<T>(vr + 16 * j) : 0.f;
     }
-    float mv[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int t = t0 + 4 * g + i;
-      mv[i] = (mrow && t < L) ? load_f32<MT>(mrow + t) : 0.f;
+      mx4[i] = (mrow && t < L) ? load_f32<MT>(mrow + t) : 0.f;
+    }
+  };
+  if (AHEAD && has_rows && tile_lo < tile_hi) fetch(tile_lo, kf, vf, mv);
+  for (int tile = tile_lo; has_rows && tile < tile_hi; ++tile) {
+    const int t0 = tile * 16;
+    float kn[AHEAD ? KS : 1], vn[AHEAD ? MTL : 1][4], mn[4];
+    const bool more = AHEAD && tile + 1 < tile_hi;
+    if constexpr (AHEAD) {
+      if (more) fetch(tile + 1, kn, vn, mn);
+    } else {
+      fetch(tile, kf, vf, mv);
     }
     f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -155,6 +167,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
       o[j] *= alpha;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j][i], pr[i], o[j], 0, 0, 0);
+    }
+    if constexpr (AHEAD) {
+      if (more) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kf[s] = kn[s];
+#pragma unroll
+        for (int j = 0; j < MTL; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vf[j][i] = vn[j][i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mv[i] = mn[i];
+      }
     }
   }
   // row sum over the four lanes of a row
@@ -246,11 +270,16 @@ extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void
   const bool mf32 = mask_dtype == PACE_DTYPE_F32;
   // vector accesses need rows that start on a 16-byte (fp32) / 8-byte (bf16) boundary
   const size_t row_align = f32 ? 16 : 8;
+  const bool ahead = p.l_split > 1;  // few query rows: bound by memory
   const bool vec = H % 4 == 0 && ((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % row_align == 0;
 #define PACE_DENSE_GO(T_, MT_, HP_) \
   do { \
-    if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true>), grid, dim3(256), 0, s, p); \
-    else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false>), grid, dim3(256), 0, s, p); \
+    constexpr bool kAheadBuilt = HP_ <= 128; /* at 256 the second set of registers does not fit */ \
+    if (ahead && kAheadBuilt) { \
+      if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt>), grid, dim3(256), 0, s, p); \
+      else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, kAheadBuilt>), grid, dim3(256), 0, s, p); \
+    } else if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, false>), grid, dim3(256), 0, s, p); \
+    else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, false>), grid, dim3(256), 0, s, p); \
   } while (0)
 #define PACE_DENSE_HP(T_, MT_) \
   do { \
