@@ -329,17 +329,6 @@ template <int D, int NQT, bool HAS_MASK, bool FULL>
 __device__ __forceinline__ void compute_unit_impl(const UnitRegs<D>& r, const u32x4 (&qreg)[NQT][D / 32],
                                                   RowState<D, NQT>& st, const PagedAttnParams& p, int t0, int tok_end,
                                                   int start, int g, const MaskRegs<NQT>& mregs = MaskRegs<NQT>{}) {
-#ifdef PACE_PROBE_LOADS_ONLY
-  {  // measurement aid: keep the loads, drop the arithmetic
-    u32x4 x = {0u, 0u, 0u, 0u};
-    for (int t = 0; t < 2; ++t)
-      for (int kk = 0; kk < D / 32; ++kk) x ^= r.k[t][kk];
-    for (int j = 0; j < D / 16; ++j) x ^= r.v[j];
-    st.o[0][0][0] += __uint_as_float(x[0] ^ x[1] ^ x[2] ^ x[3]);
-    st.l[0] = 1.f;
-    return;
-  }
-#endif
   f32x4 sc[NQT][2];
   score_products<D, NQT>(r.k, qreg, sc);
   softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, r.v, st, p, t0, tok_end, start, g, mregs);

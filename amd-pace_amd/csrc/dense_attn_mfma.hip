@@ -310,10 +310,14 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 
   typedef short tr_v4 __attribute__((ext_vector_type(4)));
   typedef tr_v4 __attribute__((address_space(3))) * tr_ptr;
-  int opaque_zero;
-  asm volatile("s_mov_b32 %0, 0" : "=s"(opaque_zero));
-  // One unit out of its stage: K rows in operand order for the scores; V comes back token-minor
-  // only once the score products are issued, into the registers the K rows leave.
+  // One unit out of its stage: K rows in operand order for the scores, then V token-minor through the LDS
+  // transpose read while the score products run.  K and V operands sit in registers of their own: the K
+  // operands are kept alive (an empty asm statement that takes them as inputs, fenced by scheduling barriers)
+  // until every V read has been issued, so no V read can be given a register the score products read from.
+  // An LDS read that returns into a register which a matrix instruction issued earlier has yet to fetch (one
+  // queued behind the accumulator of the instruction before it fetches its A / B operands late) is a
+  // write-after-read hazard that neither the hardware nor the compiler's wait-state insertion covers; with
+  // the two operand sets disjoint inside a unit, and a workgroup barrier between units, it cannot occur.
   auto unit = [&](int cur, int t0, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     if (MASK == 2) {
@@ -331,18 +335,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       for (int kk = 0; kk < KK; ++kk) kop[t][kk] = *reinterpret_cast<const u32x4*>(ks + t * 4 * KROW + kk * 32);
     f32x4 sc[NQT][2];
     score_products<D, NQT>(kop, qreg, sc);
-    // The V reads below land in registers the score products have just been issued from.  Nothing holds an LDS
-    // read back until a matrix instruction in flight has fetched its operands (one that waits in the pipeline for
-    // the accumulator of the instruction before it fetches them late), and now and then a V value arrived first:
-    // one tile's scores came out slightly wrong, differently from run to run.  So the address of the V reads is
-    // made to depend on every score tile's result (an "and" with a zero the compiler cannot see through):
-    // reading the results waits for the instructions to complete, in whatever order the compiler issued them.
-    int all_scores = 0;
-#pragma unroll
-    for (int qt = 0; qt < NQT; ++qt) all_scores |= __float_as_int(sc[qt][0][3]) | __float_as_int(sc[qt][1][3]);
-    const int done = __builtin_amdgcn_readfirstlane(all_scores) & opaque_zero;
+    __builtin_amdgcn_sched_barrier(0);  // the products above are issued before any read below
     // V: dim 16j + n of tokens 8g .. 8g+7 (see the transposed read in the kernel above)
-    const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3) + done];
+    const uint16_t* tr_base = &stage[cur][KSTAGE + (8 * g + (n >> 2)) * VROW + 4 * (n & 3)];
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       const tr_v4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(tr_base + 16 * j));
@@ -350,6 +345,12 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
       vop[j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) asm volatile("" ::"v"(kop[t][kk]));  // K operands live up to here
+    __builtin_amdgcn_sched_barrier(0);
     softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, vop, st, p, t0, L, 0, g, mcur);
   };
   // Units past the last one that matters to any row of the workgroup are not walked at all: with a

@@ -135,11 +135,6 @@ __device__ __forceinline__ void write_new_tokens(const PagedAttnParams& p, int b
   }
 }
 
-#ifdef PACE_PROBE_TIMING
-// Measurement aid: per-wave timestamps (100 MHz clock) of the phases of one launch.
-__device__ long long g_probe[1 << 20];
-__device__ unsigned int g_probe_n;
-#endif
 
 // Pool block ids of one wave's token range: up to 128 blocks (2048 tokens), one id per
 // lane in each of two registers, fetched with one coalesced load each and read back
@@ -171,9 +166,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
   static_assert(MERGE_SLOTS * 16 * NQT <= 128, "LDS merge buffer holds at most 128 query rows");
   __shared__ float merge_buf[MERGE_SLOTS * 16 * NQT * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
-#ifdef PACE_PROBE_TIMING
-  const long long pt0 = wall_clock64();
-#endif
   // Linear work index -> (KV head, row group, sequence, partition); KV head fastest.
   // (32-bit arithmetic: the host keeps total_items below 2^31.)
   const uint32_t L = blockIdx.x;
@@ -323,9 +315,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
       for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
     }
   }
-#ifdef PACE_PROBE_TIMING
-  const long long pt1 = wall_clock64();
-#endif
   MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
     const int t0 = tok_begin + 32 * uu;  // a multiple of 32: partitions and wave shares are whole units
@@ -348,9 +337,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
     }
   }
 
-#ifdef PACE_PROBE_TIMING
-  const long long pt2 = wall_clock64();
-#endif
   finish_rows<D, NQT, HAS_MASK>(st, p);  // row sums over the lanes of a row, running max in log2 units
 
   // Pairwise merge of the waves' states through LDS (fixed order: deterministic).
@@ -400,16 +386,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
       }
       __syncthreads();
     }
-#ifdef PACE_PROBE_TIMING
-    if (wave != 0 && lane == 0) {
-      const long long pt3 = wall_clock64();
-      const unsigned int slot = atomicAdd(&g_probe_n, 1u);
-      if (slot < (1u << 20) / 8) {
-        long long* o = g_probe + 8ull * slot;
-        o[0] = pt0, o[1] = pt1, o[2] = pt2, o[3] = pt3, o[4] = n_units, o[5] = (long long)kvh, o[6] = wave + 16 * (long long)__smid(), o[7] = b;
-      }
-    }
-#endif
     if (wave != 0) return;
   }
 
@@ -440,16 +416,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
       }
     }
   }
-#ifdef PACE_PROBE_TIMING
-  if (lane == 0) {
-    const long long pt3 = wall_clock64();
-    const unsigned int slot = atomicAdd(&g_probe_n, 1u);
-    if (slot < (1u << 20) / 8) {
-      long long* o = g_probe + 8ull * slot;
-      o[0] = pt0, o[1] = pt1, o[2] = pt2, o[3] = pt3, o[4] = n_units, o[5] = (long long)kvh, o[6] = wave + 16 * (long long)__smid(), o[7] = b;
-    }
-  }
-#endif
 }
 
 // One wave per (sequence, query token): the last column of the row's mask line, among those the
@@ -581,10 +547,10 @@ static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t bat
   const Shape sh = shape_for(head_dim, tiles);
   const int granule = 128;
   if (requested > 0) return requested;
-  // Enough workgroups to fill every compute unit (256) with as many as fit (4 * occ waves each); a batch
+  // Enough workgroups to fill every compute unit with as many as fit (4 * occ waves each); a batch
   // that already does so is not split at all.
   const int64_t groups = (int64_t)batch * num_kv_heads * ((tiles + sh.nqt - 1) / sh.nqt);
-  const int64_t slots = 256 * 4 * sh.occ / sh.nw;
+  const int64_t slots = (int64_t)compute_units() * 4 * sh.occ / sh.nw;
   int64_t parts = (slots + groups - 1) / groups;
   if (parts < 1) parts = 1;
   int64_t per = ((int64_t)max_seq_len + parts - 1) / parts;
@@ -786,17 +752,6 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
 
 using namespace pace_kv;
 
-#ifdef PACE_PROBE_TIMING
-extern "C" int pace_probe_read(long long* host, unsigned int* n, int reset) {
-  hipMemcpyFromSymbol(n, HIP_SYMBOL(g_probe_n), sizeof(unsigned int));
-  hipMemcpyFromSymbol(host, HIP_SYMBOL(g_probe), sizeof(long long) * (1 << 20));
-  if (reset) {
-    unsigned int z = 0;
-    hipMemcpyToSymbol(HIP_SYMBOL(g_probe_n), &z, sizeof(z));
-  }
-  return 0;
-}
-#endif
 
 extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len, int32_t head_dim,
                                                     int32_t max_seq_len, int32_t partition_tokens, int32_t num_kv_heads) {

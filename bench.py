@@ -7,7 +7,8 @@ context 4096, bf16, 32 Q / 8 KV heads, head_dim 128, KV block 16, physical block
 permuted.  A step is one pass of the hot path over one batch: append one new token per
 sequence into the block-paged cache, then GQA decode attention over the whole cache.
 Every step runs at the same cache state (the token lands at position 4096 each time), so
-the bytes per step are constant.  All inputs are resident in HBM before the timed region.
+the bytes per step are constant; the steps rotate over --layers distinct pools (default 4) so that
+every step reads its K / V from HBM, not from what the step before left in the last-level cache.  All inputs are resident in HBM before the timed region.
 One JSON line is printed.
 
 Other workloads (same JSON shape, `config.workload` names them):
@@ -276,13 +277,20 @@ def wl_decode_gptj(torch, dev, args):
 
 def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
     B, ctx, hq, hkv, D = shape
-    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute,
-                        headroom=64 + args.steps + args.warmup)
-    cache.partition_tokens = args.partition
+    # One pool per layer, each with its own seeded block permutation: step i runs on pool i mod N, as a
+    # decoder walks its layers (pace/llm/models/llama.py:312-315), so no step finds the K / V of the step
+    # before it in the 256 MB last-level cache.
+    n_layers = max(1, args.layers)
+    caches = [build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1 + 100 * i, permute=not args.no_permute,
+                          headroom=64 + args.steps + args.warmup) for i in range(n_layers)]
+    cache = caches[0]
+    for c in caches:
+        c.partition_tokens = args.partition
     g = torch.Generator(device=dev).manual_seed(2)
     k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
     q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
     keep = []
+    turn = [0]
     if args.path == "api":
         from pace_mi355.ops import MultiHeadAttention
 
@@ -295,10 +303,12 @@ def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
         keep.extend([ka, va, mask_all])
 
         def step(ev=None):
-            pk, pv = cache.update_cache(ka, va, 2)  # the context grows by one token per step on this path
+            c = caches[turn[0] % n_layers]
+            turn[0] += 1
+            pk, pv = c.update_cache(ka, va, 2)  # the context of a layer grows by one token per step on this path
             if ev:
                 ev[0].record()
-            mha(q, pk, pv, attention_mask=mask_all[..., : cache.seq_len] if args.mask else None)
+            mha(q, pk, pv, attention_mask=mask_all[..., : c.seq_len] if args.mask else None)
             if ev:
                 ev[1].record()
     else:
@@ -313,10 +323,15 @@ def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
             keep.extend([cos, sin])
             rope = nat.RopeDesc(cos=cos.data_ptr(), sin=sin.data_ptr(), table_dtype=nat.DTYPE_BF16, table_rows=cos.shape[0],
                                 rotary_dim=D, interleaved=0, positions=None, pos_stride_b=0)
-        step = FixedStep(torch, cache, q, k1, v1, args.partition, fused=not args.no_fuse, rope=rope)
+        fixed = [FixedStep(torch, c, q, k1, v1, args.partition, fused=not args.no_fuse, rope=rope) for c in caches]
+
+        def step(ev=None):
+            f = fixed[turn[0] % n_layers]
+            turn[0] += 1
+            f(ev)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
-    if args.path == "api":  # average context over the timed steps
-        ctx = ctx + args.warmup + (args.steps - 1) // 2
+    if args.path == "api":  # average context over the timed steps (each layer's cache grows once every n_layers steps)
+        ctx = ctx + (args.warmup + (args.steps - 1) // 2) // n_layers
     dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
     fused = args.path == "direct" and not args.no_fuse or args.path == "api"
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
@@ -325,7 +340,8 @@ def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
         roofline(f"paged_attn_kernel<{D},1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
                  {"traffic": traffic}),
         {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct"),
-         "mask": bool(args.mask and args.path == "api")})
+         "mask": bool(args.mask and args.path == "api"), "layers": n_layers,
+         "distinct_pool_bytes": int(n_layers * B * ctx * kv_token_bytes(hkv, D))})
     if with_cpu and not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
@@ -604,6 +620,9 @@ def main() -> int:
     ap.add_argument("--path", choices=("api", "direct"), default="direct",
                     help="decode-8b only. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
                          "MultiHeadAttention")
+    ap.add_argument("--layers", type=int, default=4,
+                    help="decode workloads: distinct layer pools (own block permutation each) the timed steps rotate over; "
+                         "4 x 1.07 GB is 16 times the last-level cache, 1 re-reads one pool every step")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--mask", action="store_true",
