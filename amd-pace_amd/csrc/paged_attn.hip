@@ -7,6 +7,8 @@
 // head.  A second small kernel merges the partitions of a sequence.
 //
 // The inner step (one 32-token unit on the matrix cores) is in attn_core.h.
+#include <mutex>
+
 #include "attn_core.h"
 
 namespace pace_kv {
@@ -612,9 +614,44 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   return false;
 }
 
-static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, void* stream, const char* who) {
+// Scratch of the entry point that allocates nothing: one array per GPU, in the library's own device image.
+// In host code the array's name is only a stand-in; the address each device holds it at comes from
+// hipGetSymbolAddress, once per device, and that address is what kernels and checks are given.
+constexpr size_t kStaticScratchBytes = (size_t)PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (resolved on the first call there).
+static int static_scratch(const char* who, void** out) {
+  int dev = 0;
+  PACE_HIP_CHECK(hipGetDevice(&dev));
+  PACE_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device ordinal %d out of range", who, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    PACE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    PACE_REQUIRE(ptr != nullptr, "%s: the scratch array has no device address", who);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PACE_KV_OK;
+}
+
+static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a_in, void* stream, const char* who,
+                          bool use_static_scratch = false) {
+  PACE_REQUIRE(a_in != nullptr, "%s: args is NULL", who);
+  pace_paged_attn_args_t a_copy = *a_in;
+  if (use_static_scratch) {
+    void* ptr = nullptr;
+    if (int rc = static_scratch(who, &ptr)) return rc;
+    a_copy.workspace = ptr;
+    a_copy.workspace_bytes = kStaticScratchBytes;
+  }
+  const pace_paged_attn_args_t* a = &a_copy;
   if (int rc = check_pool(pool, who)) return rc;
-  PACE_REQUIRE(a != nullptr, "%s: args is NULL", who);
   PACE_REQUIRE(a->batch >= 0 && a->q_len >= 1 && a->num_q_heads >= 1, "%s: bad batch (%d), q_len (%d) or num_q_heads (%d)",
                who, a->batch, a->q_len, a->num_q_heads);
   if (a->batch == 0) return PACE_KV_OK;
@@ -698,6 +735,11 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
     const size_t need = rows_total * max_parts * (pool->head_dim + 2) * sizeof(float);
+    if (use_static_scratch)
+      PACE_REQUIRE(need <= kStaticScratchBytes,
+                   "%s: this launch needs %zu bytes of scratch, the static buffer holds %zu; use pace_paged_attn_verify with a "
+                   "workspace of that size",
+                   who, need, kStaticScratchBytes);
     PACE_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need,
                  "%s: workspace too small (%zu bytes given, %zu needed)", who, a->workspace_bytes, need);
     PACE_REQUIRE(aligned16(a->workspace), "%s: workspace must be 16-byte aligned", who);
@@ -795,4 +837,8 @@ extern "C" int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_pag
 
 extern "C" int pace_paged_attn_verify(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {
   return run_paged_attn(pool, args, stream, "pace_paged_attn_verify");
+}
+
+extern "C" int pace_paged_attn_verify_static(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {
+  return run_paged_attn(pool, args, stream, "pace_paged_attn_verify_static", true);
 }

@@ -15,6 +15,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
 ABI_VERSION = 8
+STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
 EXPORTED_SYMBOLS = (
@@ -31,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "pace_paged_attn_workspace_bytes_for_parts",
     "pace_paged_attn_decode",
     "pace_paged_attn_verify",
+    "pace_paged_attn_verify_static",
     "pace_attn_dense",
 )
 
@@ -173,6 +175,8 @@ def load() -> ctypes.CDLL:
     lib.pace_paged_attn_decode.argtypes = [P, A, c_void_p]
     lib.pace_paged_attn_verify.restype = ctypes.c_int
     lib.pace_paged_attn_verify.argtypes = [P, A, c_void_p]
+    lib.pace_paged_attn_verify_static.restype = ctypes.c_int
+    lib.pace_paged_attn_verify_static.argtypes = [P, A, c_void_p]
     lib.pace_attn_dense.restype = ctypes.c_int
     lib.pace_attn_dense.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,

@@ -266,6 +266,21 @@ int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_paged_attn_arg
 int pace_paged_attn_verify(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream);
 
 /*
+ * pace_paged_attn_verify (any q_len >= 1, so decode too) for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference.  args->workspace / workspace_bytes are ignored; the partial results of sequences cut
+ * into several partitions (and the per-row mask summary of prefill-sized masked launches) live in an array of
+ * PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES that is part of the library's device image -- every GPU the library
+ * runs on holds one copy until the process ends.  A launch that needs more (see
+ * pace_paged_attn_workspace_bytes*) is refused with PACE_KV_EINVAL and nothing is launched.  The call
+ * allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that may overlap there
+ * (different streams, different threads) race; order them on one stream.  Nothing in the array needs
+ * clearing between calls: every partial a launch reads, it has written.
+ */
+#define PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES (32u << 20)
+int pace_paged_attn_verify_static(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream);
+
+/*
  * Dense attention: body of the torch op
  *   pace::attention(Tensor input_Q, Tensor input_K, Tensor input_V,
  *                   Tensor? input_mask, Scalar? use_KQ) -> Tensor
