@@ -145,61 +145,118 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
 
 // ---------------------------------------------------------------------------------
 // Gather.  One 256-thread workgroup rebuilds one logical block (16 tokens) of one KV
-// head of one sequence in the dense [B][H*n_rep][L][D] layout.  K chunks are read
-// from their slab position; V slabs are staged in LDS and read back transposed.
+// head of one sequence as token rows.  K chunks are read from their slab position; V
+// slabs are staged in LDS and read back transposed.  Two output forms:
+//   dense   [B][H*n_rep][out_len][D]   (the reference's layout; rows >= len zero-filled on request)
+//   packed  [sum len][H*n_rep][D]      (sequence b starts at row cu_seqlens[b]; no padding at all)
+// A workgroup past the end of its sequence leaves at once; the packed form launches none (its grid is
+// built from cu_seqlens).
 // ---------------------------------------------------------------------------------
-template <int D>
+struct GatherOut {
+  uint16_t* k;
+  uint16_t* v;
+  const int32_t* cu_seqlens;  // packed form only
+  int64_t stride_b;           // dense: elements between sequences
+  int64_t stride_h;           // elements between output heads
+  int64_t stride_t;           // elements between token rows
+  int32_t out_len;            // dense: rows per sequence; packed: unused
+  int32_t zero_fill;          // dense: write zeros to rows in [len, out_len)
+  int32_t batch;              // packed: sequences (cu_seqlens has batch + 1 entries)
+  int32_t total_rows;         // packed: rows of the outputs
+};
+
+template <int D, bool PACKED>
 __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
                                                         int32_t table_stride, const int32_t* __restrict__ seq_lens,
-                                                        int32_t len_bias, int32_t n_rep, uint16_t* __restrict__ k_out,
-                                                        uint16_t* __restrict__ v_out, int64_t osb, int64_t osh,
-                                                        int32_t out_len) {
+                                                        int32_t len_bias, int32_t n_rep, const GatherOut out) {
   constexpr int CHUNKS = D / 8;                             // 16-byte chunks per row
   constexpr int SLAB_CHUNKS = PACE_KV_BLOCK_TOKENS * CHUNKS;  // per (block, head)
   __shared__ uint16_t vt[D * PACE_KV_BLOCK_TOKENS + 8];
-  const int j = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  int j = blockIdx.x, b = blockIdx.z, h = blockIdx.y;
+  if (PACKED) {
+    // One grid entry per (logical block that can exist, KV head): sequence b owns the block entries
+    // [cu[b] / 16 + b, cu[b+1] / 16 + b + 1) -- at least ceil(len_b / 16) of them, disjoint, in order -- so a
+    // ragged batch launches (almost) no workgroup without rows.  Entries run sequence by sequence, head by
+    // head, block by block (the order of the dense grid: with the heads of a block side by side instead the
+    // launch measured 6 % slower).  The owner is found by bisection, uniform over the workgroup: scalar loads
+    // from a table that stays in the scalar cache.
+    const int H = pool.num_kv_heads;
+    int lo = 0, hi = out.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if ((int64_t)(out.cu_seqlens[mid] / PACE_KV_BLOCK_TOKENS + mid) * H <= (int64_t)blockIdx.x) lo = mid; else hi = mid;
+    }
+    b = lo;
+    const int first = out.cu_seqlens[b] / PACE_KV_BLOCK_TOKENS + b;
+    const int n = out.cu_seqlens[b + 1] / PACE_KV_BLOCK_TOKENS + b + 1 - first;  // >= 1
+    const int r = (int)((int64_t)blockIdx.x - (int64_t)first * H);
+    h = min(r / n, H - 1), j = r % n;
+  }
+  // The length and the block id are fetched side by side (the table row exists whatever the length is; an
+  // entry past the live blocks is clamped into the pool and never used): one round trip, not two, before
+  // the slab loads can start.
   const int len = seq_lens[b] + len_bias;
+  int64_t blk = table[(int64_t)b * table_stride + min(j, table_stride - 1)];
   const int t0 = j * PACE_KV_BLOCK_TOKENS;
   const bool live = t0 < len;  // uniform per workgroup
-  int64_t blk = 0;
-  if (live) blk = table[(int64_t)b * table_stride + j];
+  const int row_end = PACKED ? len : out.out_len;
+  if (!live && (PACKED || !out.zero_fill || t0 >= row_end)) return;  // nothing to write
   blk = blk < 0 ? 0 : (blk >= pool.num_blocks ? pool.num_blocks - 1 : blk);  // never read outside the pool
   const uint16_t* ksrc = reinterpret_cast<const uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
   const uint16_t* vsrc = reinterpret_cast<const uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
-  if (live) {
-    for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x)
-      *reinterpret_cast<u32x4*>(&vt[c * 8]) = load16_stream(vsrc + c * 8);
+  // Every load of the workgroup goes out before the barrier: the V slab (to LDS, to be read back transposed)
+  // and the K chunks of this lane's rows (kept in registers).
+  constexpr int PER = (SLAB_CHUNKS + 255) / 256;
+  u32x4 kreg[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * 256;
+    kreg[i] = u32x4{0u, 0u, 0u, 0u};
+    if (live && c < SLAB_CHUNKS) {
+      const u32x4 vraw = load16_stream(vsrc + c * 8);
+      const int tok = c / CHUNKS, chunk = c % CHUNKS;
+      if (t0 + tok < len) kreg[i] = load16_stream(ksrc + k_slab_offset<D>(tok, chunk * 8));
+      *reinterpret_cast<u32x4*>(&vt[c * 8]) = vraw;
+    }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < SLAB_CHUNKS; c += blockDim.x) {
+  const int64_t base = PACKED ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c >= SLAB_CHUNKS) continue;
     const int tok = c / CHUNKS, chunk = c % CHUNKS;
     const int t = t0 + tok;
-    if (t >= out_len) continue;
-    u32x4 kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
+    if (t >= row_end) continue;
+    if (PACKED && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
+    u32x4 vv = {0u, 0u, 0u, 0u};
     if (t < len) {
-      kv = load16_stream(ksrc + k_slab_offset<D>(tok, chunk * 8));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const uint32_t lo = vt[v_slab_offset<D>(tok, chunk * 8 + 2 * e)];
         const uint32_t hi = vt[v_slab_offset<D>(tok, chunk * 8 + 2 * e + 1)];
         vv[e] = lo | (hi << 16);
       }
+    } else if (!out.zero_fill) {
+      continue;
     }
     for (int r = 0; r < n_rep; ++r) {
-      const int64_t o = (int64_t)b * osb + (int64_t)(h * n_rep + r) * osh + (int64_t)t * D + chunk * 8;
-      store16_stream(k_out + o, kv);
-      store16_stream(v_out + o, vv);
+      const int64_t o = base + (int64_t)(h * n_rep + r) * out.stride_h + (int64_t)t * out.stride_t + chunk * 8;
+      store16_stream(out.k + o, kreg[i]);
+      store16_stream(out.v + o, vv);
     }
   }
 }
 
 // ---------------------------------------------------------------------------------
-// Block copy.  One workgroup per (pair, head): both slabs of that head, 16 bytes per
-// lane access.  Layout-agnostic (a slab is copied verbatim).
+// Block copy.  Layout-agnostic (a slab is copied verbatim), 16 bytes per lane access.
+// kv_copy_blocks_kernel: one workgroup per (pair, head), both slabs of that head.
+// kv_copy_whole_blocks_kernel: pools whose blocks are one contiguous run each (all heads, K and V):
+// one workgroup per pair moves the whole run, every lane with several loads in flight.
 // ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void kv_copy_blocks_kernel(pace_kv_pool_t src, pace_kv_pool_t dst,
                                                              const int32_t* __restrict__ pairs) {
-  const int pair = blockIdx.x, h = blockIdx.y;
+  const int pair = blockIdx.y, h = blockIdx.x;  // heads fastest: the slabs of one block move together
   const int64_t s = pairs[2 * pair], d = pairs[2 * pair + 1];
   if (s < 0 || s >= src.num_blocks || d < 0 || d >= dst.num_blocks) return;  // uniform per workgroup
   const int slab_chunks = PACE_KV_BLOCK_TOKENS * src.head_dim / 8;
@@ -215,6 +272,20 @@ __global__ __launch_bounds__(256) void kv_copy_blocks_kernel(pace_kv_pool_t src,
     store16_stream(kd + c, a);
     store16_stream(vd + c, bq);
   }
+}
+
+__global__ __launch_bounds__(256) void kv_copy_whole_blocks_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                                   int64_t src_block_chunks, int64_t dst_block_chunks,
+                                                                   int32_t run_chunks, int32_t src_blocks, int32_t dst_blocks,
+                                                                   const int32_t* __restrict__ pairs) {
+  // blockIdx.x: 4 KiB piece of the run (fastest, so that the pieces of one block are in flight together and
+  // both streams stay inside a few DRAM pages); blockIdx.y: pair.  One 16-byte access per lane: workgroups this
+  // small measured 14 % faster than one workgroup per 64 KiB block with eight loads in flight per lane.
+  const int pair = blockIdx.y;
+  const int64_t s = pairs[2 * pair], d = pairs[2 * pair + 1];
+  if (s < 0 || s >= src_blocks || d < 0 || d >= dst_blocks) return;  // uniform per workgroup
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c < run_chunks) store16_stream(dst + d * dst_block_chunks + c, load16_stream(src + s * src_block_chunks + c));
 }
 
 }  // namespace pace_kv
@@ -304,29 +375,61 @@ extern "C" int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_ne
                     stream);
 }
 
-extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
-                              const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep, void* k_out, void* v_out,
-                              int64_t out_stride_b, int64_t out_stride_h, int32_t out_len, void* stream) {
-  if (int rc = check_pool(pool, "pace_kv_gather")) return rc;
-  PACE_REQUIRE(batch >= 0 && out_len >= 0 && n_rep >= 1, "pace_kv_gather: bad batch (%d), out_len (%d) or n_rep (%d)",
-               batch, out_len, n_rep);
-  if (batch == 0 || out_len == 0) return PACE_KV_OK;
-  PACE_REQUIRE(block_table && seq_lens && k_out && v_out, "pace_kv_gather: NULL pointer");
-  PACE_REQUIRE(aligned16(k_out) && aligned16(v_out), "pace_kv_gather: outputs must be 16-byte aligned");
-  PACE_REQUIRE(out_stride_b % 8 == 0 && out_stride_h % 8 == 0, "pace_kv_gather: output strides must be multiples of 8");
-  const int n_blocks = (out_len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
-  PACE_REQUIRE(table_stride >= 1, "pace_kv_gather: table_stride %d", table_stride);
-  PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "pace_kv_gather: batch/heads exceed grid limits");
+static int run_gather(const char* who, const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                      const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep, int32_t rows,
+                      const GatherOut& out_in, bool packed, void* stream) {
+  const GatherOut& out = out_in;
+  if (int rc = check_pool(pool, who)) return rc;
+  PACE_REQUIRE(batch >= 0 && rows >= 0 && n_rep >= 1, "%s: bad batch (%d), row count (%d) or n_rep (%d)", who, batch, rows, n_rep);
+  if (batch == 0 || rows == 0) return PACE_KV_OK;
+  PACE_REQUIRE(block_table && seq_lens && out.k && out.v, "%s: NULL pointer", who);
+  PACE_REQUIRE(aligned16(out.k) && aligned16(out.v), "%s: outputs must be 16-byte aligned", who);
+  PACE_REQUIRE(out.stride_b % 8 == 0 && out.stride_h % 8 == 0 && out.stride_t % 8 == 0 && out.stride_t >= pool->head_dim &&
+                   out.stride_h >= pool->head_dim,
+               "%s: output strides must be multiples of 8 elements and hold a row of head_dim", who);
+  const int n_blocks = (rows + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
+  PACE_REQUIRE(table_stride >= 1, "%s: table_stride %d", who, table_stride);
+  PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch/heads exceed grid limits", who);
   dim3 grid(n_blocks, pool->num_kv_heads, batch);
+  if (packed) {
+    const int64_t entries = ((int64_t)out.total_rows / PACE_KV_BLOCK_TOKENS + batch) * pool->num_kv_heads;
+    PACE_REQUIRE(entries < ((int64_t)1 << 31), "%s: grid too large", who);
+    grid = dim3((unsigned)entries, 1, 1);
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  uint16_t* ko = static_cast<uint16_t*>(k_out);
-  uint16_t* vo = static_cast<uint16_t*>(v_out);
   for_head_dim(pool->head_dim, [&](auto d) {
-    hipLaunchKernelGGL(kv_gather_kernel<decltype(d)::value>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens,
-                       seq_len_bias, n_rep, ko, vo, out_stride_b, out_stride_h, out_len);
+    constexpr int DIM = decltype(d)::value;
+    if (packed)
+      hipLaunchKernelGGL((kv_gather_kernel<DIM, true>), grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens,
+                         seq_len_bias, n_rep, out);
+    else
+      hipLaunchKernelGGL((kv_gather_kernel<DIM, false>), grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens,
+                         seq_len_bias, n_rep, out);
   });
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
+}
+
+extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                              const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep, void* k_out, void* v_out,
+                              int64_t out_stride_b, int64_t out_stride_h, int32_t out_len, int32_t zero_fill, void* stream) {
+  PACE_REQUIRE(pool != nullptr, "pace_kv_gather: pool is NULL");
+  GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), nullptr, out_stride_b, out_stride_h,
+                   pool->head_dim, out_len, zero_fill ? 1 : 0, batch, 0};
+  return run_gather("pace_kv_gather", pool, block_table, table_stride, seq_lens, seq_len_bias, batch, n_rep, out_len, out, false,
+                    stream);
+}
+
+extern "C" int pace_kv_gather_packed(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                                     const int32_t* seq_lens, int32_t seq_len_bias, const int32_t* cu_seqlens, int32_t batch,
+                                     int32_t n_rep, void* k_out, void* v_out, int32_t total_tokens, void* stream) {
+  PACE_REQUIRE(pool != nullptr, "pace_kv_gather_packed: pool is NULL");
+  if (batch > 0 && total_tokens > 0) PACE_REQUIRE(cu_seqlens != nullptr, "pace_kv_gather_packed: cu_seqlens is NULL");
+  PACE_REQUIRE(n_rep >= 1, "pace_kv_gather_packed: bad n_rep (%d)", n_rep);
+  const int64_t row = (int64_t)pool->num_kv_heads * n_rep * pool->head_dim;  // one token, every output head
+  GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), cu_seqlens, 0, pool->head_dim, row, 0, 0, batch, total_tokens};
+  return run_gather("pace_kv_gather_packed", pool, block_table, table_stride, seq_lens, seq_len_bias, batch, n_rep, total_tokens,
+                    out, true, stream);
 }
 
 extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst, const int32_t* pairs,
@@ -338,9 +441,31 @@ extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool
   PACE_REQUIRE(n_pairs >= 0, "pace_kv_copy_blocks: negative n_pairs");
   if (n_pairs == 0) return PACE_KV_OK;
   PACE_REQUIRE(pairs != nullptr, "pace_kv_copy_blocks: pairs is NULL");
-  PACE_REQUIRE(src->num_kv_heads <= 65535, "pace_kv_copy_blocks: too many heads");
-  hipLaunchKernelGGL(kv_copy_blocks_kernel, dim3(n_pairs, src->num_kv_heads), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), *src, *dst, pairs);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // A pool laid out [block][head][K|V][16 * head_dim] holds a block as one contiguous run: move it whole.
+  const int64_t slab = (int64_t)PACE_KV_BLOCK_TOKENS * src->head_dim;
+  auto one_run = [&](const pace_kv_pool_t* p) {
+    return static_cast<const uint16_t*>(p->v) == static_cast<const uint16_t*>(p->k) + slab && p->k_head_stride == 2 * slab &&
+           p->v_head_stride == 2 * slab && p->k_block_stride == p->v_block_stride &&
+           p->k_block_stride >= (int64_t)p->num_kv_heads * 2 * slab;
+  };
+  if (one_run(src) && one_run(dst)) {
+    const int64_t run_chunks = (int64_t)src->num_kv_heads * 2 * slab / 8;
+    PACE_REQUIRE(n_pairs <= 65535 * 32, "pace_kv_copy_blocks: too many pairs (%d)", n_pairs);
+    // grid.y holds at most 65535 pairs per launch
+    for (int32_t p0 = 0; p0 < n_pairs; p0 += 65535) {
+      const int32_t n = n_pairs - p0 < 65535 ? n_pairs - p0 : 65535;
+      hipLaunchKernelGGL(kv_copy_whole_blocks_kernel, dim3((unsigned)((run_chunks + 255) / 256), n), dim3(256), 0, s,
+                         static_cast<const u32x4*>(src->k), static_cast<u32x4*>(dst->k), src->k_block_stride / 8,
+                         dst->k_block_stride / 8, (int32_t)run_chunks, src->num_blocks, dst->num_blocks, pairs + 2 * (int64_t)p0);
+    }
+  } else {
+    PACE_REQUIRE(n_pairs <= 65535 * 32, "pace_kv_copy_blocks: too many pairs (%d)", n_pairs);
+    for (int32_t p0 = 0; p0 < n_pairs; p0 += 65535) {
+      const int32_t n = n_pairs - p0 < 65535 ? n_pairs - p0 : 65535;
+      hipLaunchKernelGGL(kv_copy_blocks_kernel, dim3(src->num_kv_heads, n), dim3(256), 0, s, *src, *dst, pairs + 2 * (int64_t)p0);
+    }
+  }
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }

@@ -416,8 +416,11 @@ class PagedKVCache(KVCacheBase):
                 nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), dev.data_ptr(), len(pairs), nat.current_stream_ptr()))
         self.cow_blocks_copied += len(pairs)
 
-    def gather(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-        """Dense ``[B, Hkv*n_rep, L, D]`` copies of K and V (zeros past each length)."""
+    def gather(self, n_rep: Optional[int] = None, pad_to: Optional[int] = None,
+               zero_fill: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Dense ``[B, Hkv*n_rep, L, D]`` copies of K and V, zeros past each length (what the
+        reference's caches hold, ``pace/llm/cache.py:255-266``).  ``zero_fill=False`` leaves the rows
+        past each length unwritten: in a ragged batch they are most of the tensor."""
         self._flush()
         n_rep = self.n_rep if n_rep is None else int(n_rep)
         L = int(self.lens.max(initial=0)) if pad_to is None else int(pad_to)
@@ -431,12 +434,41 @@ class PagedKVCache(KVCacheBase):
             nat.check(
                 nat.load().pace_kv_gather(
                     ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, self.batch, n_rep,
-                    k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, nat.current_stream_ptr(),
+                    k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, 1 if zero_fill else 0, nat.current_stream_ptr(),
                 )
             )
         if padded:
             k, v = k[..., : self.model_dim].contiguous(), v[..., : self.model_dim].contiguous()
         return k, v
+
+    def gather_packed(self, n_rep: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """K and V without padding: ``[sum(lens), Hkv*n_rep, D]`` each, the rows of sequence ``b`` at
+        ``cu_seqlens[b] : cu_seqlens[b+1]`` (third result, device int32 ``[B+1]``).  Row ``t`` of
+        sequence ``b`` is ``dense[b, :, t, :]``."""
+        self._flush()
+        n_rep = self.n_rep if n_rep is None else int(n_rep)
+        cu = np.zeros(self.batch + 1, dtype=np.int64)
+        np.cumsum(self.lens, out=cu[1:])
+        total = int(cu[-1])
+        if total >= 1 << 31:
+            raise RuntimeError("packed gather addresses rows with 32-bit offsets")
+        dev = self.pool.device
+        cu_dev = torch.from_numpy(cu.astype(np.int32)).pin_memory().to(dev, non_blocking=True)
+        shape = (total, self.num_kv_heads * n_rep, self.head_dim)
+        k = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+        v = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+        if total:
+            st = self.state
+            table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
+            nat.check(
+                nat.load().pace_kv_gather_packed(
+                    ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, cu_dev.data_ptr(),
+                    self.batch, n_rep, k.data_ptr(), v.data_ptr(), total, nat.current_stream_ptr(),
+                )
+            )
+        if self.head_dim != self.model_dim:
+            k, v = k[..., : self.model_dim].contiguous(), v[..., : self.model_dim].contiguous()
+        return k, v, cu_dev
 
     def _plan(self, B: int, hq: int, S: int, D: int, max_len: int):
         """How one attention launch is cut: (work items, partitions per sequence, partition size,

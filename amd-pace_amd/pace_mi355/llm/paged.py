@@ -342,16 +342,19 @@ class PagedState:
         out[b] -= removed_tokens
         return out
 
+    def _live_mask(self) -> np.ndarray:
+        """``[B, cols]`` bool: the table entries in use."""
+        return np.arange(self.table.shape[1])[None, :] < self.n_blocks[:, None]
+
     def plan_compaction(self) -> np.ndarray:
         """Moves that pack all live blocks into ids ``0 .. n_live-1`` with the
         fewest copies: every live block at or above ``n_live`` moves into a free
         id below it.  Returns ``[n_moves, 2]`` int32 ``(src, dst)``; the two id
         sets are disjoint."""
-        live = np.unique(np.concatenate([self.table[b, : int(self.n_blocks[b])] for b in range(self.batch)] or [np.zeros(0, np.int32)]))
-        n_live = live.size
-        src = np.sort(live[live >= n_live])
         is_live = np.zeros(self.allocator.num_blocks, dtype=bool)
-        is_live[live] = True
+        is_live[self.table[self._live_mask()]] = True
+        n_live = int(is_live.sum())
+        src = np.nonzero(is_live[n_live:])[0] + n_live
         dst = np.nonzero(~is_live[:n_live])[0]
         assert src.size == dst.size
         return np.stack([src, dst], axis=1).astype(np.int32) if src.size else np.zeros((0, 2), np.int32)
@@ -362,11 +365,9 @@ class PagedState:
             return
         remap = np.arange(self.allocator.num_blocks, dtype=np.int32)
         remap[moves[:, 0]] = moves[:, 1]
-        refs = np.zeros(self.allocator.num_blocks, dtype=np.int32)
-        for b in range(self.batch):
-            n = int(self.n_blocks[b])
-            self.table[b, :n] = remap[self.table[b, :n]]
-            np.add.at(refs, self.table[b, :n], 1)
+        mask = self._live_mask()
+        self.table[mask] = remap[self.table[mask]]
+        refs = np.bincount(self.table[mask], minlength=self.allocator.num_blocks).astype(np.int32)
         self.allocator.reset_free(refs == 0, refs)
         self._table_dirty = True
 

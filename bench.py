@@ -21,6 +21,8 @@ Other workloads (same JSON shape, `config.workload` names them):
   dense-f32     the dense op on fp32 tensors (the general kernel; roofline against the fp32 matrix-core peak)
   compact   Llama-3-70B-shape KV, batch 8, context 32768: evict 40% of the blocks, then time the
             compaction copy and the decode over the compacted cache
+  gather / append    the block-table gather (dense and packed output) and the stand-alone append (1 / 8 / 512
+            tokens per sequence) at the headline shape, each against the HBM roofline
   copy-calibration   block copy of a known byte count, used to scale the HBM byte counters
 """
 from __future__ import annotations
@@ -362,13 +364,88 @@ def wl_ragged(torch, dev, args):
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
     lens1 = [n + 1 for n in lens]
     dec = decode_bytes(lens1, hq, hkv, D)
-    gather_ms = time_call(torch, lambda: cache.gather(n_rep=1), reps=5, warmup=1)
     gather_b = 2 * sum(lens) * kv_token_bytes(hkv, D)
+    forms = {}
+    for form in ("packed", "dense", "dense_zero_fill"):
+        fn = gather_call(torch, cache, form)
+        forms[form] = roofline(f"kv_gather_kernel<128,{'true' if form == 'packed' else 'false'}> ({form.replace('_', ' ')})", gather_b,
+                               time_call(torch, fn, reps=5, warmup=1))
     return result_line(
         args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x, "
         "1-token append + GQA decode", dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline("paged_attn_kernel<128,1,...> (decode, ragged) + merge", dec, attn_ms),
-        extra={"gather": roofline("kv_gather_kernel<128> (includes output allocation)", gather_b, gather_ms)})
+        extra={"gather": forms})
+
+
+def gather_call(torch, cache, form):
+    """A closure that runs one gather of the whole cache into preallocated outputs (KV heads only, no
+    repeat_kv expansion).  form: "packed" ([sum len][H][D] + cu_seqlens), "dense" ([B][H][Lmax][D], rows past
+    each length left alone) or "dense_zero_fill" (the same with the padding written as zeros)."""
+    import numpy as np
+    from pace_mi355 import _native as nat
+
+    lib, dev = nat.load(), cache.pool.device
+    st = cache.state
+    table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
+    B, H, D, L = cache.batch, cache.num_kv_heads, cache.head_dim, int(cache.lens.max())
+    if form == "packed":
+        cu = np.zeros(B + 1, dtype=np.int64)
+        np.cumsum(cache.lens, out=cu[1:])
+        cu_dev = torch.from_numpy(cu.astype(np.int32)).to(dev)
+        k, v = (torch.empty(int(cu[-1]), H, D, dtype=torch.bfloat16, device=dev) for _ in range(2))
+
+        def fn(_keep=(cu_dev, k, v, table, lens_dev)):
+            nat.check(lib.pace_kv_gather_packed(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias,
+                                                cu_dev.data_ptr(), B, 1, k.data_ptr(), v.data_ptr(), int(cu[-1]), nat.current_stream_ptr()))
+        return fn
+    k, v = (torch.empty(B, H, L, D, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    zero = 1 if form == "dense_zero_fill" else 0
+
+    def fn(_keep=(k, v, table, lens_dev)):
+        nat.check(lib.pace_kv_gather(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, B, 1,
+                                     k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, zero, nat.current_stream_ptr()))
+    return fn
+
+
+def wl_gather(torch, dev, args):
+    """Block-table gather of the whole headline cache (batch 64 x 4096 tokens, permuted blocks) back into
+    token rows: 2 x 1.07 GB of algorithmic traffic per call."""
+    B, ctx, hq, hkv, D = 64, 4096, 32, 8, 128
+    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, headroom=16)
+    nbytes = 2 * B * ctx * kv_token_bytes(hkv, D)
+    ms = {form: time_call(torch, gather_call(torch, cache, form), reps=args.steps, warmup=args.warmup) for form in ("dense", "packed")}
+    return result_line(args, "block-table gather: batch 64 x 4096 tokens, 8 KV heads, head_dim 128, permuted blocks -> dense [B,H,L,D]",
+                       nbytes, B * ctx, ms["dense"] * 1e-3, roofline("kv_gather_kernel<128,false> (dense)", nbytes, ms["dense"]),
+                       extra={"packed": roofline("kv_gather_kernel<128,true> (packed)", nbytes, ms["packed"])})
+
+
+def wl_append(torch, dev, args):
+    """KV append on its own (not fused into the attention launch): T new tokens per sequence on top of the
+    headline cache, T = 1 (decode), 8 (verify), 512 (prefill chunk).  Bytes = new K/V read + written."""
+    from pace_mi355 import _native as nat
+
+    B, ctx, hq, hkv, D = 64, 4096, 32, 8, 128
+    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, headroom=512 + 16)
+    lib = nat.load()
+    g = torch.Generator(device=dev).manual_seed(3)
+    res = {}
+    for T in (1, 8, 512):
+        k, v = _randn_bf16(torch, (B, hkv, T, D), g, dev), _randn_bf16(torch, (B, hkv, T, D), g, dev)
+        lens_after = cache.lens + T
+        cache.state.ensure_capacity(lens_after)
+        table = cache.state.device_table()
+        lens_dev = torch.from_numpy(lens_after.astype("int32")).to(dev)
+
+        def fn():
+            nat.check(lib.pace_kv_append_paged(ctypes.byref(cache._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1),
+                                               k.stride(2), B, T, table.data_ptr(), table.stride(0), lens_dev.data_ptr(), -T,
+                                               nat.current_stream_ptr()))
+        ms = time_call(torch, fn, reps=args.steps, warmup=args.warmup)
+        kernel = "kv_append_kernel<128,true>" if T < 8 else "kv_append_block_kernel<128,false>"
+        res[T] = roofline(f"{kernel} ({T} tokens per sequence)", append_bytes(B, T, hkv, D), ms)
+    return result_line(args, "KV append alone: batch 64, 8 KV heads, head_dim 128, 512 / 8 / 1 new tokens per sequence through the block "
+                       "table (headline line: 512)", append_bytes(B, 512, hkv, D), B * 512, res[512]["avg_launch_ms"] * 1e-3, res[512],
+                       extra={"append_8_tokens": res[8], "append_1_token": res[1]})
 
 
 def wl_verify(torch, dev, args):
@@ -499,32 +576,31 @@ def wl_compact(torch, dev, args):
     g = torch.Generator(device=dev).manual_seed(7)
     q = _randn_bf16(torch, (B, hq, 1, D), g, dev)
     block_bytes = 16 * kv_token_bytes(hkv, D)
-    times, moved = [], 0
+    times, walls, moved = [], [], 0
     for rep in range(3):  # compaction is destructive: rebuild, evict, then time one compaction
         cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=6, headroom=0)
         rng = np.random.default_rng(6)
         for b in range(B):
             cache.evict_blocks(b, np.sort(rng.choice(ctx // 16, size=int(0.4 * ctx // 16), replace=False)).tolist())
         torch.cuda.synchronize()
-        # compact() = plan on the host, upload the (src, dst) pairs, copy on the GPU, rewrite the tables;
-        # the copy is bracketed by events, the host part by the wall clock
+        # compact() = plan on the host, upload the (src, dst) pairs, copy on the GPU, rewrite the tables.
+        # Here the same steps, with the copy bracketed by events and the whole by the wall clock
+        # (synchronize on both sides).
         from pace_mi355 import _native as nat
-        t_host = time.perf_counter()
+        t_wall = time.perf_counter()
         moves = cache.state.plan_compaction()
         pairs = torch.from_numpy(moves).pin_memory().to(dev, non_blocking=True)
-        plan_ms = (time.perf_counter() - t_host) * 1e3
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         nat.check(nat.load().pace_kv_copy_blocks(ctypes.byref(cache._desc), ctypes.byref(cache._desc), pairs.data_ptr(),
                                                  len(moves), nat.current_stream_ptr()))
         e1.record()
-        t_host = time.perf_counter()
-        cache.state.apply_moves(moves)
-        plan_ms += (time.perf_counter() - t_host) * 1e3
-        moved = len(moves)
+        cache.state.apply_moves(moves)  # host work overlaps the copy
         torch.cuda.synchronize()
+        walls.append((time.perf_counter() - t_wall) * 1e3)
+        moved = len(moves)
         times.append(e0.elapsed_time(e1))
-        host_ms = plan_ms
+    host_ms = min(walls)
     compact_ms = min(times)
     cache.partition_tokens = args.partition
     lens = cache.lens.tolist()
@@ -535,7 +611,8 @@ def wl_compact(torch, dev, args):
         f"(seed 6), {moved} blocks moved, then decode over {lens[0]} tokens/seq", dec, B, attn_ms * 1e-3,
         roofline("paged_attn_kernel<128,1,...> (decode after compaction) + merge", dec, attn_ms),
         extra={"compaction": roofline("kv_copy_blocks_kernel", 2 * moved * block_bytes, compact_ms,
-                                      {"blocks_moved": moved, "host_plan_ms": round(host_ms, 3)})})
+                                      {"blocks_moved": moved, "end_to_end_ms": round(host_ms, 3),
+                                       "end_to_end_note": "plan + upload + copy + table rewrite, wall clock between two synchronizes"})})
 
 
 def wl_copy_calibration(torch, dev, args):
@@ -607,7 +684,7 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
     }
 
 
-WORKLOADS = {"decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32,
+WORKLOADS = {"gather": wl_gather, "append": wl_append, "decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32,
              "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 

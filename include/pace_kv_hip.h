@@ -101,14 +101,31 @@ int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_new, const vo
  * Produces what the reference cache holds (pace/llm/cache.py:391-399 after
  * repeat_kv, pace/llm/models/llama.py:151-158): k_out / v_out are bf16
  * [batch][num_kv_heads*n_rep][out_len][head_dim] with the element strides
- * given (rows contiguous); rows >= seq_lens[b] are written as zeros.
+ * given (rows contiguous).  Rows >= seq_lens[b] are written as zeros when
+ * zero_fill is non-zero (the reference's BMC buffers are zero-padded,
+ * pace/llm/cache.py:255-266) and left untouched otherwise -- in a ragged batch
+ * the padding is most of the dense tensor.
  * block_table: device int32 [batch][table_stride]; seq_lens: device int32 [batch]
  * (length of sequence b = seq_lens[b] + seq_len_bias).
  */
 int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
                    const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep,
                    void* k_out, void* v_out, int64_t out_stride_b, int64_t out_stride_h,
-                   int32_t out_len, void* stream);
+                   int32_t out_len, int32_t zero_fill, void* stream);
+
+/*
+ * Gather without padding: the same rows packed back to back, k_out / v_out bf16
+ * [sum of lengths][num_kv_heads*n_rep][head_dim] (contiguous), sequence b starting at row
+ * cu_seqlens[b] (device int32 [batch+1], exclusive prefix sum of the lengths).  The rows of a
+ * sequence are the rows [b, :, :len_b, :] of the dense form, token-major.  total_tokens: rows of
+ * k_out / v_out = cu_seqlens[batch], known to the host that allocated them (it sizes the grid -- one
+ * workgroup per block and KV head that can exist, none for padding -- and no row at or past it is written).
+ * Same block_table / seq_lens contract as above.
+ */
+int pace_kv_gather_packed(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                          const int32_t* seq_lens, int32_t seq_len_bias, const int32_t* cu_seqlens,
+                          int32_t batch, int32_t n_rep, void* k_out, void* v_out, int32_t total_tokens,
+                          void* stream);
 
 /*
  * Copy whole blocks (compaction, beam copy-on-write; the reference's only cache

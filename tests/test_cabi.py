@@ -70,7 +70,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     rc = lib.pace_kv_append(ctypes.byref(bad), 16, 16, 8, 8, 8, 1, 1, 16, None)
     assert rc == -1 and b"block_size 32 unsupported" in lib.pace_kv_last_error()
     bad.block_size, bad.head_dim = 16, 80
-    assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 0, 1, 1, 16, 16, 8, 8, 16, None) == -1
+    assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 0, 1, 1, 16, 16, 8, 8, 16, 1, None) == -1
     assert b"head_dim 80 unsupported" in lib.pace_kv_last_error()
     with pytest.raises(_native.NativeError, match="head_dim 80"):
         _native.check(-1)

@@ -97,6 +97,58 @@ def test_ragged_append_truncate_evict_compact(device):
     check("after post-compaction append")
 
 
+@pytest.mark.parametrize("hkv,n_rep,dim", [(2, 1, 128), (8, 4, 128), (2, 2, 64), (1, 3, 256), (2, 1, 80)])
+def test_packed_gather_and_gather_without_zero_fill(device, hkv, n_rep, dim):
+    """The two gather forms that write no padding: packed [sum len][H][D] with cu_seqlens, and the
+    dense layout with the rows past each length left alone.  Both bit-exact on every row a sequence has."""
+    B = 6
+    rng = np.random.default_rng(5)
+    lens = [0, 1, 16, 17, 333, 40]
+    cache = _paged(400, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, dim)
+    k, v = seeded_kv(77, B, hkv, max(lens), dim)
+    cache.append_ragged(k.to(device), v.to(device), lens)
+    model.append(k, v, lens)
+    cache.truncate([0, 0, 3, 0, 13, 0])
+    model.truncate([0, 0, 3, 0, 13, 0])
+    lens = model.seq_lens()
+    for rep in (1, n_rep):
+        K, V = model.dense(rep)
+        pk, pv, cu = cache.gather_packed(n_rep=rep)
+        assert cu.cpu().tolist() == np.concatenate([[0], np.cumsum(lens)]).tolist()
+        assert tuple(pk.shape) == (sum(lens), hkv * rep, dim)
+        want_k = torch.cat([K[b, :, :n].transpose(0, 1) for b, n in enumerate(lens)], dim=0)
+        want_v = torch.cat([V[b, :, :n].transpose(0, 1) for b, n in enumerate(lens)], dim=0)
+        assert_bits_equal(pk, want_k, f"packed K n_rep={rep}")
+        assert_bits_equal(pv, want_v, f"packed V n_rep={rep}")
+        gk, gv = cache.gather(n_rep=rep, zero_fill=False)
+        for b, n in enumerate(lens):
+            assert_bits_equal(gk[b, :, :n], K[b, :, :n], f"K rows of sequence {b}")
+            assert_bits_equal(gv[b, :, :n], V[b, :, :n], f"V rows of sequence {b}")
+
+
+def test_gather_without_zero_fill_leaves_padding_untouched(device):
+    import ctypes
+
+    from pace_mi355 import _native as nat
+
+    B, H, D, L = 2, 2, 128, 40
+    cache = _paged(64)
+    k, v = seeded_kv(3, B, H, 30, D)
+    cache.append_ragged(k.to(device), v.to(device), [30, 5])
+    st = cache.state
+    table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
+    outs = [torch.full((B, H, L, D), 3.0, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    nat.check(nat.load().pace_kv_gather(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, B, 1,
+                                        outs[0].data_ptr(), outs[1].data_ptr(), outs[0].stride(0), outs[0].stride(1), L, 0,
+                                        nat.current_stream_ptr()))
+    torch.cuda.synchronize()
+    for o, src in zip(outs, (k, v)):
+        assert_bits_equal(o[0, :, :30], src[0, :, :30], "rows of sequence 0")
+        assert_bits_equal(o[1, :, :5], src[1, :, :5], "rows of sequence 1")
+        assert bool((o[0, :, 30:] == 3.0).all()) and bool((o[1, :, 5:] == 3.0).all()), "padding rows were written"
+
+
 def test_beam_reorder(device):
     B, H, D = 4, 2, 64
     cache = _paged(128, num_blocks=80)
