@@ -18,7 +18,7 @@ REPO = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "pace_mi355", "_lib")
 LIB = os.path.join(OUT_DIR, "libpace_kv_hip.so")
-SOURCES = ["common.cpp", "kv_ops.hip", "rope.hip", "paged_attn.hip", "dense_attn_mfma.hip", "dense_attn.hip"]
+SOURCES = ["common.cpp", "block_plan.cpp", "kv_ops.hip", "rope.hip", "paged_attn.hip", "dense_attn_mfma.hip", "dense_attn.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

@@ -44,8 +44,9 @@ struct PagedAttnParams {
   int32_t n_qgroups;
   int32_t num_kv_heads;
   long long total_items;  // work items of the launch: KV heads x row groups x (sequence, partition) pairs
-  const int32_t* items;  // optional (sequence, partition) pairs
-  const int32_t* seq_parts;  // optional partitions per sequence (else derived from part_tokens)
+  const int32_t* items;      // optional work list: one descriptor of PACE_ATTN_WORK_INTS ints per (sequence, partition)
+  const int32_t* seq_parts;  // with a work list: partitions per sequence (else derived from part_tokens)
+  int32_t batch;
   int32_t part_tokens;
   int32_t max_parts;  // 1: write bf16 output directly; >1: write partials
   float scale_log2;   // softmax scale * log2(e)

@@ -7,7 +7,9 @@
 // head.  A second small kernel merges the partitions of a sequence.
 //
 // The inner step (one 32-token unit on the matrix cores) is in attn_core.h.
+#include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "attn_core.h"
 
@@ -138,15 +140,35 @@ __device__ __forceinline__ void write_new_tokens(const PagedAttnParams& p, int b
 }
 
 
-// Pool block ids of one wave's token range: up to 128 blocks (2048 tokens), one id per
-// lane in each of two registers, fetched with one coalesced load each and read back
-// with v_readlane (no memory access inside the unit loop).
+// Pool block ids of 64 consecutive units of one wave (128 blocks), one id per lane in each of two
+// registers, fetched with one load each and read back with v_readlane (no memory access inside the
+// unit loop; a wave that walks more than 64 units fetches the next 128 ids when it gets there).
 struct WaveBlockIds {
   int lo, hi;
-  __device__ __forceinline__ int get(int idx) const {  // idx is wave-uniform
+  __device__ __forceinline__ int get(int idx) const {  // idx is wave-uniform, 0..127
     return idx < 64 ? __builtin_amdgcn_readlane(lo, idx) : __builtin_amdgcn_readlane(hi, idx - 64);
   }
 };
+
+// The waves of a workgroup take the partition's 32-token units in turn: wave w walks units w, w + NW,
+// w + 2 NW, ...  Ids of this wave's units first .. first + 63: lane l holds block (l & 1) of unit
+// first + l / 2 in `lo`, of unit first + 32 + l / 2 in `hi`.  The loads depend on nothing but the
+// partition's first token, not on the sequence's length: a table row exists in full, entries past the
+// live blocks are clamped into the pool and belong to units that are never walked.
+template <int NW>
+__device__ __forceinline__ WaveBlockIds load_block_ids(const PagedAttnParams& p, int b, int part_begin, int wave, int first,
+                                                       int lane) {
+  const int32_t* row = p.table + (int64_t)b * p.table_stride;
+  const int at = part_begin / PACE_KV_BLOCK_TOKENS + 2 * (wave + NW * (first + (lane >> 1))) + (lane & 1);
+  const int at2 = at + 2 * NW * 32;
+  const int lo = at < p.table_stride ? row[at] : 0;
+  const int hi = at2 < p.table_stride ? row[at2] : 0;
+  WaveBlockIds ids;
+  // never read outside the pool, whatever the table holds
+  ids.lo = lo < 0 ? 0 : (lo >= p.num_blocks ? p.num_blocks - 1 : lo);
+  ids.hi = hi < 0 ? 0 : (hi >= p.num_blocks ? p.num_blocks - 1 : hi);
+  return ids;
+}
 
 // NW waves per workgroup split the partition's units among themselves and merge their
 // softmax states through LDS.  OCC is the least number of waves that must fit on one SIMD
@@ -168,35 +190,59 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
   static_assert(MERGE_SLOTS * 16 * NQT <= 128, "LDS merge buffer holds at most 128 query rows");
   __shared__ float merge_buf[MERGE_SLOTS * 16 * NQT * (D + 2)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // the same number, known to be uniform
   // Linear work index -> (KV head, row group, sequence, partition); KV head fastest.
   // (32-bit arithmetic: the host keeps total_items below 2^31.)
   const uint32_t L = blockIdx.x;
   const bool active_item = L < (uint32_t)p.total_items;
+  const bool listed = p.items != nullptr;
   int kvh = 0, part = 0, b = 0, qg = 0;
+  int d_parts = 1, d_begin = 0, d_end = -1, d_first = 0, pre_a = 0, pre_b = 0;
   if (active_item) {
     kvh = (int)(L % (uint32_t)p.num_kv_heads);
     const uint32_t rest = L / (uint32_t)p.num_kv_heads;
-    if (p.items) {  // compact work list: no empty entries, longest partitions first
+    if (listed) {
+      // Work list: one 64-byte descriptor per (sequence, partition), in scheduling order.  It carries
+      // everything the first loads need -- the partition's token range and the pool blocks of its first
+      // units -- so a wave's first K / V loads wait for this one read only; the sequence's length, the
+      // rest of its block ids and the query rows are fetched while those loads travel.
       qg = (int)(rest % (uint32_t)p.n_qgroups);
-      const uint32_t item = rest / (uint32_t)p.n_qgroups;
-      b = p.items[2 * (int64_t)item], part = p.items[2 * (int64_t)item + 1];
+      const int32_t* d = p.items + (int64_t)(rest / (uint32_t)p.n_qgroups) * PACE_ATTN_WORK_INTS;
+      b = min(max(d[0], 0), p.batch - 1), part = min(max(d[1], 0), p.max_parts - 1);
+      d_parts = d[2], d_begin = max(d[3], 0) & ~31, d_end = d[4], d_first = d[5];
+      pre_a = d[8 + 2 * wave_s], pre_b = d[9 + 2 * wave_s];
     } else {
       part = (int)(rest % (uint32_t)p.max_parts);
       const uint32_t bz = rest / (uint32_t)p.max_parts;
       b = (int)(bz / (uint32_t)p.n_qgroups), qg = (int)(bz % (uint32_t)p.n_qgroups);
     }
   }
+  UnitRegs<D> buf;
+  bool pre = false;  // buf already holds (or is being sent) this wave's first unit
+  if (listed && wave_s < d_first) {
+    pre_a = pre_a < 0 ? 0 : (pre_a >= p.num_blocks ? p.num_blocks - 1 : pre_a);  // never read outside the pool
+    pre_b = pre_b < 0 ? 0 : (pre_b >= p.num_blocks ? p.num_blocks - 1 : pre_b);
+    load_unit<D, ONCE>(buf, p, kvh, pre_a, pre_b, n, g);
+    pre = true;
+  }
   const int len_b = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
   // An idle slot (past the end of the work, or a partition this sequence does not have) runs
   // as an empty sequence without query rows: it loads and stores nothing but keeps the barriers.
-  const int n_parts_b = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len_b, p.part_tokens);
+  const int n_parts_b = listed ? max(1, d_parts) : partition_count(len_b, p.part_tokens);
   const bool active = active_item && part < n_parts_b;
   const int len = active ? len_b : 0;
   const int n_parts = active ? n_parts_b : 1;
   if (!active) part = 0;
-  const int P = partition_size(len, n_parts);
   const int start = p.kv_start ? p.kv_start[b] : 0;
-  const int part_begin = part * P;
+  // Token range of the partition.  Listed: as the host cut it (the last partition of a sequence is open
+  // ended: it grows with the sequence).  Otherwise: equal shares of the current length.
+  int part_begin, part_end;
+  if (listed) {
+    part_begin = d_begin, part_end = d_end < 0 ? 0x7fffffff : d_end;
+  } else {
+    const int P = partition_size(len, n_parts);
+    part_begin = part * P, part_end = part_begin + P;
+  }
   // Tokens [pool_end, len) are this step's new tokens when the append is fused in.
   const int n_new = FUSED ? min(p.n_new, len) : 0;
   const int pool_end = len - n_new;
@@ -262,7 +308,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
   // full / partial decision per unit is a scalar branch
   min_limit = __builtin_amdgcn_readfirstlane(min_limit);
 
-  int tok_end = min(min(pool_end, part_begin + P), group_end);
+  int tok_end = min(min(pool_end, part_end), group_end);
   if (HAS_MASK && p.row_last) {
     // Explicit mask on a prefill-sized launch: nothing past the last column any row of the group can
     // use is needed (the diagonal of a causal mask) -- provided every row has a real score somewhere,
@@ -282,48 +328,26 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
     for (int o = 1; o < 64; o *= 2) last = max(last, __shfl_xor(last, o, 64));
     if (__all(real)) tok_end = min(tok_end, __builtin_amdgcn_readfirstlane(last) + 1);
   }
-  // This wave's share of the partition's 32-token units.
+  // This wave's share of the partition's 32-token units: units wave, wave + NW, wave + 2 NW, ...
   const int part_units = max(0, (tok_end - part_begin + 31) / 32);
-  const int per_wave = (part_units + NW - 1) / NW;
-  const int u_begin = min(part_units, wave * per_wave);
-  const int n_units = min(part_units, u_begin + per_wave) - u_begin;
-  const int tok_begin = part_begin + 32 * u_begin;
+  const int n_units = part_units > wave ? (part_units - wave + NW - 1) / NW : 0;
 
-  WaveBlockIds ids;
-  {
-    const int first_blk = tok_begin / PACE_KV_BLOCK_TOKENS;
-    const int live_blks = (len + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
-    const int32_t* row = p.table + (int64_t)b * p.table_stride;
-    int lo = 0, hi = 0;
-    if (n_units > 0 && first_blk + lane < live_blks) lo = row[first_blk + lane];
-    if (n_units > 32 && first_blk + 64 + lane < live_blks) hi = row[first_blk + 64 + lane];
-    // never read outside the pool, whatever the table holds
-    ids.lo = lo < 0 ? 0 : (lo >= p.num_blocks ? p.num_blocks - 1 : lo);
-    ids.hi = hi < 0 ? 0 : (hi >= p.num_blocks ? p.num_blocks - 1 : hi);
-  }
-
-  UnitRegs<D> buf;
+  WaveBlockIds ids = load_block_ids<NW>(p, b, part_begin, wave, 0, lane);
+  // a first unit the descriptor did not name (or no descriptor): its blocks come from the table like all others
+  if (!pre && n_units > 0) load_unit<D, ONCE>(buf, p, kvh, ids.get(0), ids.get(1), n, g);
   if (ROPE) {
-    // Put the first unit's loads in flight, then rotate the query rows while they travel.  The
-    // rotation is written out in both arms: after a join the wait for the (older) table loads
-    // would have to assume the worst and cover the unit's loads as well.
-    if (n_units > 0) {
-      load_unit<D, ONCE>(buf, p, kvh, ids.get(0), ids.get(1), n, g);
+    // rotate the query rows while the first unit travels (padding rows stay zero)
 #pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);  // padding rows stay zero
-      asm volatile("; query rows rotated, first unit in flight");  // keeps the two arms from being merged
-    } else {
-#pragma unroll
-      for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
-    }
+    for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
   }
   MaskRegs<NQT> mregs;
   for (int uu = 0; uu < n_units; ++uu) {
-    const int t0 = tok_begin + 32 * uu;  // a multiple of 32: partitions and wave shares are whole units
+    if (uu != 0 && (uu & 63) == 0) ids = load_block_ids<NW>(p, b, part_begin, wave, uu, lane);
+    const int t0 = part_begin + 32 * (wave + NW * uu);  // a multiple of 32: partitions begin on whole units
     // The mask values go first, so that they are back before the unit's K / V: the wait for those
     // is then the only one, as without a mask.
     if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);
-    if (!ROPE || uu > 0) load_unit<D, ONCE>(buf, p, kvh, ids.get(2 * uu), ids.get(2 * uu + 1), n, g);
+    if (uu > 0) load_unit<D, ONCE>(buf, p, kvh, ids.get(2 * (uu & 63)), ids.get(2 * (uu & 63) + 1), n, g);  // the first one is on its way
     const bool full = (t0 + 32 <= tok_end) && (t0 + 31 <= min_limit) && (t0 >= start);
     compute_unit<D, NQT, HAS_MASK>(buf, qreg, st, p, t0, tok_end, start, full, g, mregs);
   }
@@ -470,8 +494,14 @@ __global__ __launch_bounds__(64) void paged_attn_merge_kernel(const PagedAttnPar
   const int s = (int)(row % S);
   const int hq = (int)((row / S) % p.num_q_heads);
   const int b = (int)(row / ((int64_t)S * p.num_q_heads));
-  const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
-  const int n_parts = p.seq_parts ? max(1, p.seq_parts[b]) : partition_count(len, p.part_tokens);
+  int n_parts;
+  if (p.seq_parts) {
+    n_parts = p.seq_parts[b];
+  } else {
+    const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
+    n_parts = partition_count(len, p.part_tokens);
+  }
+  n_parts = min(max(n_parts, 1), p.max_parts);  // the workspace holds max_parts partials per row
   const float* ml = p.part_ml + row * p.max_parts * 2;
   const float* po = p.part_o + row * p.max_parts * D;
   float M = kNegInf;
@@ -562,14 +592,25 @@ static int resolve_partition(int32_t requested, int32_t max_seq_len, int32_t bat
   return (int)per;
 }
 
+// pace_paged_attn_kernel_name(): while this points at a buffer, launch() writes the name of the kernel
+// instantiation it would start there instead of starting it.
+static thread_local char* g_name_out = nullptr;
+static thread_local size_t g_name_cap = 0;
+
 template <int D, int NQT, int NW, int OCC, int OCC_MAX>
 static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
   const bool fused = p.n_new > 0;
   const unsigned blocks = (unsigned)p.total_items;
   // K / V are read once per launch when one group of query rows covers a sequence's rows: always with one
   // or four tiles per wave, never with three, either way with two.
-#define PACE_GO1(M_, F_, R_, O_) \
-  hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_, O_>), dim3(blocks), dim3(64 * NW), 0, s, p)
+#define PACE_GO1(M_, F_, R_, O_)                                                                                          \
+  do {                                                                                                                    \
+    if (g_name_out)                                                                                                       \
+      snprintf(g_name_out, g_name_cap, "pace_kv::paged_attn_kernel<%d, %d, %s, %d, %d, %d, %s, %s, %s>", D, NQT, #M_, NW, OCC, \
+               OCC_MAX, #F_, #R_, (O_) ? "true" : "false");                                                               \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((paged_attn_kernel<D, NQT, M_, NW, OCC, OCC_MAX, F_, R_, O_>), dim3(blocks), dim3(64 * NW), 0, s, p); \
+  } while (0)
 #define PACE_GO(M_, F_, R_)                                                              \
   do {                                                                                   \
     if constexpr (NQT == 2) {                                                            \
@@ -697,12 +738,13 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const int tiles = (rows + 15) / 16;
   const Shape sh = shape_for(pool->head_dim, tiles, a->mask != nullptr);
   const int part = resolve_partition(a->partition_tokens, a->max_seq_len, a->batch, pool->num_kv_heads, rows, pool->head_dim);
-  PACE_REQUIRE(part % 32 == 0 && part >= 32 && part <= max_partition(sh.nw),
-               "%s: partition_tokens %d must be a multiple of 32 in [32, %d]", who, part, partition_cap(pool->head_dim, tiles));
+  PACE_REQUIRE(part % 32 == 0 && part >= 32, "%s: partition_tokens %d must be a positive multiple of 32", who, part);
   int max_parts = a->max_seq_len > 0 ? (a->max_seq_len + part - 1) / part : 1;
-  if (a->seq_parts) {
-    PACE_REQUIRE(a->work_items != nullptr && a->max_parts >= 1,
-                 "%s: seq_parts needs a work list and max_parts (the largest entry of seq_parts)", who);
+  if (a->work_items || a->seq_parts) {
+    PACE_REQUIRE(a->work_items != nullptr && a->seq_parts != nullptr && a->max_parts >= 1 && a->n_work_items >= 1,
+                 "%s: a work list comes with seq_parts, max_parts (the largest entry of seq_parts) and n_work_items; see "
+                 "pace_paged_attn_plan",
+                 who);
     max_parts = a->max_parts;
   }
 
@@ -720,7 +762,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.seq_lens = a->seq_lens, p.len_bias = a->seq_len_bias, p.len_bias_dev = a->seq_len_bias_ptr, p.kv_start = a->kv_start;
   p.mask = a->mask, p.mask_is_f32 = a->mask_dtype == PACE_DTYPE_F32, p.mask_len = a->mask_len;
   p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
-  p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads;
+  p.n_rep = n_rep, p.q_len = a->q_len, p.num_q_heads = a->num_q_heads, p.batch = a->batch;
   p.causal = a->causal;
   p.part_tokens = part, p.max_parts = max_parts;
   p.scale_log2 = a->scale * kLog2e;
@@ -762,7 +804,6 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   p.seq_parts = a->seq_parts;
   long long pairs = (long long)a->batch * max_parts;  // (sequence, partition) pairs of the dense grid
   if (a->work_items) {
-    PACE_REQUIRE(a->n_work_items >= 1, "%s: bad n_work_items %d", who, a->n_work_items);
     p.items = a->work_items;
     pairs = a->n_work_items;
   }
@@ -770,7 +811,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   PACE_REQUIRE(p.total_items < (1ll << 31), "%s: grid too large", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool has_mask = a->mask != nullptr;
-  if (row_last) {
+  if (row_last && !g_name_out) {
     PACE_REQUIRE((long long)a->batch * a->q_len < (1ll << 31), "%s: too many query rows", who);
     hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
     PACE_HIP_CHECK(hipGetLastError());
@@ -778,6 +819,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   bool ok = false;
   for_head_dim(pool->head_dim, [&](auto d) { ok = launch_shape<decltype(d)::value>(sh, p, has_mask, s); });
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
+  if (g_name_out) return PACE_KV_OK;
   PACE_HIP_CHECK(hipGetLastError());
   if (max_parts > 1) {
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
@@ -825,6 +867,127 @@ extern "C" size_t pace_paged_attn_workspace_bytes_for_parts(int32_t batch, int32
   if (batch <= 0 || num_q_heads <= 0 || q_len <= 0 || head_dim <= 0 || max_parts < 1) return 0;
   // rows per KV head are not known here: room for the per-row mask summary whenever the launch could be prefill-sized
   return workspace_need(batch, num_q_heads, q_len, head_dim, max_parts, q_len * num_q_heads);
+}
+
+extern "C" int pace_paged_attn_kernel_name(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, char* out,
+                                           size_t out_bytes) {
+  PACE_REQUIRE(out != nullptr && out_bytes > 0, "pace_paged_attn_kernel_name: no output buffer");
+  out[0] = 0;
+  g_name_out = out, g_name_cap = out_bytes;
+  const int rc = run_paged_attn(pool, args, nullptr, "pace_paged_attn_kernel_name");
+  g_name_out = nullptr, g_name_cap = 0;
+  return rc;
+}
+
+// Host-side planner: how the sequences of a batch are cut into (sequence, partition) work items, in which
+// order they are scheduled, and the descriptors the kernel reads.  Pure host arithmetic on host arrays.
+extern "C" int pace_paged_attn_plan(const int32_t* seq_lens, const int32_t* block_table, int32_t table_stride, int32_t batch,
+                                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t q_len, int32_t masked,
+                                    int32_t partition_tokens, int32_t* work_items, int32_t work_capacity, int32_t* seq_parts,
+                                    pace_attn_plan_t* plan) {
+  const char* who = "pace_paged_attn_plan";
+  PACE_REQUIRE(plan != nullptr, "%s: plan is NULL", who);
+  *plan = pace_attn_plan_t{};
+  PACE_REQUIRE(batch >= 0 && num_q_heads >= 1 && num_kv_heads >= 1 && q_len >= 1 && table_stride >= 1,
+               "%s: bad batch (%d), heads (%d / %d), q_len (%d) or table_stride (%d)", who, batch, num_q_heads, num_kv_heads, q_len,
+               table_stride);
+  PACE_REQUIRE(num_q_heads % num_kv_heads == 0, "%s: num_q_heads %d not a multiple of num_kv_heads %d", who, num_q_heads,
+               num_kv_heads);
+  PACE_REQUIRE(head_dim_supported(head_dim), "%s: head_dim %d unsupported (64, 96, 128 or 256)", who, head_dim);
+  PACE_REQUIRE(partition_tokens >= 0 && partition_tokens % 32 == 0, "%s: partition_tokens %d must be 0 or a multiple of 32", who,
+               partition_tokens);
+  if (batch == 0) return PACE_KV_OK;
+  PACE_REQUIRE(seq_lens && block_table && seq_parts && (work_items || work_capacity == 0), "%s: NULL pointer", who);
+  const int rows = q_len * (num_q_heads / num_kv_heads), tiles = (rows + 15) / 16;
+  const Shape sh = shape_for(head_dim, tiles, masked != 0);
+  const int n_qgroups = (tiles + sh.nqt - 1) / sh.nqt;
+  int64_t total = 0;
+  int max_len = 0;
+  bool uniform = true;
+  for (int b = 0; b < batch; ++b) {
+    PACE_REQUIRE(seq_lens[b] >= 0 && (int64_t)seq_lens[b] <= (int64_t)table_stride * PACE_KV_BLOCK_TOKENS,
+                 "%s: length %d of sequence %d does not fit a table row of %d blocks", who, seq_lens[b], b, table_stride);
+    total += seq_lens[b];
+    max_len = seq_lens[b] > max_len ? seq_lens[b] : max_len;
+    uniform = uniform && seq_lens[b] == seq_lens[0];
+  }
+  // A ragged batch is cut at about its mean length: the long sequences then spread over several workgroups
+  // (scheduled longest first) instead of forming the tail of the launch.
+  int want = partition_tokens;
+  const double mean = (double)total / batch;
+  if (want == 0 && batch > 1 && !uniform && max_len > 1.5 * mean) {
+    want = ((int)mean + 127) / 128 * 128;
+    if (want < 1024) want = 1024;
+  }
+  const int part = max_len > 0 ? resolve_partition(want, max_len, batch, num_kv_heads, rows, head_dim) : 128;
+  const int cap = partition_cap(head_dim, tiles);
+  // Workgroups resident at a time, per (KV head, row group): the launch's slots for (sequence, partition) pairs.
+  const int64_t slots = std::max<int64_t>(1, (int64_t)compute_units() * 4 * sh.occ / sh.nw / ((int64_t)num_kv_heads * n_qgroups));
+  std::vector<int> n(batch);
+  int64_t sum_base = 0, sum_cap = 0;
+  for (int b = 0; b < batch; ++b) {
+    n[b] = std::max(1, (seq_lens[b] + part - 1) / part);
+    sum_base += n[b];
+    sum_cap += std::max(1, (seq_lens[b] + cap - 1) / cap);
+  }
+  if (!uniform && sum_cap < slots && sum_base <= slots) {
+    // The whole launch fits the GPU in one round: choose the partition counts so that the partitions are as
+    // equal as possible and fill the slots (the longest share is cut next, while a cut leaves 256 tokens or more).
+    int64_t used = 0;
+    for (int b = 0; b < batch; ++b) used += n[b] = std::max(1, (seq_lens[b] + cap - 1) / cap);
+    while (used < slots) {
+      int best = -1;
+      double best_size = 0.0;
+      for (int b = 0; b < batch; ++b) {
+        const double size = (double)seq_lens[b] / n[b];
+        if (size > best_size) best_size = size, best = b;
+      }
+      if (best < 0 || (double)seq_lens[best] / (n[best] + 1) < 256.0) break;
+      ++n[best], ++used;
+    }
+  }
+  // Equal partitions of whole 32-token units; none may be empty.
+  std::vector<int> psize(batch);
+  int64_t n_items = 0;
+  int max_parts = 1;
+  for (int b = 0; b < batch; ++b) {
+    psize[b] = std::max(32, partition_size(seq_lens[b], n[b]));
+    n[b] = std::max(1, (seq_lens[b] + psize[b] - 1) / psize[b]);
+    seq_parts[b] = n[b];
+    n_items += n[b];
+    max_parts = std::max(max_parts, n[b]);
+  }
+  plan->n_work_items = (int32_t)std::min<int64_t>(n_items, 0x7fffffff);
+  plan->max_parts = max_parts;
+  plan->partition_tokens = part;
+  plan->workspace_bytes = workspace_need(batch, num_q_heads, q_len, head_dim, max_parts, rows);
+  PACE_REQUIRE(n_items <= work_capacity, "%s: %lld work items do not fit the capacity of %d", who, (long long)n_items, work_capacity);
+  // Scheduling order: longest partitions first in a ragged batch (short tail), as they come otherwise.
+  struct Item { int b, part; double size; };
+  std::vector<Item> items;
+  items.reserve((size_t)n_items);
+  for (int b = 0; b < batch; ++b)
+    for (int i = 0; i < n[b]; ++i) items.push_back({b, i, (double)seq_lens[b] / n[b]});
+  if (!uniform) std::stable_sort(items.begin(), items.end(), [](const Item& x, const Item& y) { return x.size > y.size; });
+  for (size_t k = 0; k < items.size(); ++k) {
+    const Item& it = items[k];
+    int32_t* d = work_items + k * PACE_ATTN_WORK_INTS;
+    const int len = seq_lens[it.b];
+    const int begin = it.part * psize[it.b];
+    const bool last = it.part == n[it.b] - 1;
+    const int end = last ? len : begin + psize[it.b];
+    d[0] = it.b, d[1] = it.part, d[2] = n[it.b], d[3] = begin, d[4] = last ? -1 : end;
+    int first = 0;
+    for (int u = 0; u < PACE_ATTN_WORK_FIRST_UNITS; ++u) {
+      const int j = begin / PACE_KV_BLOCK_TOKENS + 2 * u;
+      const bool whole = begin + 32 * (u + 1) <= end && j + 1 < table_stride && first == u;
+      d[8 + 2 * u] = whole ? block_table[(int64_t)it.b * table_stride + j] : 0;
+      d[9 + 2 * u] = whole ? block_table[(int64_t)it.b * table_stride + j + 1] : 0;
+      if (whole) first = u + 1;
+    }
+    d[5] = first, d[6] = 0, d[7] = 0;
+  }
+  return PACE_KV_OK;
 }
 
 extern "C" int pace_paged_attn_decode(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream) {

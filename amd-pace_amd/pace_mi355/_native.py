@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 9
+ABI_VERSION = 10
 STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
@@ -29,6 +29,10 @@ EXPORTED_SYMBOLS = (
     "pace_rope_apply",
     "pace_rope_append_paged",
     "pace_paged_attn_partition_tokens",
+    "pace_paged_attn_plan",
+    "pace_paged_attn_kernel_name",
+    "pace_kv_plan_compaction",
+    "pace_kv_apply_moves",
     "pace_paged_attn_workspace_bytes",
     "pace_paged_attn_workspace_bytes_for_parts",
     "pace_paged_attn_decode",
@@ -116,6 +120,21 @@ class PagedAttnArgs(Structure):
     ]
 
 
+class AttnPlan(Structure):
+    """``pace_attn_plan_t``."""
+
+    _fields_ = [
+        ("n_work_items", c_int32),
+        ("max_parts", c_int32),
+        ("partition_tokens", c_int32),
+        ("reserved", c_int32),
+        ("workspace_bytes", c_size_t),
+    ]
+
+
+WORK_INTS = 16  # PACE_ATTN_WORK_INTS: int32 per work descriptor
+
+
 class NativeError(RuntimeError):
     """A C-ABI entry point returned a failure code."""
 
@@ -171,6 +190,14 @@ def load() -> ctypes.CDLL:
     )
     lib.pace_paged_attn_partition_tokens.restype = c_int32
     lib.pace_paged_attn_partition_tokens.argtypes = [c_int32] * 7
+    lib.pace_paged_attn_plan.restype = ctypes.c_int
+    lib.pace_paged_attn_plan.argtypes = [c_void_p, c_void_p] + [c_int32] * 8 + [c_void_p, c_int32, c_void_p, POINTER(AttnPlan)]
+    lib.pace_paged_attn_kernel_name.restype = ctypes.c_int
+    lib.pace_paged_attn_kernel_name.argtypes = [P, POINTER(PagedAttnArgs), ctypes.c_char_p, c_size_t]
+    lib.pace_kv_plan_compaction.restype = c_int32
+    lib.pace_kv_plan_compaction.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_int32, c_int32, c_void_p]
+    lib.pace_kv_apply_moves.restype = ctypes.c_int
+    lib.pace_kv_apply_moves.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_int32, c_void_p]
     lib.pace_paged_attn_workspace_bytes.restype = c_size_t
     lib.pace_paged_attn_workspace_bytes.argtypes = [c_int32] * 7
     lib.pace_paged_attn_workspace_bytes_for_parts.restype = c_size_t
@@ -194,22 +221,11 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-def row_groups(query_rows: int, masked: bool = False, head_dim: int = 128) -> int:
-    """Workgroups one (sequence, KV head, partition) needs for ``query_rows`` = q_len * n_rep rows:
-    the library packs 16, 32, 48 or 64 rows per workgroup (one 16-row tile up to 16 rows, two for
-    17..32, four for 33..64, three beyond 64; never more than two with an explicit mask or with
-    head_dim 256)."""
-    tiles = max(1, -(-int(query_rows) // 16))
-    two_at_most = masked or head_dim == 256
-    per_group = 1 if tiles <= 1 else (2 if tiles == 2 or two_at_most else (4 if tiles <= 4 else 3))
-    return -(-tiles // per_group)
-
-
-def workgroup_slots(query_rows: int, head_dim: int = 128) -> int:
-    """Workgroups of one attention launch that are resident at the same time on the 256 compute
-    units: two per unit, except one with head_dim 256 and a single 16-row tile (one wave per SIMD,
-    four waves per workgroup)."""
-    return 512
+def kernel_name(pool_desc: PoolDesc, args: PagedAttnArgs) -> str:
+    """The kernel instantiation an attention call with these arguments launches (nothing is launched)."""
+    buf = ctypes.create_string_buffer(256)
+    check(load().pace_paged_attn_kernel_name(ctypes.byref(pool_desc), ctypes.byref(args), buf, len(buf)))
+    return buf.value.decode()
 
 
 def check(rc: int) -> None:

@@ -134,9 +134,6 @@ class PagedKVCache(KVCacheBase):
         self.state: Optional[PagedState] = None
         self.pool: Optional[torch.Tensor] = None
         self._desc: Optional[nat.PoolDesc] = None
-        self._uniform: Optional[bool] = None  # every sequence has the same length (None: not known)
-        self._plan_key = None
-        self._plan_val = None
         self.lens = np.zeros(0, dtype=np.int64)
         self.seq_len = 0
         self.concat_dim = None
@@ -165,7 +162,6 @@ class PagedKVCache(KVCacheBase):
     @lens.setter
     def lens(self, value: np.ndarray) -> None:
         self._lens = value
-        self._uniform = None
 
     # -- set-up -----------------------------------------------------------------
     def _lazy_init(self, key_states: torch.Tensor) -> None:
@@ -305,9 +301,7 @@ class PagedKVCache(KVCacheBase):
                     B, T, slots.data_ptr(), stream,
                 )
             )
-        uniform = self._uniform if counts is None else None  # equal appends keep equal lengths equal
         self.lens = new_lens
-        self._uniform = uniform
         self.seq_len = self.seq_len + T if counts is None else int(new_lens.max(initial=0))
         if self.key is None:
             self.key, self.value = PagedKVView(self, "key"), PagedKVView(self, "value")
@@ -378,12 +372,12 @@ class PagedKVCache(KVCacheBase):
                 p._flush()
         moves = self.state.plan_compaction()
         if len(moves):
-            pairs = torch.from_numpy(moves).pin_memory().to(self.pool.device, non_blocking=True)
+            pairs = self.state.upload_pairs(moves)
             lib = nat.load()
             for pool in self.state.pools:
                 desc = self._describe(pool)
                 nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), pairs.data_ptr(), len(moves), nat.current_stream_ptr()))
-            self.state.apply_moves(moves)
+            self.state.apply_moves(moves)  # the table rewrite runs on the host while the GPU copies
         return len(moves)
 
     def reorder(self, beam_idx: Sequence[int]) -> None:
@@ -409,7 +403,7 @@ class PagedKVCache(KVCacheBase):
         lens = np.min([p.lens for p in peers], axis=0)  # the earliest position any layer will write
         pairs = st.unshare_tails(lens)
         if len(pairs):
-            dev = torch.from_numpy(pairs).pin_memory().to(self.pool.device, non_blocking=True)
+            dev = st.upload_pairs(pairs)
             lib = nat.load()
             for pool in st.pools:
                 desc = self._describe(pool)
@@ -470,43 +464,6 @@ class PagedKVCache(KVCacheBase):
             k, v = k[..., : self.model_dim].contiguous(), v[..., : self.model_dim].contiguous()
         return k, v, cu_dev
 
-    def _plan(self, B: int, hq: int, S: int, D: int, max_len: int):
-        """How one attention launch is cut: (work items, partitions per sequence, partition size,
-        most partitions per sequence, workspace bytes).  Equal lengths -- the usual decode batch --
-        take a short path that only asks the library again when the partition count changes."""
-        lib = nat.load()
-        if self._uniform is None:
-            self._uniform = bool(self.lens.size == 0 or (self.lens == self.lens[0]).all())
-        want = self.partition_tokens
-        if self._uniform:
-            key = (B, hq, S, D, want, -(-max_len // 128))
-            if key != self._plan_key:
-                part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, max_len, want, self.num_kv_heads))
-                max_parts = max(1, -(-max_len // part)) if part else 1
-                ws = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, -(-max_len // 128) * 128, part, self.num_kv_heads))
-                self._plan_key, self._plan_val = key, (None, None, part, max_parts, ws)
-            return self._plan_val
-        if want == 0 and B > 1:
-            # A ragged batch is cut at about its mean length: the long sequences then spread over
-            # several workgroups (scheduled longest first) instead of forming the tail of the launch.
-            mean = float(self.lens.mean())
-            if max_len > 1.5 * mean:
-                want = max(1024, (int(mean) + 127) // 128 * 128)
-        part = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, max_len, want, self.num_kv_heads))
-        items = parts = None
-        max_parts = 1
-        if part:
-            cap = int(lib.pace_paged_attn_partition_tokens(B, hq, S, self.head_dim, 1 << 30, 0, self.num_kv_heads))
-            rows = S * (hq // self.num_kv_heads)
-            groups = self.num_kv_heads * nat.row_groups(rows, head_dim=self.head_dim)
-            slots = max(1, nat.workgroup_slots(rows, self.head_dim) // groups)
-            items, parts, max_parts = self.state.plan_attention(self.lens, part, cap, slots)
-        if parts is not None:
-            ws_bytes = int(lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
-        else:
-            ws_bytes = int(lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, self.num_kv_heads))
-        return items, parts, part, max_parts, ws_bytes
-
     def attend(self, query: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                kv_start: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``softmax(q K^T / sqrt(D) + mask) V`` of ``query [B, Hq, S, D]`` over this cache.
@@ -539,7 +496,8 @@ class PagedKVCache(KVCacheBase):
         st = self.state
         max_len = self.seq_len
         lib = nat.load()
-        items, parts, part, max_parts, ws_bytes = self._plan(B, hq, S, D, max_len)
+        items, parts, n_items, max_parts, ws_bytes = st.plan_attention(
+            self.lens, hq, self.num_kv_heads, self.head_dim, S, attention_mask is not None, self.partition_tokens)
         ws = st.workspace(ws_bytes)
         table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
         a = nat.PagedAttnArgs()
@@ -566,11 +524,9 @@ class PagedKVCache(KVCacheBase):
         else:
             a.mask, a.causal = None, 1
         a.batch, a.num_q_heads, a.q_len = B, hq, S
-        a.max_seq_len, a.partition_tokens = max_len, part
-        if items is not None:
-            a.work_items, a.n_work_items = items.data_ptr(), items.shape[0]
-        if parts is not None:
-            a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
+        a.max_seq_len, a.partition_tokens = max_len, 0
+        a.work_items, a.n_work_items = items.data_ptr(), n_items
+        a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
         a.scale = 1.0 / math.sqrt(self.model_dim)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes

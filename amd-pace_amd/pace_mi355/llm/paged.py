@@ -10,6 +10,8 @@ from __future__ import annotations
 
 from typing import Iterable, List, Optional, Sequence, Tuple
 
+import ctypes
+
 import numpy as np
 import torch
 
@@ -25,28 +27,30 @@ def blocks_for(n_tokens: int) -> int:
 class BlockAllocator:
     """LIFO free list over pool block ids ``0 .. num_blocks-1`` (lowest ids first), with a
     reference count per block: sequences forked from one another (beam search) point at the
-    same blocks until one of them writes."""
+    same blocks until one of them writes.  The free list is a stack in a numpy array (its top at
+    ``_n_free``), so allocation, release and wholesale rebuilds cost no per-block interpreter work."""
 
     def __init__(self, num_blocks: int):
         self.num_blocks = int(num_blocks)
-        self._free: List[int] = list(range(self.num_blocks - 1, -1, -1))
+        self._stack = np.arange(self.num_blocks - 1, -1, -1, dtype=np.int32)
+        self._n_free = self.num_blocks
         self._is_free = np.ones(self.num_blocks, dtype=bool)
         self.refs = np.zeros(self.num_blocks, dtype=np.int32)
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return self._n_free
 
     def allocate(self, n: int) -> List[int]:
-        if n > len(self._free):
-            raise MemoryError(f"KV block pool exhausted: need {n} blocks, {len(self._free)} free of {self.num_blocks}")
+        if n > self._n_free:
+            raise MemoryError(f"KV block pool exhausted: need {n} blocks, {self._n_free} free of {self.num_blocks}")
         if n == 0:
             return []
-        out = self._free[-n:][::-1]
-        del self._free[-n:]
+        out = self._stack[self._n_free - n:self._n_free][::-1].copy()
+        self._n_free -= n
         self._is_free[out] = False
         self.refs[out] = 1
-        return out
+        return out.tolist()
 
     def share(self, ids: Iterable[int]) -> None:
         """One more owner for each of ``ids`` (an id may occur several times)."""
@@ -58,34 +62,40 @@ class BlockAllocator:
 
     def free(self, ids: Iterable[int]) -> None:
         """Drop one owner of each of ``ids``; a block returns to the free list with its last owner."""
-        ids = [int(i) for i in ids]
-        if not ids:
+        arr = np.asarray(ids if isinstance(ids, np.ndarray) else list(ids), dtype=np.int64)
+        if not arr.size:
             return
-        arr = np.asarray(ids, dtype=np.int64)
         if self._is_free[arr].any():
-            raise ValueError(f"block {[i for i in ids if self._is_free[i]][0]} freed twice")
+            raise ValueError(f"block {int(arr[self._is_free[arr]][0])} freed twice")
         np.subtract.at(self.refs, arr, 1)
         if (self.refs[arr] < 0).any():
-            raise ValueError(f"block {[i for i in ids if self.refs[i] < 0][0]} freed twice")
-        gone = [i for i in dict.fromkeys(ids) if self.refs[i] == 0]
-        if gone:
+            raise ValueError(f"block {int(arr[self.refs[arr] < 0][0])} freed twice")
+        gone = arr[self.refs[arr] == 0]
+        if gone.size:
+            _, first = np.unique(gone, return_index=True)  # an id listed twice is pushed once, in order of appearance
+            gone = gone[np.sort(first)]
             self._is_free[gone] = True
-            self._free.extend(gone)
+            self._stack[self._n_free:self._n_free + gone.size] = gone
+            self._n_free += gone.size
 
     def take(self, ids: Iterable[int]) -> None:
         """Mark specific ids as used (compaction destinations)."""
-        want = set(int(i) for i in ids)
-        for i in want:
-            if not self._is_free[i]:
-                raise ValueError(f"block {i} is not free")
-            self._is_free[i] = False
-            self.refs[i] = 1
-        self._free = [i for i in self._free if i not in want]
+        want = np.unique(np.asarray(list(ids), dtype=np.int64))
+        if want.size and not self._is_free[want].all():
+            raise ValueError(f"block {int(want[~self._is_free[want]][0])} is not free")
+        self._is_free[want] = False
+        self.refs[want] = 1
+        keep = self._stack[:self._n_free]
+        keep = keep[self._is_free[keep]]
+        self._stack[:keep.size] = keep
+        self._n_free = keep.size
 
     def reset_free(self, is_free: np.ndarray, refs: Optional[np.ndarray] = None) -> None:
         """Replace the free list wholesale (lowest ids are handed out first again)."""
         self._is_free = is_free.copy()
-        self._free = np.nonzero(is_free)[0][::-1].tolist()
+        free = np.nonzero(is_free)[0][::-1]
+        self._stack[:free.size] = free
+        self._n_free = free.size
         self.refs = refs.astype(np.int32) if refs is not None else (~is_free).astype(np.int32)
 
     def free_ids(self) -> np.ndarray:
@@ -120,10 +130,17 @@ class PagedState:
         self.min_capacity = 0  # tokens every sequence can hold in the blocks it already owns
         self.has_shared = False  # some block has more than one owner (after a fork)
         self.tails_dirty = False  # a sequence's last, partly filled block may have other owners
+        self.table_version = 0  # bumped when table entries below the sequences' lengths change (not by appends)
         self._items_key = None
         self._items_dev: Optional[torch.Tensor] = None
         self._parts_dev: Optional[torch.Tensor] = None
-        self._max_parts = 1
+        self._items_host: Optional[torch.Tensor] = None
+        self._items_dev_buf: Optional[torch.Tensor] = None
+        self._items_copied = None
+        self._pairs_host: Optional[torch.Tensor] = None
+        self._pairs_dev: Optional[torch.Tensor] = None
+        self._pairs_copied = None
+        self._n_items, self._max_parts, self._plan_ws = 0, 1, 0
 
     # -- capacity ---------------------------------------------------------------
     def _min_blocks(self) -> int:
@@ -162,6 +179,7 @@ class PagedState:
             freed += have - want
             self._table_dirty = True
         if freed:
+            self.table_version += 1
             self.min_capacity = self._min_blocks() * BLOCK
         return freed
 
@@ -193,6 +211,7 @@ class PagedState:
         self.has_shared = bool((self.allocator.refs > 1).any())
         self.tails_dirty = self.has_shared
         self._table_dirty = True
+        self.table_version += 1
         self.min_capacity = self._min_blocks() * BLOCK
 
     def unshare_tails(self, lens: np.ndarray) -> np.ndarray:
@@ -215,6 +234,7 @@ class PagedState:
                 self.table[b, jb] = new
                 pairs.append((old, new))
                 self._table_dirty = True
+                self.table_version += 1
         self.has_shared = bool((self.allocator.refs > 1).any())
         return np.asarray(pairs, dtype=np.int32).reshape(-1, 2)
 
@@ -244,58 +264,73 @@ class PagedState:
         self._lens_host = lens.copy()
         return self._lens_dev, 0
 
-    def plan_attention(self, lens: np.ndarray, part_tokens: int, part_cap: int, slots: int):
-        """How to cut the sequences of a batch for one attention launch.
+    def plan_attention(self, lens: np.ndarray, num_q_heads: int, num_kv_heads: int, head_dim: int, q_len: int,
+                       masked: bool, partition_tokens: int):
+        """Work list of one attention launch over sequences of ``lens`` tokens (new tokens included).
 
-        Returns ``(items, seq_parts, max_parts)``: ``items`` is a device ``int32 [n][2]`` list of
-        (sequence, partition) pairs, longest partitions first, or ``None`` when a dense grid has no
-        empty entries (equal lengths, one partition rule).  ``seq_parts`` (device ``int32 [B]``) is
-        set when the whole launch fits the GPU in one round: the partition counts are then chosen
-        so that the partitions are as equal as possible and fill the ``slots`` workgroup slots
-        (largest-remainder apportionment), instead of all sequences being cut at one length.
+        Returns ``(items, seq_parts, n_items, max_parts, workspace_bytes)``: ``items`` is the device ``int32
+        [n_items][16]`` descriptor list ``pace_paged_attn_plan`` wrote (the cut of every sequence into
+        partitions, in scheduling order, with the pool blocks of each partition's first units), ``seq_parts``
+        the device ``int32 [B]`` partition counts.  A plan is kept while the lengths stay in the same 64-token
+        buckets and no table entry below them changed: appends in between grow the last partition of each
+        sequence, which the kernels follow from the device-side lengths.
         """
-        if lens.size == 0:
-            return None, None, 1
-        base = np.maximum(1, -(-lens // part_tokens))
-        uniform = bool((lens == lens[0]).all())
-        cap_parts = np.maximum(1, -(-lens // part_cap))
-        if not uniform and int(cap_parts.sum()) < slots and int(base.sum()) <= slots:
-            key = ("even", part_cap, slots, (lens // 64).tobytes())
-            if key != self._items_key:
-                n = cap_parts.copy()
-                size = lens / n
-                while int(n.sum()) < slots:
-                    b = int(np.argmax(size))
-                    if lens[b] / (n[b] + 1) < 256:
-                        break
-                    n[b] += 1
-                    size[b] = lens[b] / n[b]
-                self._store_items(key, lens, n, with_parts=True)
-            return self._items_dev, self._parts_dev, self._max_parts
-        if uniform:
-            return None, None, int(base.max())
-        key = ("cut", part_tokens, base.tobytes(), np.argsort(-lens, kind="stable")[:8].tobytes())
-        if key != self._items_key:
-            self._store_items(key, lens, base, with_parts=False)
-        return self._items_dev, None, int(base.max())
-
-    def _upload(self, host: torch.Tensor) -> torch.Tensor:
-        """Asynchronous copy to the device through fresh pinned memory (plain tensor on a CPU state)."""
-        if self.device.type != "cuda":
-            return host
-        return host.pin_memory().to(self.device, non_blocking=True)
-
-    def _store_items(self, key, lens: np.ndarray, n_parts: np.ndarray, with_parts: bool) -> None:
-        seq = np.repeat(np.arange(lens.size), n_parts)
-        first = np.repeat(np.cumsum(n_parts) - n_parts, n_parts)
-        part = np.arange(seq.size) - first
-        size = np.repeat(lens / n_parts, n_parts)
-        order = np.argsort(-size, kind="stable")
-        items = np.stack([seq, part], axis=1)[order].astype(np.int32)
-        self._items_dev = self._upload(torch.from_numpy(items))
-        self._parts_dev = self._upload(torch.from_numpy(n_parts.astype(np.int32))) if with_parts else None
-        self._max_parts = int(n_parts.max())
+        key = (self.table_version, num_q_heads, num_kv_heads, head_dim, q_len, bool(masked), partition_tokens,
+               (lens // 64).tobytes())
+        if key == self._items_key:
+            return self._items_dev, self._parts_dev, self._n_items, self._max_parts, self._plan_ws
+        B = self.batch
+        lens32 = np.ascontiguousarray(lens, dtype=np.int32)
+        cap = int(((lens32 + 31) // 32).sum()) + B  # most work items there can be: a partition holds a unit or more
+        if self._items_host is None or self._items_host.shape[0] < cap + B:
+            size = max(2 * cap, 64) + B
+            pin = self.device.type == "cuda"
+            self._items_copied = None
+            self._items_host = torch.empty((size, nat.WORK_INTS), dtype=torch.int32, pin_memory=pin)
+            self._items_dev_buf = torch.empty((size, nat.WORK_INTS), dtype=torch.int32, device=self.device)
+        host = self._items_host
+        if self._items_copied is not None:
+            self._items_copied.synchronize()  # the upload of the plan before this one has read the staging buffer
+        # row 0 .. : descriptors; the partition counts ride behind them in the same buffer (one upload)
+        plan = nat.AttnPlan()
+        parts_row = host.shape[0] - (B + nat.WORK_INTS - 1) // nat.WORK_INTS
+        parts_ptr = host.data_ptr() + parts_row * nat.WORK_INTS * 4
+        nat.check(nat.load().pace_paged_attn_plan(
+            lens32.ctypes.data, self.table.ctypes.data, self.table.shape[1], B, num_q_heads, num_kv_heads, head_dim, q_len,
+            1 if masked else 0, partition_tokens, host.data_ptr(), parts_row, parts_ptr, ctypes.byref(plan)))
+        n = int(plan.n_work_items)
+        dev = self._items_dev_buf
+        if self.device.type == "cuda":
+            dev[:n].copy_(host[:n], non_blocking=True)
+            dev[parts_row:].copy_(host[parts_row:], non_blocking=True)
+            self._items_copied = torch.cuda.Event()
+            self._items_copied.record()
+        else:
+            dev = host
+        self._items_dev = dev[:n]
+        self._parts_dev = dev[parts_row:].view(-1)[:B]
+        self._n_items, self._max_parts, self._plan_ws = n, int(plan.max_parts), int(plan.workspace_bytes)
         self._items_key = key
+        return self._items_dev, self._parts_dev, n, self._max_parts, self._plan_ws
+
+    def upload_pairs(self, pairs: np.ndarray) -> torch.Tensor:
+        """Device copy of an ``int32 [n][2]`` list of (src, dst) blocks, through a pinned staging buffer that
+        is kept (allocating pinned memory costs more than the copy of a few thousand pairs)."""
+        n = len(pairs)
+        if self.device.type != "cuda":
+            return torch.from_numpy(np.ascontiguousarray(pairs, dtype=np.int32))
+        if self._pairs_host is None or self._pairs_host.shape[0] < n:
+            size = max(1024, 2 * n)
+            self._pairs_copied = None
+            self._pairs_host = torch.empty((size, 2), dtype=torch.int32, pin_memory=True)
+            self._pairs_dev = torch.empty((size, 2), dtype=torch.int32, device=self.device)
+        if self._pairs_copied is not None:
+            self._pairs_copied.synchronize()  # the upload before this one has read the staging buffer
+        self._pairs_host.numpy()[:n] = pairs
+        self._pairs_dev[:n].copy_(self._pairs_host[:n], non_blocking=True)
+        self._pairs_copied = torch.cuda.Event()
+        self._pairs_copied.record()
+        return self._pairs_dev[:n]
 
     def workspace(self, nbytes: int) -> Optional[torch.Tensor]:
         if nbytes == 0:
@@ -337,6 +372,7 @@ class PagedState:
         self.table[b, : len(keep)] = row
         self.n_blocks[b] = len(keep)
         self._table_dirty = True
+        self.table_version += 1
         self.min_capacity = self._min_blocks() * BLOCK
         out = lens.copy()
         out[b] -= removed_tokens
@@ -350,26 +386,28 @@ class PagedState:
         """Moves that pack all live blocks into ids ``0 .. n_live-1`` with the
         fewest copies: every live block at or above ``n_live`` moves into a free
         id below it.  Returns ``[n_moves, 2]`` int32 ``(src, dst)``; the two id
-        sets are disjoint."""
-        is_live = np.zeros(self.allocator.num_blocks, dtype=bool)
-        is_live[self.table[self._live_mask()]] = True
-        n_live = int(is_live.sum())
-        src = np.nonzero(is_live[n_live:])[0] + n_live
-        dst = np.nonzero(~is_live[:n_live])[0]
-        assert src.size == dst.size
-        return np.stack([src, dst], axis=1).astype(np.int32) if src.size else np.zeros((0, 2), np.int32)
+        sets are disjoint.  (The passes over the table run in the library.)"""
+        moves = np.empty((self.allocator.num_blocks, 2), dtype=np.int32)
+        n = int(nat.load().pace_kv_plan_compaction(
+            self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch, self.allocator.num_blocks,
+            moves.ctypes.data, moves.shape[0], 0, None))
+        if n < 0:
+            nat.check(n)
+        return moves[:n]
 
     def apply_moves(self, moves: np.ndarray) -> None:
-        """Rewrite the tables and the free list after the data of ``moves`` was copied."""
+        """Rewrite the tables and the free list for ``moves`` (whose data the caller copies; the copy may
+        still be running: nothing here touches the device)."""
         if not len(moves):
             return
-        remap = np.arange(self.allocator.num_blocks, dtype=np.int32)
-        remap[moves[:, 0]] = moves[:, 1]
-        mask = self._live_mask()
-        self.table[mask] = remap[self.table[mask]]
-        refs = np.bincount(self.table[mask], minlength=self.allocator.num_blocks).astype(np.int32)
+        moves = np.ascontiguousarray(moves, dtype=np.int32)
+        refs = np.empty(self.allocator.num_blocks, dtype=np.int32)
+        nat.check(nat.load().pace_kv_apply_moves(
+            self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch, self.allocator.num_blocks,
+            moves.ctypes.data, len(moves), refs.ctypes.data))
         self.allocator.reset_free(refs == 0, refs)
         self._table_dirty = True
+        self.table_version += 1
 
     def live_block_count(self) -> int:
         """Pool blocks in use (a block with several owners counts once)."""

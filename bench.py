@@ -45,9 +45,26 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix-core peak, published
 MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X fp32 matrix-core peak, published
 METRIC = "decode-attention+KV-append HBM GB/s (% of peak) & tokens/s, 8B shape, 1 GPU"
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, scaled by the
-# same counters on the copy-calibration workload (figures and commands: profiles/decode_8b_paged_attn_kernel.txt).
-MEASURED_TRAFFIC_BYTES = {"decode-8b": 1_075_000_000}
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` as the committed counter summary states them, or None.
+
+    profiles/decode_8b_paged_attn_kernel.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE runs of the default workload,
+    scaled by the same counters on the copy-calibration workload) ends in a line
+    `traffic_bytes_per_launch <bytes> kernel <name as the profiler prints it>`.  The figure is used only when
+    that name is the instantiation this run launches (asked from the library), so a change of the kernel's
+    template arguments drops the figure instead of carrying a stale one."""
+    path = os.path.join(REPO, "profiles", "decode_8b_paged_attn_kernel.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch "):
+                _, nbytes, _, name = line.rstrip("\n").split(" ", 3)
+                if name.strip() == kernel:
+                    return int(nbytes)
+    except OSError:
+        pass
+    return None
 
 
 def kv_token_bytes(kv_heads, head_dim):
@@ -131,24 +148,15 @@ class FixedStep:
             a.mask, a.mask_dtype, a.mask_len, a.causal = mask.data_ptr(), nat.DTYPE_BF16, mask.shape[3], 0
             a.mask_stride_b, a.mask_stride_s = mask.stride(0), mask.stride(2)
         a.batch, a.num_q_heads, a.q_len = B, hq, S
-        if partition == 0 and max_len > 1.5 * float(lens_after.mean()):  # same rule as PagedKVCache.attend
-            partition = max(1024, (int(lens_after.mean()) + 127) // 128 * 128)
-        part = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, cache.head_dim, max_len, partition, cache.num_kv_heads))
-        cap = int(self.lib.pace_paged_attn_partition_tokens(B, hq, S, cache.head_dim, 1 << 30, 0, cache.num_kv_heads))
-        rows = S * (hq // cache.num_kv_heads)
-        slots = max(1, nat.workgroup_slots(rows, cache.head_dim) // (cache.num_kv_heads * nat.row_groups(rows, head_dim=cache.head_dim)))
-        # ragged batches: compact longest-first work list; single-round launches: evened-out partition counts
-        self.items, self.parts, max_parts = cache.state.plan_attention(lens_after, part, cap, slots)
-        a.max_seq_len, a.partition_tokens, a.scale = max_len, part, 1.0 / math.sqrt(D)
-        if self.parts is not None:
-            ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes_for_parts(B, hq, S, D, max_parts))
-            a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
-        else:
-            ws_bytes = int(self.lib.pace_paged_attn_workspace_bytes(B, hq, S, D, max_len, part, cache.num_kv_heads))
+        # the library's planner cuts the batch: descriptors of (sequence, partition) work items in scheduling order
+        self.items, self.parts, n_items, max_parts, ws_bytes = cache.state.plan_attention(
+            lens_after, hq, cache.num_kv_heads, cache.head_dim, S, mask is not None, partition)
+        a.max_seq_len, a.partition_tokens, a.scale = max_len, 0, 1.0 / math.sqrt(D)
+        a.work_items, a.n_work_items = self.items.data_ptr(), n_items
+        a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
         self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
-        if self.items is not None:
-            a.work_items, a.n_work_items = self.items.data_ptr(), self.items.shape[0]
+        self.n_items, self.max_parts = n_items, max_parts
         self.fused = fused
         if fused:  # the attention launch reads the new tokens from k_new / v_new and stores them into the pool
             a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
@@ -164,6 +172,7 @@ class FixedStep:
         self.args, self.q = a, q
         self.attn = self.lib.pace_paged_attn_decode if S == 1 else self.lib.pace_paged_attn_verify
         self.stream = nat.current_stream_ptr()
+        self.kernel = nat.kernel_name(cache._desc, a)  # the instantiation these arguments launch
 
     def append(self):
         k, v = self.k, self.v
@@ -266,7 +275,7 @@ def wl_decode_8b(torch, dev, args):
     return _wl_decode(torch, dev, args, (64, 4096, 32, 8, 128),
                       "Llama-3-8B-shape single-layer decode: batch 64, context 4096 (+1 appended), 32 Q / 8 KV heads, head_dim 128, "
                       "KV block 16, seeded random physical block permutation, 1-token append + GQA decode",
-                      MEASURED_TRAFFIC_BYTES["decode-8b"], with_cpu=True)
+                      True, with_cpu=True)
 
 
 def wl_decode_gptj(torch, dev, args):
@@ -274,10 +283,10 @@ def wl_decode_gptj(torch, dev, args):
     as the headline with half the context."""
     return _wl_decode(torch, dev, args, (64, 2048, 16, 16, 256),
                       "GPT-J-6B-shape single-layer decode: batch 64, context 2048 (+1 appended), 16 Q / 16 KV heads, head_dim 256, "
-                      "KV block 16, seeded random physical block permutation, 1-token append + decode", None, with_cpu=False)
+                      "KV block 16, seeded random physical block permutation, 1-token append + decode", False, with_cpu=False)
 
 
-def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
+def _wl_decode(torch, dev, args, shape, label, has_traffic_profile, with_cpu):
     B, ctx, hq, hkv, D = shape
     # One pool per layer, each with its own seeded block permutation: step i runs on pool i mod N, as a
     # decoder walks its layers (pace/llm/models/llama.py:312-315), so no step finds the K / V of the step
@@ -337,10 +346,11 @@ def _wl_decode(torch, dev, args, shape, label, traffic, with_cpu):
     dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
     fused = args.path == "direct" and not args.no_fuse or args.path == "api"
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
+    kernel = fixed[0].kernel if args.path == "direct" else "pace_kv::paged_attn_kernel (through PagedKVCache / MultiHeadAttention)"
+    traffic = measured_traffic(kernel) if has_traffic_profile else None
     line = result_line(
         args, label, dec + append_bytes(B, 1, hkv, D), B, dt,
-        roofline(f"paged_attn_kernel<{D},1,...> (decode" + (", append fused in)" if fused else ")"), launch_bytes, attn_ms,
-                 {"traffic": traffic}),
+        roofline(kernel + (" (decode, append fused in)" if fused else " (decode)"), launch_bytes, attn_ms, {"traffic": traffic}),
         {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct"),
          "mask": bool(args.mask and args.path == "api"), "layers": n_layers,
          "distinct_pool_bytes": int(n_layers * B * ctx * kv_token_bytes(hkv, D))})
@@ -373,7 +383,7 @@ def wl_ragged(torch, dev, args):
     return result_line(
         args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x, "
         "1-token append + GQA decode", dec + append_bytes(B, 1, hkv, D), B, dt,
-        roofline("paged_attn_kernel<128,1,...> (decode, ragged) + merge", dec, attn_ms),
+        roofline(step.kernel + " (decode, ragged) + merge", dec, attn_ms, {"work_items": step.n_items, "max_parts": step.max_parts}),
         extra={"gather": forms})
 
 
@@ -466,8 +476,8 @@ def wl_verify(torch, dev, args):
     return result_line(
         args, "PARD speculative verify: batch 32, contexts U[1024,8192] (seed 4), 8 draft tokens appended + causal "
         "8-query attention", dec + append_bytes(B, S, hkv, D), B * S, dt,
-        roofline("paged_attn_kernel<128,2,...> (verify)", dec, attn_ms,
-                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2)}))
+        roofline(step.kernel + " (verify) + merge", dec, attn_ms,
+                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2), "work_items": step.n_items, "max_parts": step.max_parts}))
 
 
 def wl_prefill(torch, dev, args):
@@ -495,7 +505,7 @@ def wl_prefill(torch, dev, args):
     return result_line(
         args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
         "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
-        {"bound": "mfma", "kernel": "paged_attn_kernel<128,2,true,...> (prefill chunk, explicit mask)" if args.mask else "paged_attn_kernel<128,3,...> (prefill chunk)", "achieved": round(tflops, 1),
+        {"bound": "mfma", "kernel": step.kernel + (" (prefill chunk, explicit mask)" if args.mask else " (prefill chunk)"), "achieved": round(tflops, 1),
          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5),
          "hbm_gbs_if_kv_read_once": round(kv_once / (attn_ms * 1e-3) / 1e9, 1)},
@@ -582,20 +592,21 @@ def wl_compact(torch, dev, args):
         rng = np.random.default_rng(6)
         for b in range(B):
             cache.evict_blocks(b, np.sort(rng.choice(ctx // 16, size=int(0.4 * ctx // 16), replace=False)).tolist())
+        cache.state.upload_pairs(np.zeros((8192, 2), dtype=np.int32))  # a cache that lives on has its staging buffer already
         torch.cuda.synchronize()
-        # compact() = plan on the host, upload the (src, dst) pairs, copy on the GPU, rewrite the tables.
-        # Here the same steps, with the copy bracketed by events and the whole by the wall clock
-        # (synchronize on both sides).
+        # PagedKVCache.compact(): plan the moves (native pass over the table), upload the (src, dst) pairs, start
+        # the copy, rewrite the table and the free list while the GPU copies.  Here the same steps, with the copy
+        # bracketed by events and the whole by the wall clock (synchronize on both sides).
         from pace_mi355 import _native as nat
         t_wall = time.perf_counter()
         moves = cache.state.plan_compaction()
-        pairs = torch.from_numpy(moves).pin_memory().to(dev, non_blocking=True)
+        pairs = cache.state.upload_pairs(moves)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         nat.check(nat.load().pace_kv_copy_blocks(ctypes.byref(cache._desc), ctypes.byref(cache._desc), pairs.data_ptr(),
                                                  len(moves), nat.current_stream_ptr()))
         e1.record()
-        cache.state.apply_moves(moves)  # host work overlaps the copy
+        cache.state.apply_moves(moves)
         torch.cuda.synchronize()
         walls.append((time.perf_counter() - t_wall) * 1e3)
         moved = len(moves)
@@ -635,52 +646,58 @@ def wl_copy_calibration(torch, dev, args):
                        roofline("kv_copy_blocks_kernel", nbytes, ms, {"bytes_read": nbytes // 2, "bytes_written": nbytes // 2}))
 
 
-def cpu_baseline(torch, batch, ctx, hq, hkv, D, budget_s=12.0):
-    """The reference's CPU path, restated by the oracle, on a bounded sample of the workload:
-    BMC cache (its benchmark default) holding GQA-expanded K/V + torch SDPA in bf16."""
+def cpu_baseline(torch, batch, ctx, hq, hkv, D, warmup=2, timed=5):
+    """The reference's CPU path, restated by the oracle, at the full batch of the workload: GQA-expanded K/V
+    in the reference's cache + torch CPU SDPA in bf16 (pace/llm/models/llama.py:151-165).  Two legs: the BMC
+    cache its benchmark configuration selects (benchmarks/llm/performance/benchmark_config.json) and the
+    DYNAMIC cache its generator defaults to (pace/llm/llm.py:59), whose torch.cat re-copies the whole cache on
+    every step (pace/llm/cache.py:391-395).  2 warm-up + 5 timed steps, as the reference's benchmark runs
+    (benchmark_config.json:29-30)."""
     from oracle.attention_ref import lengths_mask_4d, sdpa_native
-    from oracle.cache_ref import BMCKVCacheRef, repeat_kv
+    from oracle.cache_ref import BMCKVCacheRef, DynamicKVCacheRef, repeat_kv
 
     cores = torch.get_num_threads()
-    B = 8
-    n_rep = hq // hkv
+    B, n_rep = batch, hq // hkv
     g = torch.Generator().manual_seed(0)
-    cache = BMCKVCacheRef(ctx + 128)
     k = torch.randn(B, hkv, ctx, D, generator=g).to(torch.bfloat16)
     v = torch.randn(B, hkv, ctx, D, generator=g).to(torch.bfloat16)
-    cache.update_cache(repeat_kv(k, n_rep), repeat_kv(v, n_rep), 2)
-    del k, v
     k1 = torch.randn(B, hkv, 1, D, generator=g).to(torch.bfloat16)
     v1 = torch.randn(B, hkv, 1, D, generator=g).to(torch.bfloat16)
     q = torch.randn(B, hq, 1, D, generator=g).to(torch.bfloat16)
-
-    def step():
-        ke, ve = repeat_kv(k1, n_rep), repeat_kv(v1, n_rep)
-        K, V = cache.update_cache(ke, ve, 2)
-        n = cache.seq_len
-        mask = cache.update_mask(lengths_mask_4d([n] * B, 1, n, torch.bfloat16), n)
-        out = sdpa_native(q, K, V, mask)
-        cache.remove_cache(1)
-        return out
-
-    for _ in range(2):
-        step()
-    t0 = time.perf_counter()
-    n_steps = 0
-    while n_steps < 5 or (time.perf_counter() - t0 < budget_s and n_steps < 200):
-        step()
-        n_steps += 1
-    dt = (time.perf_counter() - t0) / n_steps
     nbytes = decode_bytes([ctx + 1] * B, hq, hkv, D) + append_bytes(B, 1, hkv, D)
+    legs = {}
+    for name, cls in (("bmc", BMCKVCacheRef), ("dynamic", DynamicKVCacheRef)):
+        cache = cls(ctx + 128)
+        cache.update_cache(repeat_kv(k, n_rep).contiguous(), repeat_kv(v, n_rep).contiguous(), 2)
+
+        def step():
+            ke, ve = repeat_kv(k1, n_rep), repeat_kv(v1, n_rep)
+            K, V = cache.update_cache(ke, ve, 2)
+            n = cache.seq_len
+            mask = cache.update_mask(lengths_mask_4d([n] * B, 1, n, torch.bfloat16), n)
+            out = sdpa_native(q, K, V, mask)
+            cache.remove_cache(1)  # every step runs at the same cache state, like the GPU line
+            return out
+
+        for _ in range(warmup):
+            step()
+        t0 = time.perf_counter()
+        for _ in range(timed):
+            step()
+        dt = (time.perf_counter() - t0) / timed
+        legs[name] = {"value": round(nbytes / dt / 1e9, 3), "tokens_per_s": round(B / dt, 2), "ms_per_step": round(dt * 1e3, 3)}
+        del cache
     return {
-        "value": round(nbytes / dt / 1e9, 3),
+        "value": legs["bmc"]["value"],
         "unit": "GB/s",
-        "tokens_per_s": round(B / dt, 2),
-        "ms_per_step": round(dt * 1e3, 3),
+        "tokens_per_s": legs["bmc"]["tokens_per_s"],
+        "ms_per_step": legs["bmc"]["ms_per_step"],
         "cores": cores,
         "kind": "port",
-        "sample": f"batch {B} of {batch}, context {ctx}, BMC cache with GQA-expanded K/V + torch CPU SDPA bf16; "
-                  f"2 warm-up + {n_steps} timed steps; GB/s uses the same GQA-minimal algorithmic bytes as the GPU line",
+        "sample": f"the whole workload: batch {B}, context {ctx}, BMC cache with GQA-expanded K/V + torch CPU SDPA bf16; "
+                  f"{warmup} warm-up + {timed} timed steps; GB/s uses the same GQA-minimal algorithmic bytes as the GPU line",
+        "dynamic_cache": dict(legs["dynamic"], note="the same step with the reference's default DYNAMIC cache (torch.cat of the "
+                                                    "whole cache per step)"),
     }
 
 

@@ -137,6 +137,24 @@ int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst,
                         const int32_t* pairs, int32_t n_pairs, void* stream);
 
 /*
+ * Host-side compaction plan (no GPU work; host arrays).  block_table [batch][table_stride] with
+ * n_blocks[b] entries in use per row.  Finds the moves that pack the live blocks into ids 0 .. n_live-1 with
+ * the fewest copies (every live block at or above n_live goes to a free id below it), writes them to
+ * moves [capacity][2] = (src, dst) -- the layout pace_kv_copy_blocks takes -- and, when apply is non-zero,
+ * rewrites the table in place and fills refs [num_blocks] with the owners of every block after the moves.
+ * Returns the number of moves, or a negative code.  A block owned by several rows moves once.
+ */
+int32_t pace_kv_plan_compaction(int32_t* block_table, int32_t table_stride, const int64_t* n_blocks,
+                                int32_t batch, int32_t num_blocks, int32_t* moves, int32_t capacity,
+                                int32_t apply, int32_t* refs);
+
+/* The second half of pace_kv_plan_compaction on its own: rewrite the table for moves [n_moves][2] whose data
+ * is being copied, and count the owners of every block into refs [num_blocks].  (Planning, starting the copy
+ * and then applying lets the host's table rewrite run while the GPU copies.) */
+int pace_kv_apply_moves(int32_t* block_table, int32_t table_stride, const int64_t* n_blocks, int32_t batch,
+                        int32_t num_blocks, const int32_t* moves, int32_t n_moves, int32_t* refs);
+
+/*
  * Rotary position embedding, the step the models run on q and k right before the
  * append (pace/llm/models/llama.py:147-158; operator pace/ops/rotary_embedding.py:370-474).
  * cos / sin: device tables [table_rows][rotary_dim/2] as RotaryEmbedding builds them
@@ -219,18 +237,18 @@ typedef struct pace_paged_attn_args {
   const void* v_new;
   int64_t new_stride_b, new_stride_h, new_stride_t;
   int32_t n_new;
-  /* Optional compact work list (NULL = a dense partition x sequence grid).  Device int32
-   * [n_work_items][2] = (sequence, partition): exactly the pairs with partition <
-   * ceil(seq_len / partition_tokens), in the order they should be scheduled (longest first
-   * shortens the tail of a ragged batch).  Needs an explicit partition_tokens. */
+  /* Optional work list (NULL = a dense partition x sequence grid whose partitions the kernel derives from
+   * each length and partition_tokens).  Device int32 [n_work_items][PACE_ATTN_WORK_INTS], one descriptor per
+   * (sequence, partition) in the order they should be scheduled, as pace_paged_attn_plan() writes them (layout
+   * below).  A descriptor carries the partition's token range and the pool blocks of its first units, so a
+   * workgroup's first K / V loads wait for one 64-byte read instead of the length -> block table -> K / V chain;
+   * the ranges are fixed by the host, and only the last partition of a sequence (open ended) grows with it.
+   * The list stays valid while the lengths only grow and the block-table entries below the planned lengths
+   * keep their values (appends qualify; rollback, eviction, compaction and beam forks need a new plan).
+   * With a work list, seq_parts (device int32 [batch]: partitions of each sequence) and max_parts (its
+   * largest entry) are required, and the workspace is sized by pace_paged_attn_workspace_bytes_for_parts(). */
   const int32_t* work_items;
   int32_t n_work_items;
-  /* Optional partition count per sequence (device int32 [batch], NULL = ceil(seq_len /
-   * partition_tokens)); sequence b is cut into seq_parts[b] equal partitions, none longer than
-   * pace_paged_attn_partition_tokens(...)'s upper bound.  Needs work_items listing exactly
-   * (b, 0 .. seq_parts[b]-1), max_parts = the largest entry, and a workspace of
-   * pace_paged_attn_workspace_bytes_for_parts(...).  Lets the caller even out the work when
-   * the whole launch fits the GPU in one round. */
   const int32_t* seq_parts;
   int32_t max_parts;
   int32_t seq_len_bias;       /* host-side constant added to every seq_lens entry, so that uniform
@@ -254,6 +272,48 @@ typedef struct pace_paged_attn_args {
 int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q_heads, int32_t q_len,
                                          int32_t head_dim, int32_t max_seq_len,
                                          int32_t partition_tokens, int32_t num_kv_heads);
+
+/*
+ * Work descriptor of one (sequence, partition), PACE_ATTN_WORK_INTS int32:
+ *   [0] sequence   [1] partition index   [2] partitions of the sequence
+ *   [3] first token (multiple of 32)     [4] one past the last token, -1 = up to the sequence's length
+ *   [5] n: how many of the unit entries below are set   [6..7] 0
+ *   [8 + 2u], [9 + 2u], u < PACE_ATTN_WORK_FIRST_UNITS: pool block ids of tokens first + 32u .. first + 32u + 31
+ *       (set for the leading units that lay wholly below the planned length)
+ */
+#define PACE_ATTN_WORK_INTS 16
+#define PACE_ATTN_WORK_FIRST_UNITS 4
+
+typedef struct pace_attn_plan {
+  int32_t n_work_items;     /* descriptors written (or needed, when the capacity was too small)  */
+  int32_t max_parts;        /* largest entry of seq_parts                                        */
+  int32_t partition_tokens; /* the split size the cut started from (informational)               */
+  int32_t reserved;
+  size_t workspace_bytes;   /* scratch a launch with this plan needs                             */
+} pace_attn_plan_t;
+
+/*
+ * Host-side planner for one attention launch; no GPU work, every pointer is host memory.  It stands where the
+ * reference has nothing: its attention walks one contiguous [B, H, L, D] tensor per call
+ * (csrc/ops/kernels/attention_kernels.cpp:218-257).  seq_lens [batch]: the lengths the launch will see
+ * (new tokens included); block_table [batch][table_stride]: the host copy of the table.  Cuts every sequence
+ * into equal partitions of whole 32-token units -- at partition_tokens (0: chosen from the sizes; a ragged
+ * batch is cut at about its mean length), or, when the whole launch fits the GPU in one round, into the
+ * partition counts that make the partitions most equal -- and writes the descriptors to work_items
+ * (capacity in descriptors; longest partitions first in a ragged batch) and the counts to seq_parts [batch].
+ * masked: the launch will carry an explicit mask (changes the launch shape).  The caller uploads both
+ * arrays and passes them, with plan->max_parts and plan->n_work_items, in pace_paged_attn_args_t.
+ */
+int pace_paged_attn_plan(const int32_t* seq_lens, const int32_t* block_table, int32_t table_stride,
+                         int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                         int32_t q_len, int32_t masked, int32_t partition_tokens,
+                         int32_t* work_items, int32_t work_capacity, int32_t* seq_parts,
+                         pace_attn_plan_t* plan);
+
+/* Name of the kernel instantiation pace_paged_attn_decode / _verify would launch for these arguments, as a
+ * profiler prints it (nothing is launched): lets a measurement be tied to the kernel it was taken on. */
+int pace_paged_attn_kernel_name(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args,
+                                char* out, size_t out_bytes);
 
 /* Scratch bytes the two entry points below need for these sizes (0 = none): the partial results
  * of sequences cut into several partitions and, for launches of more than 64 query rows per KV

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in _declared_functions():
         assert getattr(lib, name) is not None, name
     assert lib.pace_kv_abi_version() == _native.ABI_VERSION
-    assert lib.pace_kv_last_error() == b""
+    assert isinstance(lib.pace_kv_last_error(), bytes)  # "" until a call on this thread fails
 
 
 def test_struct_layouts_match_the_header():
@@ -57,6 +57,8 @@ def test_struct_layouts_match_the_header():
     assert fields("pace_kv_pool") == [f[0] for f in _native.PoolDesc._fields_]
     assert fields("pace_paged_attn_args") == [f[0] for f in _native.PagedAttnArgs._fields_]
     assert fields("pace_rope") == [f[0] for f in _native.RopeDesc._fields_]
+    assert fields("pace_attn_plan") == [f[0] for f in _native.AttnPlan._fields_]
+    assert int(re.search(r"#define PACE_ATTN_WORK_INTS (\d+)", text).group(1)) == _native.WORK_INTS
     assert ctypes.sizeof(_native.PoolDesc) == 64
 
 

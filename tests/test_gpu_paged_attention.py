@@ -51,6 +51,37 @@ def test_decode_matches_oracle(device, B, hkv, n_rep, D, lens, partition):
     assert_attention_close(out, ref, f"decode lens={lens}")
 
 
+@pytest.mark.parametrize("listed", [True, False])
+def test_partitions_longer_than_one_fetch_of_block_ids(device, listed):
+    """A wave holds the pool block ids of 64 of its units and fetches the next ones when it gets there: one
+    partition of 20 000 tokens is 157 units per wave.  Through the planner's work list, and through the plain
+    grid of a caller that passes no list."""
+    import ctypes
+    import math
+
+    from pace_mi355 import _native as nat
+
+    B, hkv, n_rep, D, lens = 2, 1, 4, 128, [20000, 9000]
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=99, partition=32768)
+    q = seeded_q(7, B, hkv * n_rep, 1, D)
+    ref = model.attention(q, n_rep)
+    if listed:
+        out = cache.attend(q.to(device))
+    else:
+        qd = q.to(device)
+        out = torch.zeros_like(qd)
+        st = cache.state
+        table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
+        a = nat.PagedAttnArgs()
+        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = qd.data_ptr(), qd.stride(0), qd.stride(1), qd.stride(2)
+        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+        a.block_table, a.table_stride, a.seq_lens, a.seq_len_bias = table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias
+        a.causal, a.batch, a.num_q_heads, a.q_len = 1, B, hkv * n_rep, 1
+        a.max_seq_len, a.partition_tokens, a.scale = max(lens), 32768, 1.0 / math.sqrt(D)
+        nat.check(nat.load().pace_paged_attn_decode(ctypes.byref(cache._desc), ctypes.byref(a), nat.current_stream_ptr()))
+    assert_attention_close(out, ref, "20 000-token partition")
+
+
 def test_decode_empty_sequence_gives_zero(device):
     cache, model = _build(device, 2, 2, 2, 128, [0, 40], seed=3)
     q = seeded_q(1, 2, 4, 1, 128)
@@ -193,8 +224,8 @@ def test_masked_prefill_without_room_for_the_mask_summary(device):
     cache.partition_tokens = 1024  # one partition per sequence: the partials need no workspace
     cache.update_cache(k.to(device), v.to(device), 2)
     with_summary = cache.attend(q.to(device), m.to(device))
-    plan = cache._plan
-    cache._plan = lambda *a: plan(*a)[:4] + (0,)  # same cut, no workspace
+    plan = cache.state.plan_attention
+    cache.state.plan_attention = lambda *a: plan(*a)[:4] + (0,)  # same cut, no workspace
     without = cache.attend(q.to(device), m.to(device))
     assert_attention_close(with_summary, ref, "with the summary")
     assert_attention_close(without, ref, "without the summary")

@@ -2,6 +2,8 @@
 contiguous caches vs the oracle, block allocator and eviction / compaction plans."""
 import re
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -294,43 +296,103 @@ def test_compaction_moves_a_shared_block_once():
     assert sorted(st.allocator.free_ids().tolist()) == list(range(6, 30))
 
 
-# ---- attention launch planning ----
-def test_plan_attention_uniform_batch_uses_dense_grid():
-    st = _state(batch=4, max_len=8192, blocks=4 * 512)
-    items, parts, max_parts = st.plan_attention(np.full(4, 4097), 4224, 8192, 64)
-    assert items is None and parts is None and max_parts == 1
-    items, parts, max_parts = st.plan_attention(np.full(4, 4097), 1024, 8192, 64)
-    assert items is None and parts is None and max_parts == 5
+# ---- attention launch planning (the library's host-side planner; no GPU involved) ----
+def _planned(st, lens, hq=32, hkv=8, dim=128, q_len=1, masked=False, partition=0):
+    lens = np.asarray(lens, dtype=np.int64)
+    st.ensure_capacity(lens)
+    items, parts, n, max_parts, ws = st.plan_attention(lens, hq, hkv, dim, q_len, masked, partition)
+    it = items.numpy().reshape(-1, 16)
+    assert it.shape[0] == n
+    return it, parts.numpy(), max_parts, ws
+
+
+def _check_cover(it, parts, lens, table):
+    """Every sequence is cut into its partitions exactly once: contiguous ranges of whole 32-token units from
+    token 0, the last one open ended; the unit entries name the table's blocks."""
+    lens = np.asarray(lens)
+    assert sorted(map(tuple, it[:, :2].tolist())) == sorted((b, p) for b in range(len(lens)) for p in range(parts[b]))
+    for b in range(len(lens)):
+        rows = it[it[:, 0] == b]
+        rows = rows[np.argsort(rows[:, 1])]
+        assert (rows[:, 2] == parts[b]).all()
+        assert rows[0, 3] == 0 and (rows[:, 3] % 32 == 0).all()
+        assert (rows[:-1, 4] == rows[1:, 3]).all() and rows[-1, 4] == -1
+        assert (rows[:, 3] < max(lens[b], 1)).all(), "no partition may be empty"
+        for r in rows:
+            end = lens[b] if r[4] < 0 else r[4]
+            whole = min(4, max(0, (end - r[3]) // 32))
+            assert r[5] == whole
+            for u in range(4):
+                j = r[3] // 16 + 2 * u
+                want = table[b, j:j + 2].tolist() if u < whole else [0, 0]
+                assert r[8 + 2 * u: 10 + 2 * u].tolist() == want
+
+
+def test_plan_attention_uniform_batch_is_cut_evenly_in_table_order():
+    st = _state(batch=4, max_len=8192, blocks=4 * 520)
+    lens = np.full(4, 4097)
+    it, parts, max_parts, ws = _planned(st, lens)
+    _check_cover(it, parts, lens, st.table)
+    assert (parts == parts[0]).all() and max_parts == parts[0] > 1          # 32 (sequence, head) pairs do not fill the GPU
+    assert it[:, 0].tolist() == sorted(it[:, 0].tolist()), "a uniform batch is scheduled as it comes"
+    assert ws == 4 * 32 * 1 * max_parts * (128 + 2) * 4
+    it, parts, max_parts, ws = _planned(st, lens, partition=4224)
+    assert parts.tolist() == [1, 1, 1, 1] and max_parts == 1 and ws == 0
+    assert it[:, 3].tolist() == [0] * 4 and it[:, 4].tolist() == [-1] * 4 and it[:, 5].tolist() == [4] * 4
 
 
 def test_plan_attention_multi_round_batch_is_cut_and_sorted_longest_first():
-    st = _state(batch=6, max_len=20000, blocks=10)
+    st = _state(batch=6, max_len=20000, blocks=2200)
     lens = np.array([100, 5000, 16385, 300, 2000, 9000])
-    items, parts, max_parts = st.plan_attention(lens, 2048, 8192, slots=8)  # 8 slots < 18 partitions: several rounds
-    assert parts is None and max_parts == 9
-    it = items.numpy()
-    n = np.maximum(1, -(-lens // 2048))
-    assert len(it) == n.sum()
-    assert sorted(map(tuple, it.tolist())) == sorted((b, p) for b in range(6) for p in range(n[b]))
-    sizes = (lens / n)[it[:, 0]]
+    it, parts, max_parts, _ = _planned(st, lens, hq=64, hkv=64, partition=2048)   # 64 heads: 8 slots per head < 18 partitions
+    _check_cover(it, parts, lens, st.table)
+    assert parts.tolist() == np.maximum(1, -(-lens // 2048)).tolist() and max_parts == 9
+    sizes = (lens / parts)[it[:, 0]]
     assert (np.diff(sizes) <= 1e-9).all(), "longest partitions first"
-    again, _, _ = st.plan_attention(lens + 1, 2048, 8192, slots=8)  # same partition counts: cached list
-    assert again is items
 
 
 def test_plan_attention_single_round_batch_gets_even_partitions():
-    st = _state(batch=5, max_len=9000, blocks=10)
+    st = _state(batch=5, max_len=9000, blocks=1500)
     lens = np.array([1024, 8192, 4000, 2500, 6000])
-    items, parts, max_parts = st.plan_attention(lens, 4736, 6144, slots=16)
-    n = parts.numpy()
-    assert n.sum() == 16 and max_parts == n.max()
-    assert (lens / n).max() <= 1.6 * lens.sum() / 16
-    assert ((lens / n) <= 6144).all() and (n >= 1).all()
-    it = items.numpy()
-    assert sorted(map(tuple, it.tolist())) == sorted((b, p) for b in range(5) for p in range(n[b]))
-    # never splits below 256 tokens per partition
-    _, parts, _ = st.plan_attention(np.array([300, 700]), 4736, 6144, slots=64)
-    assert parts.numpy().tolist() == [1, 2]
+    it, parts, max_parts, _ = _planned(st, lens, hq=32, hkv=32)                    # 32 heads: 16 slots per head
+    _check_cover(it, parts, lens, st.table)
+    assert parts.sum() == 16 and max_parts == parts.max()
+    assert (lens / parts).max() <= 1.6 * lens.sum() / 16
+    st2 = _state(batch=2, max_len=1024, blocks=128)
+    _, parts, _, _ = _planned(st2, [300, 700], hq=8, hkv=8)                        # never below 256 tokens per partition
+    assert parts.tolist() == [1, 2]
+
+
+def test_plan_attention_keeps_a_plan_while_lengths_stay_in_their_buckets_and_the_table_is_unchanged():
+    st = _state(batch=3, max_len=4096, blocks=800)
+    lens = np.array([1000, 3000, 130], dtype=np.int64)
+    st.ensure_capacity(lens + 200)
+    first = st.plan_attention(lens, 32, 8, 128, 1, False, 0)
+    assert st.plan_attention(lens + 5, 32, 8, 128, 1, False, 0)[0] is first[0]      # same 64-token buckets
+    assert st.plan_attention(lens + 64, 32, 8, 128, 1, False, 0)[0] is not first[0]
+    again = st.plan_attention(lens, 32, 8, 128, 1, False, 0)
+    st.evict(1, [3], lens)                                                           # a table entry below the lengths moved
+    lens2 = lens.copy(); lens2[1] -= 16
+    moved = st.plan_attention(lens, 32, 8, 128, 1, False, 0)
+    assert moved[0] is not again[0]
+    it = moved[0].numpy().reshape(-1, 16)
+    rows = it[(it[:, 0] == 1) & (it[:, 3] == 0)]
+    assert rows[0, 8:16].tolist() == st.table[1, :8].tolist()
+
+
+def test_plan_attention_accepts_partitions_of_any_length_and_reports_a_short_capacity():
+    from pace_mi355 import _native as nat
+
+    st = _state(batch=1, max_len=40000, blocks=2600)
+    it, parts, max_parts, ws = _planned(st, [40000], partition=65536)               # one partition of 1250 units
+    assert parts.tolist() == [1] and max_parts == 1 and it[0, 3:6].tolist() == [0, -1, 4]
+    lens = np.array([40000], dtype=np.int32)
+    plan = nat.AttnPlan()
+    out = np.zeros((2, 16), dtype=np.int32)
+    sp = np.zeros(1, dtype=np.int32)
+    rc = nat.load().pace_paged_attn_plan(lens.ctypes.data, st.table.ctypes.data, st.table.shape[1], 1, 32, 8, 128, 1, 0, 1024,
+                                         out.ctypes.data, 2, sp.ctypes.data, ctypes.byref(plan))
+    assert rc == -1 and b"do not fit the capacity" in nat.load().pace_kv_last_error() and plan.n_work_items == 40
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2, 3])
