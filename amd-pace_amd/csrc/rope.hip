@@ -78,6 +78,54 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const RopeRowsParams p) 
   store_kv_chunk<D>(kslab, vslab, off, cb, kb, vb);
 }
 
+// fp32 rows (the reference's operator on fp32 activations, pace/ops/rotary_embedding.py:412-443 with cos / sin
+// cast to fp32): one thread per (token, head, rotation pair or pass-through pair of dims).  Every product and
+// the sum are rounded separately, as the tensor operations round them -- no fused multiply-add.
+struct RopeF32Params {
+  const float* cos;
+  const float* sin;
+  int32_t rows, rot, interleaved;
+  const int32_t* positions;
+  int32_t pos_sb;
+  const float* x[2];
+  float* out[2];
+  int64_t sb[2], sh[2], st[2];
+  int32_t heads[2];
+  int32_t T, D;
+  int64_t total;  // batch * T * (heads[0] + heads[1]) * D/2
+};
+
+__global__ __launch_bounds__(256) void rope_rows_f32_kernel(const RopeF32Params p) {
+#pragma clang fp contract(off)
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= p.total) return;
+  const int half_d = p.D / 2;
+  const int i = (int)(gid % half_d);
+  const int64_t row = gid / half_d;
+  const int heads = p.heads[0] + p.heads[1];
+  const int hh = (int)(row % heads);
+  const int64_t bt = row / heads;
+  const int b = (int)(bt / p.T), t = (int)(bt % p.T);
+  const int which = hh < p.heads[0] ? 0 : 1, h = which ? hh - p.heads[0] : hh;
+  const int64_t base = (int64_t)b * p.sb[which] + (int64_t)h * p.sh[which] + (int64_t)t * p.st[which];
+  const float* x = p.x[which] + base;
+  float* o = p.out[which] + base;
+  const int half_r = p.rot / 2;
+  if (i >= half_r) {  // the dims past rotary_dim pass through, two per thread
+    const int d = p.rot + 2 * (i - half_r);
+    o[d] = x[d], o[d + 1] = x[d + 1];
+    return;
+  }
+  int pos = p.positions[(int64_t)b * p.pos_sb + t];
+  pos = pos < 0 ? 0 : (pos >= p.rows ? p.rows - 1 : pos);
+  const float c = p.cos[(int64_t)pos * half_r + i], sn = p.sin[(int64_t)pos * half_r + i];
+  const int d1 = p.interleaved ? 2 * i : i, d2 = p.interleaved ? 2 * i + 1 : i + half_r;
+  const float x1 = x[d1], x2 = x[d2];
+  const float a = x1 * c, bq = x2 * sn, cq = x2 * c, dq = x1 * sn;
+  o[d1] = a - bq;
+  o[d2] = cq + dq;
+}
+
 int make_rope_dev(const pace_rope_t* rope, int head_dim, bool need_positions, const char* who, RopeDev* out) {
   PACE_REQUIRE(rope != nullptr, "%s: rope is NULL", who);
   PACE_REQUIRE(rope->cos && rope->sin, "%s: NULL cos / sin table", who);
@@ -183,4 +231,41 @@ extern "C" int pace_rope_append_paged(const pace_kv_pool_t* pool, const pace_rop
   p.k_sb = stride_b, p.k_sh = stride_h, p.k_st = stride_t, p.Hk = pool->num_kv_heads;
   p.pool = *pool, p.to_pool = 1;
   return launch_rows(p, pool->head_dim, batch, stream, who);
+}
+
+extern "C" int pace_rope_apply_f32(const pace_rope_t* rope, const void* q, void* q_out, int64_t q_stride_b, int64_t q_stride_h,
+                                   int64_t q_stride_t, int32_t num_q_heads, const void* k, void* k_out, int64_t k_stride_b,
+                                   int64_t k_stride_h, int64_t k_stride_t, int32_t num_k_heads, int32_t batch, int32_t n_tokens,
+                                   int32_t head_dim, void* stream) {
+  const char* who = "pace_rope_apply_f32";
+  PACE_REQUIRE(rope != nullptr && rope->cos && rope->sin && rope->positions, "%s: NULL rope, table or positions", who);
+  PACE_REQUIRE(rope->table_dtype == PACE_DTYPE_F32, "%s: fp32 rows take fp32 tables", who);
+  PACE_REQUIRE(head_dim >= 2 && head_dim % 2 == 0, "%s: head_dim %d must be even", who, head_dim);
+  PACE_REQUIRE(rope->rotary_dim >= 2 && rope->rotary_dim % 2 == 0 && rope->rotary_dim <= head_dim,
+               "%s: rotary_dim %d must be even and at most head_dim %d", who, rope->rotary_dim, head_dim);
+  PACE_REQUIRE(rope->table_rows >= 1 && rope->pos_stride_b >= 0, "%s: bad table_rows (%d) or pos_stride_b (%d)", who, rope->table_rows,
+               rope->pos_stride_b);
+  PACE_REQUIRE(rope->interleaved == 0 || rope->interleaved == 1, "%s: interleaved must be 0 or 1", who);
+  PACE_REQUIRE(batch >= 0 && n_tokens >= 0, "%s: negative batch (%d) or n_tokens (%d)", who, batch, n_tokens);
+  RopeF32Params p = {};
+  p.cos = static_cast<const float*>(rope->cos), p.sin = static_cast<const float*>(rope->sin);
+  p.rows = rope->table_rows, p.rot = rope->rotary_dim, p.interleaved = rope->interleaved;
+  p.positions = rope->positions, p.pos_sb = rope->pos_stride_b;
+  if (q) {
+    PACE_REQUIRE(q_out != nullptr && num_q_heads >= 1, "%s: q has no output pointer or no heads", who);
+    p.x[0] = static_cast<const float*>(q), p.out[0] = static_cast<float*>(q_out);
+    p.sb[0] = q_stride_b, p.sh[0] = q_stride_h, p.st[0] = q_stride_t, p.heads[0] = num_q_heads;
+  }
+  if (k) {
+    PACE_REQUIRE(k_out != nullptr && num_k_heads >= 1, "%s: k has no output pointer or no heads", who);
+    p.x[1] = static_cast<const float*>(k), p.out[1] = static_cast<float*>(k_out);
+    p.sb[1] = k_stride_b, p.sh[1] = k_stride_h, p.st[1] = k_stride_t, p.heads[1] = num_k_heads;
+  }
+  p.T = n_tokens, p.D = head_dim;
+  p.total = (int64_t)batch * n_tokens * (p.heads[0] + p.heads[1]) * (head_dim / 2);
+  if (p.total == 0) return PACE_KV_OK;
+  PACE_REQUIRE((p.total + 255) / 256 < (int64_t)1 << 31, "%s: grid too large", who);
+  hipLaunchKernelGGL(rope_rows_f32_kernel, dim3((unsigned)((p.total + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
 }

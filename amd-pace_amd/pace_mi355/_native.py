@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "pace_kv_gather_packed",
     "pace_kv_copy_blocks",
     "pace_rope_apply",
+    "pace_rope_apply_f32",
     "pace_rope_append_paged",
     "pace_paged_attn_partition_tokens",
     "pace_paged_attn_plan",
@@ -183,6 +184,8 @@ def load() -> ctypes.CDLL:
     rows = [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32]  # in, out, strides b/h/t, heads
     lib.pace_rope_apply.restype = ctypes.c_int
     lib.pace_rope_apply.argtypes = [R] + rows + rows + [c_int32, c_int32, c_int32, c_void_p]
+    lib.pace_rope_apply_f32.restype = ctypes.c_int
+    lib.pace_rope_apply_f32.argtypes = [R] + rows + rows + [c_int32, c_int32, c_int32, c_void_p]
     lib.pace_rope_append_paged.restype = ctypes.c_int
     lib.pace_rope_append_paged.argtypes = (
         [P, R] + rows + [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32]

@@ -261,8 +261,8 @@ class PagedKVCache(KVCacheBase):
     def _append(self, k: torch.Tensor, v: torch.Tensor, counts: Optional[np.ndarray], rope=None,
                 right_aligned: bool = False) -> None:
         B, h_in, T, D = k.shape
-        if rope is not None and (counts is not None or tuple(rope.rows.shape) != (B, T)):
-            raise RuntimeError("rope rows must be [B, T] and cannot be combined with per-sequence counts")
+        if rope is not None and (counts is not None or tuple(rope.rows.shape) not in ((B, T), (1, T))):
+            raise RuntimeError("rope rows must be [B, T] (or [1, T]) and cannot be combined with per-sequence counts")
         if B != self.batch or D != self.model_dim or h_in % self.num_kv_heads:
             raise RuntimeError(f"update of shape {tuple(k.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={D}]")
         if v.shape != k.shape:
@@ -484,7 +484,7 @@ class PagedKVCache(KVCacheBase):
         rope, self._query_rope = self._query_rope, None
         rope_desc = None
         if rope is not None:
-            if tuple(rope.rows.shape) != (B, S):
+            if tuple(rope.rows.shape) not in ((B, S), (1, S)):
                 raise RuntimeError(f"rope rows {tuple(rope.rows.shape)} do not match the query [B={B}, S={S}]")
             rope_desc = rope.desc()
             if attention_mask is not None or rope_desc.rotary_dim != D or D % 64:

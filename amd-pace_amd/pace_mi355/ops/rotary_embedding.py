@@ -12,8 +12,9 @@ rotation can run
                                                                      -> ``pace_rope_append_paged``
   * folded into the attention launch together with the append (decode / verify steps).
 
-bf16 device tensors with head_dim 64, 96, 128 or 256 only; anything else raises (there is
-no second implementation).
+Device tensors only (there is no second implementation): bf16 with head_dim 64, 96, 128 or 256 and
+a rotary_dim that is a multiple of 16, or fp32 with any even head_dim / rotary_dim (dense form only);
+``[B, H, S, D]`` (``unsqueeze_dim=1``) or ``[B, S, H, D]`` (``unsqueeze_dim=2``).
 """
 from __future__ import annotations
 
@@ -79,38 +80,55 @@ _TABLE_BUILDERS: Dict[str, Callable] = {
 
 
 def _check_rows(x: torch.Tensor, name: str) -> None:
-    if not x.is_cuda or x.dtype != torch.bfloat16 or x.dim() != 4:
-        raise NotImplementedError(f"rotary embedding runs on bf16 device tensors [B, H, S, D]; {name} is "
+    if not x.is_cuda or x.dtype not in (torch.bfloat16, torch.float32) or x.dim() != 4:
+        raise NotImplementedError(f"rotary embedding runs on bf16 / fp32 device tensors of four dims; {name} is "
                                   f"{x.dtype} {tuple(x.shape)} on {x.device}")
-    if x.shape[-1] not in (64, 96, 128, 256):
-        raise NotImplementedError(f"rotary embedding supports head_dim 64, 96, 128 or 256, got {x.shape[-1]}")
+    if x.dtype == torch.bfloat16 and x.shape[-1] not in (64, 96, 128, 256):
+        raise NotImplementedError(f"rotary embedding on bf16 supports head_dim 64, 96, 128 or 256, got {x.shape[-1]}")
+    if x.shape[-1] % 2:
+        raise NotImplementedError(f"rotary embedding needs an even head_dim, got {x.shape[-1]}")
 
 
 def _strided(x: torch.Tensor) -> torch.Tensor:
+    step = 8 if x.dtype == torch.bfloat16 else 1  # bf16 rows move in 16-byte chunks
     ok = x.stride(3) == 1 and x.data_ptr() % 16 == 0 and all(
-        s % 8 == 0 and (s > 0 or n == 1) for s, n in zip(x.stride()[:3], x.shape[:3]))
+        s % step == 0 and (s > 0 or n == 1) for s, n in zip(x.stride()[:3], x.shape[:3]))
     return x if ok else x.contiguous()
 
 
-def launch_rope_apply(desc: nat.RopeDesc, query: Optional[torch.Tensor], key: Optional[torch.Tensor]):
-    """Rotate dense ``query`` / ``key`` [B, H, S, D] into new tensors with ``pace_rope_apply``."""
+def launch_rope_apply(desc: nat.RopeDesc, query: Optional[torch.Tensor], key: Optional[torch.Tensor],
+                      unsqueeze_dim: int = 1, rows_shape: Optional[Tuple[int, int]] = None):
+    """Rotate dense ``query`` / ``key`` into new tensors with ``pace_rope_apply`` (bf16) or
+    ``pace_rope_apply_f32``.  ``unsqueeze_dim`` names the head axis as the reference does
+    (``pace/ops/rotary_embedding.py:418-419``): 1 for ``[B, H, S, D]``, 2 for ``[B, S, H, D]``.
+    ``rows_shape``: shape of the position rows behind ``desc``; ``(1, S)`` rows serve every sequence,
+    as the reference's broadcast of ``cos.unsqueeze(1)`` does."""
+    if unsqueeze_dim not in (1, 2):
+        raise NotImplementedError(f"rotary embedding takes [B, H, S, D] (unsqueeze_dim=1) or [B, S, H, D] (2), not {unsqueeze_dim}")
+    t_ax, h_ax = (2, 1) if unsqueeze_dim == 1 else (1, 2)
     outs = []
     args = []
     ref = query if query is not None else key
-    B, _, S, D = ref.shape
+    B, S, D = ref.shape[0], ref.shape[t_ax], ref.shape[3]
+    if rows_shape is not None:
+        if tuple(rows_shape) not in ((B, S), (1, S)):
+            raise RuntimeError(f"position rows {tuple(rows_shape)} fit neither [B={B}, S={S}] nor [1, S={S}]")
+        if rows_shape[0] == 1:
+            desc.pos_stride_b = 0
     for x, name in ((query, "query"), (key, "key")):
         if x is None:
             outs.append(None)
             args += [None, None, 0, 0, 0, 0]
             continue
         _check_rows(x, name)
-        if x.shape[0] != B or x.shape[2] != S or x.shape[3] != D:
-            raise RuntimeError(f"query / key disagree: {tuple(query.shape)} vs {tuple(key.shape)}")
+        if x.shape[0] != B or x.shape[t_ax] != S or x.shape[3] != D or x.dtype != ref.dtype:
+            raise RuntimeError(f"query / key disagree: {tuple(query.shape)} {query.dtype} vs {tuple(key.shape)} {key.dtype}")
         xin = _strided(x)
         out = torch.empty_strided(xin.shape, xin.stride(), dtype=xin.dtype, device=xin.device) if xin is x else xin
         outs.append(out)
-        args += [xin.data_ptr(), out.data_ptr(), xin.stride(0), xin.stride(1), xin.stride(2), xin.shape[1]]
-    nat.check(nat.load().pace_rope_apply(ctypes.byref(desc), *args, B, S, D, nat.current_stream_ptr()))
+        args += [xin.data_ptr(), out.data_ptr(), xin.stride(0), xin.stride(h_ax), xin.stride(t_ax), xin.shape[h_ax]]
+    fn = nat.load().pace_rope_apply if ref.dtype == torch.bfloat16 else nat.load().pace_rope_apply_f32
+    nat.check(fn(ctypes.byref(desc), *args, B, S, D, nat.current_stream_ptr()))
     return outs[0], outs[1]
 
 
@@ -124,18 +142,21 @@ class RopeCall:
 
     def __init__(self, module: "RotaryEmbedding", rows: torch.Tensor):
         self.module = module
-        self.rows = rows  # int32 [B, S] table rows, on the device
+        self.rows = rows  # int32 [B, S] (or [1, S]) table rows, on the device
         self.is_neox_style = True
 
-    def desc(self, is_neox_style: Optional[bool] = None) -> nat.RopeDesc:
+    def desc(self, is_neox_style: Optional[bool] = None, dtype: torch.dtype = torch.bfloat16) -> nat.RopeDesc:
         neox = self.is_neox_style if is_neox_style is None else is_neox_style
-        cos, sin = self.module.device_tables(self.rows.device)
+        if self.module.rope_type == "longrope":
+            neox = True  # the reference's longrope branch always pairs dim i with i + rotary_dim / 2 (:421-430)
+        cos, sin = self.module.device_tables(self.rows.device, dtype)
         d = nat.RopeDesc()
         d.cos, d.sin = cos.data_ptr(), sin.data_ptr()
-        d.table_dtype = nat.DTYPE_BF16
+        d.table_dtype = nat.DTYPE_BF16 if dtype == torch.bfloat16 else nat.DTYPE_F32
         d.table_rows, d.rotary_dim = cos.shape[0], 2 * cos.shape[1]
         d.interleaved = 0 if neox else 1
-        d.positions, d.pos_stride_b = self.rows.data_ptr(), self.rows.stride(0)
+        d.positions = self.rows.data_ptr()
+        d.pos_stride_b = 0 if self.rows.shape[0] == 1 else self.rows.stride(0)
         return d
 
     def with_style(self, is_neox_style: bool) -> "RopeCall":
@@ -143,8 +164,9 @@ class RopeCall:
         other.is_neox_style = bool(is_neox_style)
         return other
 
-    def __call__(self, query: torch.Tensor, key: torch.Tensor, is_neox_style: Optional[bool] = None):
-        return launch_rope_apply(self.desc(is_neox_style), query, key)
+    def __call__(self, query: torch.Tensor, key: torch.Tensor, is_neox_style: Optional[bool] = None, unsqueeze_dim: int = 1):
+        ref = query if query is not None else key
+        return launch_rope_apply(self.desc(is_neox_style, ref.dtype), query, key, unsqueeze_dim, tuple(self.rows.shape))
 
 
 class RotaryEmbedding(OperatorBase):
@@ -196,13 +218,13 @@ class RotaryEmbedding(OperatorBase):
         long_ = _table(_frequencies(self.rope_theta, self.rotary_dim, cfg["long_factor"]), rows, amp)
         return torch.cat([short[0], long_[0]], dim=0), torch.cat([short[1], long_[1]], dim=0)
 
-    def device_tables(self, device) -> Tuple[torch.Tensor, torch.Tensor]:
-        """bf16 copies of the tables on ``device`` (what ``.to(x.dtype)`` yields for bf16 activations)."""
-        key = str(device)
+    def device_tables(self, device, dtype: torch.dtype = torch.bfloat16) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Copies of the tables on ``device`` in the activations' dtype (the reference's ``.to(x.dtype)``, ``:398-399``)."""
+        key = (str(device), dtype)
         if key not in self._device_tables:
             self._device_tables[key] = (
-                self.cos_cache.to(device=device, dtype=torch.bfloat16).contiguous(),
-                self.sin_cache.to(device=device, dtype=torch.bfloat16).contiguous(),
+                self.cos_cache.to(device=device, dtype=dtype).contiguous(),
+                self.sin_cache.to(device=device, dtype=dtype).contiguous(),
             )
         return self._device_tables[key]
 
@@ -219,7 +241,7 @@ class RotaryEmbedding(OperatorBase):
                 offsets: Optional[torch.Tensor] = None):
         rows = self.table_rows(position_ids, offsets)
         if return_cos_sin:
-            flat = rows.flatten()
+            flat = rows.flatten().to(self.cos_cache.device)
             cos = self.cos_cache.index_select(0, flat).unflatten(0, rows.shape).to(x.dtype)
             sin = self.sin_cache.index_select(0, flat).unflatten(0, rows.shape).to(x.dtype)
             return cos, sin
@@ -229,20 +251,22 @@ class RotaryEmbedding(OperatorBase):
 
     def apply_rotary_emb(self, query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                          unsqueeze_dim: int = 1, is_neox_style: bool = True):
-        """Rotate with gathered ``cos`` / ``sin`` [B, S, rotary_dim/2] (reference ``:445-474``)."""
-        if unsqueeze_dim != 1:
-            raise NotImplementedError("rotary embedding takes [B, H, S, D] tensors (unsqueeze_dim=1)")
-        _check_rows(query, "query")
-        B, S = cos.shape[0], cos.shape[1]
-        cos2 = cos.to(torch.bfloat16).reshape(B * S, -1).contiguous()
-        sin2 = sin.to(torch.bfloat16).reshape(B * S, -1).contiguous()
-        rows = torch.arange(B * S, dtype=torch.int32, device=query.device).view(B, S)
+        """Rotate with gathered ``cos`` / ``sin`` ``[B | 1, S, rotary_dim/2]`` (reference ``:445-474``)."""
+        ref = query if query is not None else key
+        _check_rows(ref, "query")
+        if cos.dim() != 3 or sin.shape != cos.shape:
+            raise RuntimeError(f"cos / sin must be [B, S, rotary_dim/2]; got {tuple(cos.shape)} and {tuple(sin.shape)}")
+        nb, S = cos.shape[0], cos.shape[1]
+        cos2 = cos.to(device=ref.device, dtype=ref.dtype).reshape(nb * S, -1).contiguous()
+        sin2 = sin.to(device=ref.device, dtype=ref.dtype).reshape(nb * S, -1).contiguous()
+        rows = torch.arange(nb * S, dtype=torch.int32, device=ref.device).view(nb, S)
         d = nat.RopeDesc()
-        d.cos, d.sin, d.table_dtype = cos2.data_ptr(), sin2.data_ptr(), nat.DTYPE_BF16
-        d.table_rows, d.rotary_dim = B * S, 2 * cos2.shape[1]
-        d.interleaved = 0 if is_neox_style else 1
+        d.cos, d.sin = cos2.data_ptr(), sin2.data_ptr()
+        d.table_dtype = nat.DTYPE_BF16 if ref.dtype == torch.bfloat16 else nat.DTYPE_F32
+        d.table_rows, d.rotary_dim = nb * S, 2 * cos2.shape[1]
+        d.interleaved = 0 if (is_neox_style or self.rope_type == "longrope") else 1  # longrope: always halves (:421-430)
         d.positions, d.pos_stride_b = rows.data_ptr(), rows.stride(0)
-        return launch_rope_apply(d, query, key)
+        return launch_rope_apply(d, query, key, unsqueeze_dim, (nb, S))
 
     def extra_repr(self) -> str:
         return (f"rope_type={self.rope_type}, rotary_dim={self.rotary_dim}, "

@@ -191,6 +191,17 @@ int pace_rope_apply(const pace_rope_t* rope, const void* q, void* q_out,
                     int32_t batch, int32_t n_tokens, int32_t head_dim, void* stream);
 
 /*
+ * The same operator on fp32 tensors (the reference's operator takes any float dtype and casts cos / sin to it,
+ * pace/ops/rotary_embedding.py:398-399): q / k / outputs fp32, rope->cos / sin fp32 tables, any even head_dim and
+ * rotary_dim.  Each product and the sum are rounded separately, as the tensor operations round them.
+ */
+int pace_rope_apply_f32(const pace_rope_t* rope, const void* q, void* q_out,
+                        int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t, int32_t num_q_heads,
+                        const void* k, void* k_out,
+                        int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_t, int32_t num_k_heads,
+                        int32_t batch, int32_t n_tokens, int32_t head_dim, void* stream);
+
+/*
  * Rotate-and-append in one launch: the rope(q, k) + update_cache(k, v) sequence of
  * pace/llm/models/llama.py:147-158.  q is rotated into q_out (may alias q; NULL q = keys
  * only); k_new is rotated and stored, v_new stored, at positions seq_lens[b] + pos_offset + t

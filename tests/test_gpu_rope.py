@@ -42,6 +42,63 @@ def test_dense_rope_is_bit_exact(device, D, neox, partial):
     assert_bits_equal(ko, _oracle_rotate(k, mod, pos, neox), "key")
 
 
+@pytest.mark.parametrize("D,neox,partial", [(128, True, 1.0), (80, False, 1.0), (64, True, 0.5), (20, True, 1.0), (256, False, 0.25)])
+def test_dense_rope_on_fp32_tensors_is_bit_exact(device, D, neox, partial):
+    """The reference's operator takes any float dtype (cos / sin are cast to it, :398-399); on fp32 every product
+    and the sum are separate fp32 roundings."""
+    B, Hq, Hk, S = 2, 4, 2, 11
+    mod = _module(D, partial_rotary_factor=partial)
+    g = torch.Generator().manual_seed(D)
+    pos = torch.randint(0, 512, (B, S), generator=g)
+    q, k = torch.randn(B, Hq, S, D, generator=g), torch.randn(B, Hk, S, D, generator=g)
+    rope = mod(q.to(device), pos.to(device))
+    qo, ko = rope(q.to(device), k.to(device), is_neox_style=neox)
+    assert qo.dtype == torch.float32
+    assert torch.equal(qo.cpu(), _oracle_rotate(q, mod, pos, neox)), "query"
+    assert torch.equal(ko.cpu(), _oracle_rotate(k, mod, pos, neox)), "key"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rope_on_token_major_tensors_and_with_one_row_of_positions(device, dtype):
+    """unsqueeze_dim=2 rotates [B, S, H, D] tensors (:418-419); position ids / cos of batch 1 serve every sequence,
+    as cos.unsqueeze(1) broadcasts in the reference."""
+    B, H, S, D = 3, 4, 7, 128
+    mod = _module(D)
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, S, H, D, generator=g).to(dtype)
+    k = torch.randn(B, S, 2, D, generator=g).to(dtype)
+    pos = torch.arange(40, 40 + S).view(1, S)
+    want_q = _oracle_rotate(q.transpose(1, 2), mod, pos.expand(B, S), True).transpose(1, 2)
+    want_k = _oracle_rotate(k.transpose(1, 2), mod, pos.expand(B, S), True).transpose(1, 2)
+    cos, sin = mod(q.to(device), pos.to(device), return_cos_sin=True)
+    assert cos.shape[0] == 1
+    qo, ko = mod.apply_rotary_emb(q.to(device), k.to(device), cos, sin, unsqueeze_dim=2)
+    assert torch.equal(qo.cpu(), want_q) and torch.equal(ko.cpu(), want_k)
+    rope = mod(q.to(device), pos.to(device))            # [1, S] rows kept by the callable as well
+    qo2, _ = rope(q.to(device), None, unsqueeze_dim=2)
+    assert torch.equal(qo2.cpu(), want_q)
+    qo3, _ = rope(q.to(device).transpose(1, 2), None)   # the same rows as [B, H, S, D]
+    assert torch.equal(qo3.cpu(), want_q.transpose(1, 2))
+    with pytest.raises(RuntimeError, match="position rows"):
+        mod(q.to(device), torch.zeros(2, S, dtype=torch.long, device=device))(q.to(device).transpose(1, 2), None)
+
+
+def test_longrope_always_pairs_halves(device):
+    """The reference's longrope branch never looks at is_neox_style (:421-430)."""
+    D, S = 128, 9
+    cfg = dict(rope_type="longrope", short_factor=[1.0 + 0.01 * i for i in range(D // 2)],
+               long_factor=[2.0 + 0.02 * i for i in range(D // 2)])
+    mod = _module(D, rows=256, scaling=cfg, original_max_position_embeddings=128)
+    q = seeded_q(8, 2, 4, S, D)
+    pos = torch.arange(S).repeat(2, 1)
+    rope = mod(q.to(device), pos.to(device))
+    a, _ = rope(q.to(device), None, is_neox_style=False)
+    b, _ = rope(q.to(device), None, is_neox_style=True)
+    assert_bits_equal(a, b, "is_neox_style ignored")
+    cos, sin = rope_ref.lookup(mod.cos_cache, mod.sin_cache, rope_ref.longrope_rows(pos, 128), q.dtype)
+    assert_bits_equal(a, rope_ref.rotate_longrope_form(q, cos, sin, D), "longrope form")
+
+
 def test_dense_rope_takes_transposed_views_and_leaves_inputs_alone(device):
     """The models hand in [B, S, H, D] projections viewed as [B, H, S, D] (llama.py:125-138)."""
     B, H, S, D = 2, 4, 9, 128

@@ -62,5 +62,5 @@ def test_cpu_activations_are_refused():
     with pytest.raises(NotImplementedError, match="runs on the GPU"):
         mod(x, torch.tensor([[0, 1, 2]]))
     cos, sin = mod(x, torch.tensor([[0, 1, 2]]), return_cos_sin=True)
-    with pytest.raises(NotImplementedError, match="bf16 device tensors"):
+    with pytest.raises(NotImplementedError, match="device tensors"):
         mod.apply_rotary_emb(x, x, cos, sin)
