@@ -151,6 +151,7 @@ class PagedKVCache(KVCacheBase):
         self.fuse_append = True
         self._pending: Optional[Tuple[torch.Tensor, torch.Tensor, int, object]] = None
         self._query_rope = None
+        self._graph = None  # a DecodeGraph that has captured this cache's decode step
         self.cow_blocks_copied = 0  # blocks copied on write after forks (per layer pool)
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
@@ -277,6 +278,15 @@ class PagedKVCache(KVCacheBase):
         st = self.state
         lib = nat.load()
         stream = nat.current_stream_ptr()
+        if self._graph is not None and counts is None and self.fuse_append and T <= 32 and self._pending is None:
+            # a step of a decode graph: blocks and table were prepared for every step; the append rides in the
+            # attention launch, and the lengths advance on the device
+            self._graph.reserve(T)
+            self._pending = (k, v, head_step, rope)
+            self._query_rope = rope
+            self.lens = self.lens + T
+            self.seq_len += T
+            return
         self._flush()
         if st.tails_dirty:
             self._unshare()
@@ -328,7 +338,10 @@ class PagedKVCache(KVCacheBase):
         )
 
     def _flush(self) -> None:
-        """Store a held-back append into the pool now."""
+        """Store a held-back append into the pool now.  Every operation other than a captured decode step
+        comes through here first, which ends a decode graph (its frozen plan and lengths no longer hold)."""
+        if self._graph is not None:
+            self._graph.close()
         if self._pending is not None:
             k, v, head_step, rope = self._pending
             self._pending = None
@@ -496,12 +509,24 @@ class PagedKVCache(KVCacheBase):
         st = self.state
         max_len = self.seq_len
         lib = nat.load()
-        items, parts, n_items, max_parts, ws_bytes = st.plan_attention(
-            self.lens, hq, self.num_kv_heads, self.head_dim, S, attention_mask is not None, self.partition_tokens)
-        ws = st.workspace(ws_bytes)
-        table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
+        graph = self._graph
+        if graph is not None and self._pending is None:
+            graph.close()  # attention without the step's append is not the captured step
+            graph = None
+        plan = lambda: st.plan_attention(self.lens, hq, self.num_kv_heads, self.head_dim, S, attention_mask is not None,
+                                         self.partition_tokens)
         a = nat.PagedAttnArgs()
-        a.seq_len_bias = bias
+        if graph is None:
+            items, parts, n_items, max_parts, ws_bytes = plan()
+            table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
+            a.seq_len_bias = bias
+        else:
+            # captured step: the plan and the table are frozen, the lengths are base + new tokens + the device counter
+            items, parts, n_items, max_parts, ws_bytes = graph.plan((hq, S, attention_mask is not None), plan)
+            table, lens_dev = graph.table, graph.lens_dev
+            a.seq_len_bias, a.seq_len_bias_ptr = graph.new_tokens, graph.counter.data_ptr()
+            max_len = int(graph.base.max()) + graph.new_tokens * graph.max_steps
+        ws = st.workspace(ws_bytes)
         a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = query.data_ptr(), query.stride(0), query.stride(1), query.stride(2)
         a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
         a.block_table, a.table_stride = table.data_ptr(), table.stride(0)
@@ -589,3 +614,13 @@ class KVCacheManager:
     def remove_cache(self, remove_len: int) -> None:
         for cache_object in self.cache_objects:
             cache_object.remove_cache(remove_len)
+
+    def capture_decode(self, step_fn, max_steps: int):
+        """Capture one decode step over every layer into a HIP graph (paged caches only): see
+        ``pace_mi355.llm.graph.DecodeGraph``.  ``step_fn`` runs the step on static tensors; the returned
+        object's ``replay()`` runs it again for the next token."""
+        if self.kv_cache_class is not PagedKVCache:
+            raise RuntimeError("only the paged cache keeps its lengths on the device; capture_decode needs KVCacheType.PAGED")
+        from .graph import DecodeGraph
+
+        return DecodeGraph(list(self.cache_objects), step_fn, max_steps)

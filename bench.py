@@ -288,6 +288,9 @@ def wl_decode_gptj(torch, dev, args):
 
 def _wl_decode(torch, dev, args, shape, label, has_traffic_profile, with_cpu):
     B, ctx, hq, hkv, D = shape
+    if args.batch or args.context:
+        B, ctx = args.batch or B, args.context or ctx
+        label = f"{label} -- with batch {B} and context {ctx} instead"
     # One pool per layer, each with its own seeded block permutation: step i runs on pool i mod N, as a
     # decoder walks its layers (pace/llm/models/llama.py:312-315), so no step finds the K / V of the step
     # before it in the 256 MB last-level cache.
@@ -322,6 +325,30 @@ def _wl_decode(torch, dev, args, shape, label, has_traffic_profile, with_cpu):
             mha(q, pk, pv, attention_mask=mask_all[..., : c.seq_len] if args.mask else None)
             if ev:
                 ev[1].record()
+    elif args.path == "graph":
+        from pace_mi355.llm.graph import DecodeGraph
+        from pace_mi355.ops import MultiHeadAttention
+
+        # the same calls as --path api, captured once per layer pool into a HIP graph and replayed per step
+        mha = MultiHeadAttention(dtype=torch.bfloat16)
+        outs = {}
+
+        def one(c):
+            def fn():
+                pk, pv = c.update_cache(k1, v1, 2)
+                return mha(q, pk, pv)
+            return fn
+        graphs = [DecodeGraph([c], one(c), -(-(args.steps + args.warmup) // n_layers) + 1) for c in caches]
+        keep.append(graphs)
+
+        def step(ev=None):
+            gr = graphs[turn[0] % n_layers]
+            turn[0] += 1
+            if ev:
+                ev[0].record()
+            gr.replay()
+            if ev:
+                ev[1].record()
     else:
         rope = None
         if args.rope:  # q and k arrive un-rotated; llama-3 tables as RotaryEmbedding builds them
@@ -341,10 +368,10 @@ def _wl_decode(torch, dev, args, shape, label, has_traffic_profile, with_cpu):
             turn[0] += 1
             f(ev)
     dt, attn_ms = run_timed(torch, step, args.steps, args.warmup)
-    if args.path == "api":  # average context over the timed steps (each layer's cache grows once every n_layers steps)
+    if args.path in ("api", "graph"):  # average context over the timed steps (each layer's cache grows once every n_layers steps)
         ctx = ctx + (args.warmup + (args.steps - 1) // 2) // n_layers
     dec = decode_bytes([ctx + 1] * B, hq, hkv, D)
-    fused = args.path == "direct" and not args.no_fuse or args.path == "api"
+    fused = args.path == "direct" and not args.no_fuse or args.path in ("api", "graph")
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
     kernel = fixed[0].kernel if args.path == "direct" else "pace_kv::paged_attn_kernel (through PagedKVCache / MultiHeadAttention)"
     traffic = measured_traffic(kernel) if has_traffic_profile else None
@@ -711,9 +738,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="decode-8b")
-    ap.add_argument("--path", choices=("api", "direct"), default="direct",
-                    help="decode-8b only. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
-                         "MultiHeadAttention")
+    ap.add_argument("--path", choices=("api", "direct", "graph"), default="direct",
+                    help="decode workloads. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
+                         "MultiHeadAttention; graph: the api calls captured once into a HIP graph and replayed per step")
+    ap.add_argument("--batch", type=int, default=0, help="decode workloads: override the batch size (latency studies)")
+    ap.add_argument("--context", type=int, default=0, help="decode workloads: override the context length")
     ap.add_argument("--layers", type=int, default=4,
                     help="decode workloads: distinct layer pools (own block permutation each) the timed steps rotate over; "
                          "4 x 1.07 GB is 16 times the last-level cache, 1 re-reads one pool every step")

@@ -151,3 +151,79 @@ def test_captured_decode_loop_advances_lengths_on_the_device(device):
     K, V = model.dense(1)
     assert_bits_equal(gk, K, "pool K after the captured loop")
     assert_bits_equal(gv, V, "pool V after the captured loop")
+
+
+def test_manager_decode_step_captured_once_and_replayed_per_token(device):
+    """KVCacheManager.capture_decode: the whole decode step of a two-layer model -- per layer update_cache +
+    MultiHeadAttention on static tensors -- captured once, replayed per token with nothing but the inputs
+    changing; lengths advance on the device.  Attention against the oracle every step, cache contents bit-exact
+    at the end; any other cache operation ends the graph and step-by-step operation carries on."""
+    from oracle.paged_ref import RaggedCacheModel
+    from pace_mi355.llm import KVCacheManager, KVCacheType
+    from pace_mi355.ops import MultiHeadAttention
+
+    class Cfg:
+        num_hidden_layers = 2
+        num_attention_heads = 8
+        num_key_value_heads = 2
+
+    B, hkv, n_rep, D, steps = 3, 2, 4, 128, 70   # 70 steps cross the 64-token buckets an eager plan is kept for
+    lens0 = [300, 17, 1200]
+    mgr = KVCacheManager(Cfg(), 2048, KVCacheType.PAGED)
+    models = [RaggedCacheModel(B, hkv, D) for _ in range(2)]
+    for layer in range(2):
+        k, v = seeded_kv(10 + layer, B, hkv, max(lens0), D)
+        mgr[layer].append_ragged(k.to(device), v.to(device), lens0)
+        models[layer].append(k, v, lens0)
+    mha = MultiHeadAttention(dtype=torch.bfloat16)
+    qs = [torch.zeros(B, hkv * n_rep, 1, D, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    ks = [torch.zeros(B, hkv, 1, D, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    vs = [torch.zeros(B, hkv, 1, D, dtype=torch.bfloat16, device=device) for _ in range(2)]
+
+    def step():
+        outs = []
+        for layer in range(2):
+            pk, pv = mgr[layer].update_cache(ks[layer], vs[layer], 2)
+            outs.append(mha(qs[layer], pk, pv))
+        return outs
+
+    graph = mgr.capture_decode(step, max_steps=steps)
+    assert len(mgr) == max(lens0), "capturing leaves the cache as it was"
+    for i in range(steps):
+        new = []
+        for layer in range(2):
+            kn, vn = seeded_kv(1000 + 2 * i + layer, B, hkv, 1, D)
+            qn = seeded_q(2000 + 2 * i + layer, B, hkv * n_rep, 1, D)
+            ks[layer].copy_(kn), vs[layer].copy_(vn), qs[layer].copy_(qn)
+            models[layer].append(kn, vn)
+            new.append(qn)
+        outs = graph.replay()
+        assert len(mgr) == max(lens0) + i + 1
+        if i % 9 == 0 or i == steps - 1:
+            from helpers import assert_attention_close
+            for layer in range(2):
+                assert_attention_close(outs[layer], models[layer].attention(new[layer], n_rep), f"replay {i} layer {layer}")
+    with pytest.raises(RuntimeError, match="reserved blocks for"):
+        graph.replay()
+    for layer in range(2):
+        K, V = models[layer].dense(1)
+        gk, gv = mgr[layer].gather(n_rep=1)
+        assert_bits_equal(gk, K, f"pool K of layer {layer}")
+        assert_bits_equal(gv, V, f"pool V of layer {layer}")
+    # a second graph, ended early by a rollback; the eager path carries on from there
+    graph = mgr.capture_decode(step, max_steps=8)
+    for layer in range(2):
+        kn, vn = seeded_kv(5000 + layer, B, hkv, 1, D)
+        ks[layer].copy_(kn), vs[layer].copy_(vn)
+        models[layer].append(kn, vn)
+    graph.replay()
+    mgr.remove_cache(1)
+    for m in models:
+        m.truncate([1] * B)
+    with pytest.raises(RuntimeError, match="spent"):
+        graph.replay()
+    outs = step()
+    for layer in range(2):
+        models[layer].append(ks[layer].cpu(), vs[layer].cpu())
+        from helpers import assert_attention_close
+        assert_attention_close(outs[layer], models[layer].attention(qs[layer].cpu(), n_rep), f"eager step after the graph, layer {layer}")
