@@ -88,8 +88,30 @@ def _randn_bf16(torch, shape, gen, dev):
     return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
 
 
-def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor=None, headroom=64, permute=True):
-    """Paged cache holding lens[b] tokens per sequence, physical blocks in a seeded random order."""
+def alloc_free_history(alloc, seed, lo_blocks, hi_blocks, occupancy=0.75, turnover=4.0):
+    """Leave the free list in the order a serving history leaves it in: sequences of lo..hi blocks (log-uniform)
+    are admitted while the pool is below `occupancy` and retired at random, until `turnover` times the pool has
+    been handed out; then the survivors retire in random order.  Seeded."""
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    live, handed = [], 0
+    while handed < turnover * alloc.num_blocks:
+        used = alloc.num_blocks - alloc.num_free
+        n = int(round(math.exp(rng.uniform(math.log(lo_blocks), math.log(hi_blocks)))))
+        if used + n <= occupancy * alloc.num_blocks and (not live or rng.random() < 0.7):
+            live.append(alloc.allocate(n))
+            handed += n
+        elif live:
+            alloc.free(live.pop(int(rng.integers(len(live)))))
+    for i in rng.permutation(len(live))[::-1]:
+        alloc.free(live[i])
+
+
+def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor=None, headroom=64, permute=True,
+                history=False):
+    """Paged cache holding lens[b] tokens per sequence, physical blocks in a seeded random order (a shuffle of
+    the free list) or, with `history`, in the order a seeded admit / retire history of sequences leaves behind."""
     import numpy as np
     from pace_mi355.llm import PagedKVCache
 
@@ -107,6 +129,10 @@ def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor
         if t0 == 0:
             cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)  # creates the pool and the free list
             alloc = cache.state.allocator
+            if history:
+                alloc_free_history(alloc, seed, 8, 1024)
+                cache.append_ragged(k, v, np.clip(lens_np - t0, 0, n))
+                continue
             ids = alloc.allocate(alloc.num_free)
             if permute:
                 np.random.default_rng(seed).shuffle(ids)  # consecutive logical blocks end up far apart in HBM
@@ -392,7 +418,8 @@ def wl_ragged(torch, dev, args):
     B, hq, hkv, D = 256, 32, 8, 128
     rng = np.random.default_rng(2)
     lens = np.round(np.exp(rng.uniform(math.log(128), math.log(16384), B))).astype(int).tolist()
-    cache = build_cache(torch, dev, lens, hq, hkv, D, seed=3, pool_factor=1.3, headroom=16)
+    # pool 1.3x the live blocks, free list as a seeded admit / retire history of sequences leaves it (seed 3)
+    cache = build_cache(torch, dev, lens, hq, hkv, D, seed=3, pool_factor=1.3, headroom=16, history=True)
     cache.partition_tokens = args.partition
     g = torch.Generator(device=dev).manual_seed(4)
     k1, v1 = _randn_bf16(torch, (B, hkv, 1, D), g, dev), _randn_bf16(torch, (B, hkv, 1, D), g, dev)
@@ -408,7 +435,8 @@ def wl_ragged(torch, dev, args):
         forms[form] = roofline(f"kv_gather_kernel<128,{'true' if form == 'packed' else 'false'}> ({form.replace('_', ' ')})", gather_b,
                                time_call(torch, fn, reps=5, warmup=1))
     return result_line(
-        args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x, "
+        args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x "
+        "with the free list left by a seeded admit / retire history (seed 3), "
         "1-token append + GQA decode", dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline(step.kernel + " (decode, ragged) + merge", dec, attn_ms, {"work_items": step.n_items, "max_parts": step.max_parts}),
         extra={"gather": forms})

@@ -18,16 +18,22 @@ def _randn_bf16(shape, gen, dev):
     return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
 
 
-def _scramble(cache, k1, v1, seed, churn=None):
-    """Initialise the cache's state and leave its free list in a seeded, fragmented order."""
+def _scramble(cache, k1, v1, seed, history=False):
+    """Initialise the cache's state and leave its free list in a seeded, fragmented order: a shuffle, or what a
+    seeded admit / retire history of sequences leaves behind (the ragged serving mix)."""
     cache.append_ragged(k1, v1, [0] * k1.shape[0])
     alloc = cache.state.allocator
+    if history:
+        from bench import alloc_free_history
+
+        alloc_free_history(alloc, seed, 8, 1024)
+        return
     ids = alloc.allocate(alloc.num_free)
     np.random.default_rng(seed).shuffle(ids)
     alloc.free(ids)
 
 
-def _fill(cache, lens, gen, dev, hkv, D, chunk=1024, seed=0):
+def _fill(cache, lens, gen, dev, hkv, D, chunk=1024, seed=0, history=False):
     """Append lens[b] tokens to each sequence; returns the source K/V as [B, hkv, max, D] on the GPU."""
     B, T = len(lens), max(lens)
     K = torch.zeros(B, hkv, T, D, dtype=torch.bfloat16, device=dev)
@@ -38,7 +44,7 @@ def _fill(cache, lens, gen, dev, hkv, D, chunk=1024, seed=0):
         n = min(chunk, T - t0)
         k, v = _randn_bf16((B, hkv, n, D), gen, dev), _randn_bf16((B, hkv, n, D), gen, dev)
         if first:
-            _scramble(cache, k[:, :, :1], v[:, :, :1], seed)
+            _scramble(cache, k[:, :, :1], v[:, :, :1], seed, history)
             first = False
         counts = np.clip(lens - t0, 0, n)
         cache.append_ragged(k, v, counts)
@@ -136,7 +142,7 @@ def test_cfg3_ragged_mix_properties(device):
     live_blocks = sum((n + 15) // 16 for n in lens)
     cache = PagedKVCache(max(lens) + 16, num_kv_heads=Hkv, n_rep=4, num_blocks=int(1.3 * live_blocks))
     gen = torch.Generator(device=device).manual_seed(3)
-    K, V = _fill(cache, lens, gen, device, Hkv, D, chunk=2048, seed=3)
+    K, V = _fill(cache, lens, gen, device, Hkv, D, chunk=2048, seed=3, history=True)
     # append one more token everywhere, then decode
     k1, v1 = _randn_bf16((B, Hkv, 1, D), gen, device), _randn_bf16((B, Hkv, 1, D), gen, device)
     cache.update_cache(k1, v1, 2)
