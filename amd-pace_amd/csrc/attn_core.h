@@ -76,6 +76,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 // (value * log2(e)) is exact and equal values cancel exactly in the exponent.
 constexpr float kMaskFloor = -0x1p100f;
 constexpr uint32_t kMaskFloorBf16x2 = 0xf180f180u;  // the same value as a pair of bf16
+// How far (in powers of two of the weight) a row's scores may rise above the softmax reference before the reference
+// is moved and the accumulators rescaled.
+constexpr float kLazyLog2 = 8.0f;
 
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
@@ -102,6 +105,8 @@ struct RowState {
   f32x4 o[NQT][D / 16];  // O^T accumulators: dims 16j + 4g + i, query row n
   float m[NQT];          // running max while units are consumed: of the raw score products (no mask) or
                          // of scale * product + mask (with a mask); in log2 units after finish_rows()
+  float m_top[NQT];      // m + the slack a score may have over the reference before the reference moves
+  float m_neg[NQT];      // -(m * c), the addend of the exponent (0 while m is -inf); c: see softmax_and_output
   float l[NQT];          // this lane's share of the running sum
   int limit[NQT];        // last readable token of the row (-1: row is padding)
   int64_t mask_off[NQT]; // element offset of the row's mask line
@@ -277,13 +282,26 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
                      fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
     mx = row_max4(mx);
-    const float m_old = st.m[qt];
-    const float m_new = fmaxf(m_old, mx);
-    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-    // exponent = (score - max) * c with c = log2(e) (masked: natural units) or scale * log2(e)
+    // exponent = (score - reference) * c with c = log2(e) (masked: natural units) or scale * log2(e).
+    // The reference st.m follows the row's maximum lazily: it moves (and the accumulators are rescaled) only when
+    // a score exceeds it by more than 2^kLazyLog2 in weight, for any row of the wave; until then weights may
+    // exceed 1, which fp32 sums and bf16 weights (fp32's exponent range) take without loss.  A launch bound by the
+    // SIMD's issue saves the rescaling -- one multiply per accumulator register -- in most of its units: with the
+    // reference at the exact maximum, some row of a tile sees a new maximum in most units of a short walk.
     const float c = HAS_MASK ? kLog2e : p.scale_log2;
-    const float alpha = __builtin_amdgcn_exp2f((m_old - m_use) * c);  // m_old = -inf -> 0
-    const float m_neg = -(m_use * c);
+    if (__any(mx > st.m_top[qt])) {  // m_top = -inf at first: the first real score always moves the reference
+      const float m_old = st.m[qt];
+      const float m_new = fmaxf(m_old, mx);
+      const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_old - m_use) * c);  // m_old = -inf -> 0
+      st.m[qt] = m_new;
+      st.m_top[qt] = m_new + kLazyLog2 / c;
+      st.m_neg[qt] = -(m_use * c);
+      st.l[qt] *= alpha;
+#pragma unroll
+      for (int j = 0; j < MT; ++j) st.o[qt][j] *= alpha;
+    }
+    const float m_neg = st.m_neg[qt];
     float psum = 0.f;
     f32x4 pr[2];
 #pragma unroll
@@ -293,12 +311,7 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
         pr[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, m_neg));
         psum += pr[t][i];
       }
-    st.m[qt] = m_new;
-    st.l[qt] = st.l[qt] * alpha + psum;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int j = 0; j < MT; ++j) st.o[qt][j] *= alpha;
-    }
+    st.l[qt] += psum;
     u32x4 pb;
     pb[0] = pack_bf16x2(pr[0][0], pr[0][1]);
     pb[1] = pack_bf16x2(pr[0][2], pr[0][3]);

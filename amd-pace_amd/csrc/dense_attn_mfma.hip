@@ -64,7 +64,7 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
     } else {
       st.mask_off[qt] = 0;
     }
-    st.m[qt] = kNegInf;
+    st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
     const uint16_t* qp = p.q + (((int64_t)b * dp.N + head) * S + (valid ? s : 0)) * D + 8 * g;
 #pragma unroll
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     } else {
       st.mask_off[qt] = 0;
     }
-    st.m[qt] = kNegInf;
+    st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
     const uint16_t* qp = p.q + ((int64_t)pair * S + (valid ? s : 0)) * D + 8 * g;
 #pragma unroll

@@ -9,6 +9,7 @@
 // The inner step (one 32-token unit on the matrix cores) is in attn_core.h.
 #include <algorithm>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 #include "attn_core.h"
@@ -280,7 +281,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
     st.limit[qt] = valid ? (p.causal ? len - S + s : len - 1) : -1;
     if (valid) min_limit = min(min_limit, st.limit[qt]);
     st.mask_off[qt] = HAS_MASK ? (int64_t)b * p.m_sb + (int64_t)s * p.m_ss : 0;
-    st.m[qt] = kNegInf;
+    st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
     const uint16_t* qp = p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)s * p.q_ss + 8 * g;
 #pragma unroll
@@ -440,6 +441,188 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
         ml[0] = st.m[qt];
         ml[1] = l;
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Prefill-sized launches without a mask tensor: many groups of query rows read the same K / V.  Here the four
+// waves of a workgroup own 16*NQT query rows each and walk the context together.  Every 32-token unit is fetched
+// once per workgroup, straight from the pool into LDS (global_load_lds_dwordx4: no registers in between), one
+// unit ahead of its use, and each wave reads its operands back lane for lane: the pool's slab order is the
+// operand order, so lane l takes the 16 bytes lane l would have loaded from the pool.  Against one load of the
+// whole unit per wave (paged_attn_kernel) this moves a quarter of the bytes through the vector memory path and
+// takes the K / V latency out of the wave's cycle.  No merge: a row's softmax state never leaves its wave.
+// Not fused with the append, one partition per sequence; the host falls back to paged_attn_kernel otherwise.
+// ---------------------------------------------------------------------------------
+template <int D, int NQT, bool ROPE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) void paged_prefill_kernel(const PagedAttnParams p) {
+  constexpr int KK = D / 32, MT = D / 16, NW = 4;
+  constexpr int UNIT_CHUNKS = 2 * MT * 64;  // 16-byte pieces of a unit: MT loads of K, then MT loads of V, 64 lanes each
+  constexpr int PER = MT / NW;              // K loads and V loads each wave sends per unit
+  static_assert(MT % NW == 0, "a unit's loads must divide over the four waves");
+  typedef const __attribute__((address_space(1))) void* gptr;
+  typedef __attribute__((address_space(3))) void* lptr;
+  __shared__ __attribute__((aligned(16))) u32x4 stage[2][UNIT_CHUNKS];
+  const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Linear index -> (KV head, row group, sequence); KV head fastest: workgroups are dealt to the eight XCDs in
+  // turn, so that one head's K / V stay in one L2.  Row groups from the last to the first: under the causal
+  // limit the later rows read more, and the longest workgroups should not be the last to start.
+  const uint32_t item = blockIdx.x;
+  const int kvh = (int)(item % (uint32_t)p.num_kv_heads);
+  const uint32_t rest = item / (uint32_t)p.num_kv_heads;
+  const int rg = p.n_qgroups - 1 - (int)(rest % (uint32_t)p.n_qgroups);
+  const int b = min((int)(rest / (uint32_t)p.n_qgroups), p.batch - 1);
+  const int len = max(p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0), 0);
+  const int start = p.kv_start ? min(max(p.kv_start[b], 0), len) : 0;
+  const int S = p.q_len, R = S * p.n_rep;
+  const int tile0 = (rg * NW + wave) * NQT;  // first query tile of this wave
+
+  u32x4 qreg[NQT][KK];
+  u32x4 qtab[ROPE ? NQT : 1][KK];
+  RowState<D, NQT> st;
+  int row_s[NQT], row_h[NQT];
+  int min_limit = 0x7fffffff;
+  int tab_row[ROPE ? NQT : 1];
+  if (ROPE) {
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      const int r = (tile0 + qt) * 16 + n;
+      const int s = r < R ? r / p.n_rep : 0;
+      tab_row[qt] = rope_row(p.rope, b, s, len - S + s);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int r = (tile0 + qt) * 16 + n;
+    const bool valid = r < R;
+    const int s = valid ? r / p.n_rep : 0;
+    const int hq = kvh * p.n_rep + (valid ? r % p.n_rep : 0);
+    row_s[qt] = s;
+    row_h[qt] = hq;
+    st.limit[qt] = valid ? (p.causal ? len - S + s : len - 1) : -1;
+    if (valid) min_limit = min(min_limit, st.limit[qt]);
+    st.mask_off[qt] = 0;
+    st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
+    st.l[qt] = 0.f;
+    const uint16_t* qp = p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)s * p.q_ss + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
+    }
+    if (ROPE) {
+      if (valid) {
+        rope_fetch_row<D>(p.rope, tab_row[qt], g, qtab[qt]);
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  min_limit = min(min_limit, __shfl_xor(min_limit, 1, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 2, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 4, 64));
+  min_limit = min(min_limit, __shfl_xor(min_limit, 8, 64));
+  min_limit = __builtin_amdgcn_readfirstlane(min_limit);
+
+  // Where the workgroup stops (the causal limit of its last row) and where this wave does (of its own last row).
+  const int wg_last = min(R, (rg + 1) * NW * NQT * 16) - 1;  // >= 0: the grid has no empty row group
+  const int wave_last = min(R, (tile0 + NQT) * 16) - 1;      // < tile0 * 16: this wave has no rows
+  const bool wave_rows = tile0 * 16 < R;
+  const int wg_end = p.causal ? min(len, len - S + wg_last / p.n_rep + 1) : len;
+  const int wave_end = !wave_rows ? 0 : (p.causal ? min(len, len - S + wave_last / p.n_rep + 1) : len);
+  const int u0 = start / 32;                     // units before the first readable token are not walked
+  const int u_end = max((wg_end + 31) / 32, u0);  // workgroup-uniform: every wave makes the same trips
+
+  WaveBlockIds ids = load_block_ids<1>(p, b, 0, 0, u0, lane);
+  int ids_first = u0;
+  // This wave's share of a unit's loads, sent into stage `s`: K loads wave*PER .. and V loads wave*PER .. of the
+  // unit's MT each.  A wave's K loads lie 512 bytes apart inside one token tile (PER divides KK), and so do its
+  // V loads: one address per operand and unit, the rest are immediate offsets.  What does not depend on the unit
+  // is added up here, once; the unit adds its blocks' offsets, which are wave-uniform products.
+  static_assert(KK % PER == 0, "a wave's K loads must stay inside one token tile");
+  const int k_first = wave * PER;
+  const uint16_t* const k_lane = p.kpool + (int64_t)kvh * p.k_hs + g * 64 + (n & 7) * 8 + (k_first / KK) * (D * 8) + (k_first % KK) * 256;
+  const uint16_t* const v_lane = p.vpool + (int64_t)kvh * p.v_hs + ((g & 1) * 16 + n) * 8 + k_first * 256;
+  auto send = [&](int u, int s) {
+    const int rel = u - ids_first;
+    const int ia = ids.get(2 * rel), ib = ids.get(2 * rel + 1);
+    const int64_t ka = (int64_t)ia * p.k_bs, kb = (int64_t)ib * p.k_bs, va = (int64_t)ia * p.v_bs, vb = (int64_t)ib * p.v_bs;
+    const uint16_t* kp = k_lane + (n >= 8 ? kb : ka);
+    const uint16_t* vp = v_lane + (g >= 2 ? vb : va);
+    // The instruction's immediate offset (a literal for the builtin) moves the address in the pool and the
+    // address in LDS alike: the second load of an operand is 512 bytes on in the pool but 1024 in the stage, so
+    // its LDS base makes up the difference.
+    static_assert(PER == 1 || PER == 2, "one or two loads per operand and wave");
+    u32x4* const ks = &stage[s][k_first * 64];
+    u32x4* const vs = &stage[s][(MT + k_first) * 64];
+    __builtin_amdgcn_global_load_lds((gptr)kp, (lptr)ks, 16, 0, 0);
+    if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)kp, (lptr)(ks + 32), 16, 512, 0);
+    __builtin_amdgcn_global_load_lds((gptr)vp, (lptr)vs, 16, 0, 0);
+    if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)vp, (lptr)(vs + 32), 16, 512, 0);
+  };
+  if (u0 < u_end) send(u0, 0);
+  if (ROPE) {
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
+  }
+  MaskRegs<NQT> no_mask;
+  // Unit u is complete in its stage once every wave's loads are back (each waits for its own, then the barrier);
+  // the same barrier says that every wave has taken unit u - 1 out of the other stage, which the next loads reuse.
+  auto turn = [&](int u) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (u + 1 < u_end) {
+      if (u + 1 - ids_first == 64) {
+        ids = load_block_ids<1>(p, b, 0, 0, u + 1, lane);
+        ids_first = u + 1;
+      }
+      send(u + 1, ((u - u0) & 1) ^ 1);
+    }
+  };
+  // The units every row of the wave reads in full lie in one stretch: from the first readable token to the
+  // causal limit of the wave's first row.  Before and after it, masked units; past the wave's own last row,
+  // only the loads and the barriers.  One loop per kind: with the masked and the whole form of the inner step in
+  // one loop body the accumulators have two paths through it, and the register allocator spills them.
+  const int u_mine = min(max((wave_end + 31) / 32, u0), u_end);
+  const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
+  const int u_whole_begin = min((start + 31) / 32, u_whole_end);
+  auto walk = [&](int from, int to, auto whole) {
+    for (int u = from; u < to; ++u) {
+      turn(u);
+      const int s = (u - u0) & 1, t0 = 32 * u;
+      UnitRegs<D> buf;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = stage[s][(t * KK + kk) * 64 + lane];
+#pragma unroll
+      for (int j = 0; j < MT; ++j) buf.v[j] = stage[s][(MT + j) * 64 + lane];
+      compute_unit_impl<D, NQT, false, decltype(whole)::value>(buf, qreg, st, p, t0, wave_end, start, g, no_mask);
+    }
+  };
+  walk(u0, u_whole_begin, std::false_type{});
+  walk(u_whole_begin, u_whole_end, std::true_type{});
+  walk(u_whole_end, u_mine, std::false_type{});
+  for (int u = u_mine; u < u_end; ++u) turn(u);
+  finish_rows<D, NQT, false>(st, p);
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int r = (tile0 + qt) * 16 + n;
+    if (r >= R) continue;
+    const float l = st.l[qt];
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)row_h[qt] * p.o_sh + (int64_t)row_s[qt] * p.o_ss + 4 * g;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      u32x2 w;
+      w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
+      w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
+      *reinterpret_cast<u32x2*>(op + 16 * j) = w;
     }
   }
 }
@@ -655,6 +838,49 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
   return false;
 }
 
+// Query tiles per wave for paged_prefill_kernel (four waves per workgroup, two workgroups per compute unit), or 0
+// when the launch should keep paged_attn_kernel: fewer row groups than the GPU has room for (they would leave compute
+// units idle; paged_attn_kernel splits the context over more workgroups instead).  Between two and three tiles the
+// number of rounds the workgroups need decides: a row group of three tiles per wave takes 1.5 times as long as one
+// of two, and a last round that is nearly empty costs as much as a full one.
+static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs) {
+  if (head_dim != 64 && head_dim != 128) return 0;
+  if (tiles < 8) return 0;
+  const int64_t slots = (int64_t)compute_units() * 2;
+  int best = 0;
+  double best_cost = 0.;
+  for (int nqt = 3; nqt >= 2; --nqt) {
+    const int64_t groups = pairs * ((tiles + 4 * nqt - 1) / (4 * nqt));
+    if (groups < slots / 4) continue;
+    const double cost = (double)((groups + slots - 1) / slots) * nqt * (nqt == 2 ? 1.05 : 1.0);
+    if (best == 0 || cost < best_cost) best = nqt, best_cost = cost;
+  }
+  return best;
+}
+
+template <int D>
+static bool launch_prefill(int nqt, const PagedAttnParams& p, hipStream_t s) {
+  if constexpr (D == 64 || D == 128) {
+    const bool rope = p.rope.cos != nullptr;
+    if (g_name_out) {
+      snprintf(g_name_out, g_name_cap, "pace_kv::paged_prefill_kernel<%d, %d, %s>", D, nqt, rope ? "true" : "false");
+      return true;
+    }
+    const dim3 grid((unsigned)p.total_items), block(256);
+    if (nqt == 3) {
+      if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 3, true>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((paged_prefill_kernel<D, 3, false>), grid, block, 0, s, p);
+      return true;
+    }
+    if (nqt == 2) {
+      if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 2, true>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((paged_prefill_kernel<D, 2, false>), grid, block, 0, s, p);
+      return true;
+    }
+  }
+  return false;
+}
+
 // Scratch of the entry point that allocates nothing: one array per GPU, in the library's own device image.
 // In host code the array's name is only a stand-in; the address each device holds it at comes from
 // hipGetSymbolAddress, once per device, and that address is what kernels and checks are given.
@@ -748,6 +974,11 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     max_parts = a->max_parts;
   }
 
+  // Many row groups per KV head, no mask tensor, no fused append, one partition per sequence: the cooperative kernel.
+  const int prefill_nqt = (!a->mask && !a->k_new && max_parts == 1)
+                              ? prefill_tiles_per_wave(pool->head_dim, tiles, (int64_t)a->batch * pool->num_kv_heads)
+                              : 0;
+
   PagedAttnParams p;
   p.q = static_cast<const uint16_t*>(a->q);
   p.q_sb = a->q_stride_b, p.q_sh = a->q_stride_h, p.q_ss = a->q_stride_s;
@@ -817,6 +1048,16 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     PACE_HIP_CHECK(hipGetLastError());
   }
   bool ok = false;
+  if (prefill_nqt) {
+    p.items = nullptr;  // one partition per sequence: a work list only orders the sequences, and this kernel has its own order
+    p.n_qgroups = (tiles + 4 * prefill_nqt - 1) / (4 * prefill_nqt);
+    p.total_items = (long long)a->batch * pool->num_kv_heads * p.n_qgroups;
+    for_head_dim(pool->head_dim, [&](auto d) { ok = launch_prefill<decltype(d)::value>(prefill_nqt, p, s); });
+    PACE_REQUIRE(ok, "%s: no prefill kernel built for head_dim %d with %d tiles per wave", who, pool->head_dim, prefill_nqt);
+    if (g_name_out) return PACE_KV_OK;
+    PACE_HIP_CHECK(hipGetLastError());
+    return PACE_KV_OK;
+  }
   for_head_dim(pool->head_dim, [&](auto d) { ok = launch_shape<decltype(d)::value>(sh, p, has_mask, s); });
   PACE_REQUIRE(ok, "%s: no kernel built for shape nqt=%d nw=%d occ=%d..%d", who, sh.nqt, sh.nw, sh.occ, sh.occ_max);
   if (g_name_out) return PACE_KV_OK;

@@ -3,6 +3,7 @@ array inside the library's device image instead of a caller workspace; everythin
 of pace_paged_attn_verify, so the two must agree bit for bit.  Two calls in a row share the array, the
 second with a smaller input; a launch whose partials exceed the array is refused."""
 import ctypes
+import gc
 import math
 
 import pytest
@@ -51,9 +52,10 @@ def _both(device, seed, B, hkv, n_rep, D, S, lens, partition):
     a, keep = _args(nat, cache, q, out_ws, partition, ws)
     nat.check(lib.pace_paged_attn_verify(ctypes.byref(cache._desc), ctypes.byref(a), nat.current_stream_ptr()))
     b, keep2 = _args(nat, cache, q, out_static, partition)  # no workspace at all
+    gc.collect()  # tensors of earlier tests that are still waiting for the collector would be freed in between
     before = torch.cuda.memory_allocated()
     nat.check(lib.pace_paged_attn_verify_static(ctypes.byref(cache._desc), ctypes.byref(b), nat.current_stream_ptr()))
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_allocated() <= before, "the entry point took memory from torch's allocator"
     torch.cuda.synchronize()
     return out_ws, out_static, model.attention(q_host, n_rep)
 
