@@ -839,19 +839,22 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
 }
 
 // Query tiles per wave for paged_prefill_kernel (four waves per workgroup, two workgroups per compute unit), or 0
-// when the launch should keep paged_attn_kernel: fewer row groups than the GPU has room for (they would leave compute
-// units idle; paged_attn_kernel splits the context over more workgroups instead).  Between two and three tiles the
-// number of rounds the workgroups need decides: a row group of three tiles per wave takes 1.5 times as long as one
-// of two, and a last round that is nearly empty costs as much as a full one.
-static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs) {
+// when the launch should keep paged_attn_kernel: with few row groups the compute units are better filled by
+// splitting the context over more workgroups, which only paged_attn_kernel does.  Measured with 512-token chunks of
+// 32 Q / 8 KV heads: one sequence (a quarter of the GPU's workgroup slots) is 23 % faster here on 512 cached tokens
+// and 23 % slower on 3584; from two sequences on this kernel wins at either length.
+// Between two and three tiles the number of rounds the workgroups need decides: a row group of three tiles per
+// wave takes 1.5 times as long as one of two, and a last round that is nearly empty costs as much as a full one.
+static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs, int max_seq_len) {
   if (head_dim != 64 && head_dim != 128) return 0;
   if (tiles < 8) return 0;
   const int64_t slots = (int64_t)compute_units() * 2;
+  const int64_t least = max_seq_len <= 2048 ? slots / 4 : slots / 2;
   int best = 0;
   double best_cost = 0.;
   for (int nqt = 3; nqt >= 2; --nqt) {
     const int64_t groups = pairs * ((tiles + 4 * nqt - 1) / (4 * nqt));
-    if (groups < slots / 4) continue;
+    if (groups < least) continue;
     const double cost = (double)((groups + slots - 1) / slots) * nqt * (nqt == 2 ? 1.05 : 1.0);
     if (best == 0 || cost < best_cost) best = nqt, best_cost = cost;
   }
@@ -974,10 +977,13 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     max_parts = a->max_parts;
   }
 
-  // Many row groups per KV head, no mask tensor, no fused append, one partition per sequence: the cooperative kernel.
-  const int prefill_nqt = (!a->mask && !a->k_new && max_parts == 1)
-                              ? prefill_tiles_per_wave(pool->head_dim, tiles, (int64_t)a->batch * pool->num_kv_heads)
-                              : 0;
+  // Many row groups per KV head, no mask tensor, no fused append: the cooperative kernel, which takes every sequence
+  // in one piece -- unless the caller asked for a split (an explicit partition_tokens, or a work list that has one).
+  int prefill_nqt = (!a->mask && !a->k_new) ? prefill_tiles_per_wave(pool->head_dim, tiles, (int64_t)a->batch * pool->num_kv_heads, a->max_seq_len) : 0;
+  if (prefill_nqt) {
+    if (a->work_items ? max_parts != 1 : (a->partition_tokens > 0 && max_parts != 1)) prefill_nqt = 0;
+    else max_parts = 1;
+  }
 
   PagedAttnParams p;
   p.q = static_cast<const uint16_t*>(a->q);
@@ -1162,16 +1168,18 @@ extern "C" int pace_paged_attn_plan(const int32_t* seq_lens, const int32_t* bloc
   }
   const int part = max_len > 0 ? resolve_partition(want, max_len, batch, num_kv_heads, rows, head_dim) : 128;
   const int cap = partition_cap(head_dim, tiles);
+  // A launch the cooperative prefill kernel takes (no mask tensor, many row groups) walks every sequence in one piece.
+  const bool one_each = partition_tokens == 0 && !masked && prefill_tiles_per_wave(head_dim, tiles, (int64_t)batch * num_kv_heads, max_len) > 0;
   // Workgroups resident at a time, per (KV head, row group): the launch's slots for (sequence, partition) pairs.
   const int64_t slots = std::max<int64_t>(1, (int64_t)compute_units() * 4 * sh.occ / sh.nw / ((int64_t)num_kv_heads * n_qgroups));
   std::vector<int> n(batch);
   int64_t sum_base = 0, sum_cap = 0;
   for (int b = 0; b < batch; ++b) {
-    n[b] = std::max(1, (seq_lens[b] + part - 1) / part);
+    n[b] = one_each ? 1 : std::max(1, (seq_lens[b] + part - 1) / part);
     sum_base += n[b];
     sum_cap += std::max(1, (seq_lens[b] + cap - 1) / cap);
   }
-  if (!uniform && sum_cap < slots && sum_base <= slots) {
+  if (!one_each && !uniform && sum_cap < slots && sum_base <= slots) {
     // The whole launch fits the GPU in one round: choose the partition counts so that the partitions are as
     // equal as possible and fill the slots (the longest share is cut next, while a cut leaves 256 tokens or more).
     int64_t used = 0;

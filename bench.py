@@ -540,6 +540,7 @@ def wl_prefill(torch, dev, args):
     causal attention of the chunk over the cache (the reference runs prefill as the same update_cache +
     attention pair with q_len = prompt length, pace/llm/models/llama.py:286-299)."""
     B, hq, hkv, D, past, S = 8, 32, 8, 128, 3584, 512
+    B, past = args.batch or B, args.context or past  # --batch / --context: other batch sizes / cached lengths
     cache = build_cache(torch, dev, [past] * B, hq, hkv, D, seed=8, headroom=S + 64)
     cache.partition_tokens = args.partition
     g = torch.Generator(device=dev).manual_seed(9)
@@ -558,7 +559,7 @@ def wl_prefill(torch, dev, args):
     kv_once = decode_bytes([past + S] * B, hq, hkv, D, q_len=S)
     tflops = flops / (attn_ms * 1e-3) / 1e12
     return result_line(
-        args, "chunked prefill: batch 8, 512-token chunk on top of 3584 cached tokens, 32 Q / 8 KV heads, head_dim 128; "
+        args, f"chunked prefill: batch {B}, 512-token chunk on top of {past} cached tokens, 32 Q / 8 KV heads, head_dim 128; "
         "block append + causal attention of the chunk", kv_once + append_bytes(B, S, hkv, D), B * S, dt,
         {"bound": "mfma", "kernel": step.kernel + (" (prefill chunk, explicit mask)" if args.mask else " (prefill chunk)"), "achieved": round(tflops, 1),
          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
@@ -769,8 +770,8 @@ def main() -> int:
     ap.add_argument("--path", choices=("api", "direct", "graph"), default="direct",
                     help="decode workloads. direct: C-ABI calls with fixed metadata; api: PagedKVCache.update_cache + "
                          "MultiHeadAttention; graph: the api calls captured once into a HIP graph and replayed per step")
-    ap.add_argument("--batch", type=int, default=0, help="decode workloads: override the batch size (latency studies)")
-    ap.add_argument("--context", type=int, default=0, help="decode workloads: override the context length")
+    ap.add_argument("--batch", type=int, default=0, help="decode and prefill workloads: override the batch size (latency studies)")
+    ap.add_argument("--context", type=int, default=0, help="decode and prefill workloads: override the context length (prefill: the cached tokens)")
     ap.add_argument("--layers", type=int, default=4,
                     help="decode workloads: distinct layer pools (own block permutation each) the timed steps rotate over; "
                          "4 x 1.07 GB is 16 times the last-level cache, 1 re-reads one pool every step")

@@ -383,6 +383,55 @@ def test_prefill_sized_launch_matches_oracle(device, D, S, n_rep):
     assert_attention_close(out, ref, f"prefill-sized S={S} D={D}")
 
 
+def _kernel_of(cache, q, lens, kv_start=None):
+    """Name of the kernel an unmasked, unfused attention call of this shape launches."""
+    import math
+
+    from pace_mi355 import _native as nat
+
+    B, hq, S, D = q.shape
+    table = cache.state.device_table()
+    a = nat.PagedAttnArgs()
+    a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    lens_dev = torch.tensor(lens, dtype=torch.int32, device=q.device)
+    a.block_table, a.table_stride, a.seq_lens = table.data_ptr(), table.stride(0), lens_dev.data_ptr()
+    a.causal, a.batch, a.num_q_heads, a.q_len = 1, B, hq, S
+    a.max_seq_len, a.partition_tokens, a.scale = max(lens), 0, 1.0 / math.sqrt(D)
+    return nat.kernel_name(cache._desc, a)
+
+
+@pytest.mark.parametrize("D,S,n_rep,top", [(128, 64, 4, 2400), (64, 96, 4, 700)])
+def test_cooperative_prefill_kernel_long_ragged_and_windowed(device, D, S, n_rep, top):
+    """The workgroup-cooperative prefill kernel: ragged lengths past 64 units (the block ids are fetched 64
+    units at a time), a row group that is only partly filled, and a first readable token per sequence
+    (kv_start: aligned to a unit, inside one, zero, and past the chunk's first row)."""
+    B, hkv = 16, 8
+    rng = np.random.default_rng(D + S)
+    lens = (rng.integers(S, top, B)).tolist()
+    lens[0], lens[1], lens[2] = top, S, S + 31
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=S + D + 1)
+    q = seeded_q(33, B, hkv * n_rep, S, D)
+    qd = q.to(device)
+    assert "paged_prefill_kernel" in _kernel_of(cache, qd, lens), "the case is meant for the cooperative kernel"
+    starts = rng.integers(0, 200, B).astype(np.int32)
+    starts[0], starts[1], starts[2], starts[3] = 0, 0, 64, 45
+    starts = np.minimum(starts, np.array(lens, dtype=np.int32) - 1)
+    for start in (None, starts):
+        dev_start = None if start is None else torch.from_numpy(start).to(device)
+        out = cache.attend(qd, kv_start=dev_start)
+        K, V = model.dense(n_rep)
+        mask = lengths_mask_4d(lens, S, K.shape[2], torch.float32, kv_start=start)
+        ref = sdpa_fp32(q, K, V, mask)
+        # a row whose window holds no token (start past its position) has no defined result in the oracle (it
+        # averages every column); the kernels give 0 there
+        empty = (mask == torch.finfo(torch.float32).min).all(dim=-1, keepdim=True).expand(-1, hkv * n_rep, -1, D)
+        got = out.float().cpu()
+        assert torch.all(got[empty] == 0)
+        assert_attention_close(torch.where(empty, torch.zeros_like(got), got), torch.where(empty, torch.zeros_like(ref), ref),
+                               f"cooperative prefill D={D} S={S} window={start is not None}")
+
+
 def test_prefill_sized_launch_with_rope_rotates_queries(device):
     from oracle import rope_ref
     from pace_mi355.llm import PagedKVCache
