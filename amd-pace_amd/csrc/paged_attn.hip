@@ -453,9 +453,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
 // operand order, so lane l takes the 16 bytes lane l would have loaded from the pool.  Against one load of the
 // whole unit per wave (paged_attn_kernel) this moves a quarter of the bytes through the vector memory path and
 // takes the K / V latency out of the wave's cycle.  No merge: a row's softmax state never leaves its wave.
+// With HAS_MASK the additive mask tensor decides what a row reads; its values for the next unit are fetched a unit
+// ahead, like K / V, and where the per-row summary of the mask is at hand (row_last) the wave and the workgroup stop
+// at the last column their rows can use -- the diagonal of a causal mask.
 // Not fused with the append, one partition per sequence; the host falls back to paged_attn_kernel otherwise.
 // ---------------------------------------------------------------------------------
-template <int D, int NQT, bool ROPE>
+template <int D, int NQT, bool ROPE, bool HAS_MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) void paged_prefill_kernel(const PagedAttnParams p) {
   constexpr int KK = D / 32, MT = D / 16, NW = 4;
   constexpr int UNIT_CHUNKS = 2 * MT * 64;  // 16-byte pieces of a unit: MT loads of K, then MT loads of V, 64 lanes each
@@ -503,7 +506,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     row_h[qt] = hq;
     st.limit[qt] = valid ? (p.causal ? len - S + s : len - 1) : -1;
     if (valid) min_limit = min(min_limit, st.limit[qt]);
-    st.mask_off[qt] = 0;
+    st.mask_off[qt] = HAS_MASK ? (int64_t)b * p.m_sb + (int64_t)s * p.m_ss : 0;
     st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
     const uint16_t* qp = p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)s * p.q_ss + 8 * g;
@@ -533,8 +536,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
   const int wg_last = min(R, (rg + 1) * NW * NQT * 16) - 1;  // >= 0: the grid has no empty row group
   const int wave_last = min(R, (tile0 + NQT) * 16) - 1;      // < tile0 * 16: this wave has no rows
   const bool wave_rows = tile0 * 16 < R;
-  const int wg_end = p.causal ? min(len, len - S + wg_last / p.n_rep + 1) : len;
-  const int wave_end = !wave_rows ? 0 : (p.causal ? min(len, len - S + wave_last / p.n_rep + 1) : len);
+  int wg_end = p.causal ? min(len, len - S + wg_last / p.n_rep + 1) : len;
+  int wave_end = !wave_rows ? 0 : (p.causal ? min(len, len - S + wave_last / p.n_rep + 1) : len);
+  if (HAS_MASK && p.row_last) {
+    // Nothing past the last column any row can use is needed -- provided every row has a real score somewhere, so
+    // that the columns left out weigh exactly 0; a row masked everywhere ends as the average of V and keeps every
+    // column.  Once over this wave's rows, once over the workgroup's (each lane looks up NQT of its 64 * NQT rows).
+    const int32_t* last_of = p.row_last + (int64_t)b * S;
+    int mine = -1, ours = -1;
+    bool mine_real = true, ours_real = true;
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      if (st.limit[qt] >= 0) {
+        const int v = last_of[row_s[qt]];
+        mine = max(mine, v), mine_real = mine_real && v >= 0;
+      }
+      const int r = rg * (NW * NQT * 16) + qt * 64 + lane;
+      if (r < R) {
+        const int v = last_of[r / p.n_rep];
+        ours = max(ours, v), ours_real = ours_real && v >= 0;
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o *= 2) mine = max(mine, __shfl_xor(mine, o, 64)), ours = max(ours, __shfl_xor(ours, o, 64));
+    if (__all(mine_real)) wave_end = min(wave_end, __builtin_amdgcn_readfirstlane(mine) + 1);
+    if (__all(ours_real)) wg_end = min(wg_end, __builtin_amdgcn_readfirstlane(ours) + 1);
+    wave_end = min(wave_end, wg_end);
+  }
   const int u0 = start / 32;                     // units before the first readable token are not walked
   const int u_end = max((wg_end + 31) / 32, u0);  // workgroup-uniform: every wave makes the same trips
 
@@ -570,7 +598,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
     for (int qt = 0; qt < NQT; ++qt) rope_apply_row<D>(p.rope, qtab[qt], qreg[qt]);
   }
-  MaskRegs<NQT> no_mask;
   // Unit u is complete in its stage once every wave's loads are back (each waits for its own, then the barrier);
   // the same barrier says that every wave has taken unit u - 1 out of the other stage, which the next loads reuse.
   auto turn = [&](int u) {
@@ -591,10 +618,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
   const int u_mine = min(max((wave_end + 31) / 32, u0), u_end);
   const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
   const int u_whole_begin = min((start + 31) / 32, u_whole_end);
+  // Mask values travel a unit ahead of their use, as K / V do: `coming` holds those of the next unit this wave walks.
+  MaskRegs<NQT> coming;
+  if (HAS_MASK && u0 < u_mine) load_mask_regs<NQT>(coming, p, st.mask_off, 32 * u0, g);
   auto walk = [&](int from, int to, auto whole) {
     for (int u = from; u < to; ++u) {
       turn(u);
       const int s = (u - u0) & 1, t0 = 32 * u;
+      MaskRegs<NQT> mregs;
+      if (HAS_MASK) {
+        mregs = coming;
+        if (u + 1 < u_mine) load_mask_regs<NQT>(coming, p, st.mask_off, t0 + 32, g);
+      }
       UnitRegs<D> buf;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -602,14 +637,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = stage[s][(t * KK + kk) * 64 + lane];
 #pragma unroll
       for (int j = 0; j < MT; ++j) buf.v[j] = stage[s][(MT + j) * 64 + lane];
-      compute_unit_impl<D, NQT, false, decltype(whole)::value>(buf, qreg, st, p, t0, wave_end, start, g, no_mask);
+      compute_unit_impl<D, NQT, HAS_MASK, decltype(whole)::value>(buf, qreg, st, p, t0, wave_end, start, g, mregs);
     }
   };
   walk(u0, u_whole_begin, std::false_type{});
   walk(u_whole_begin, u_whole_end, std::true_type{});
   walk(u_whole_end, u_mine, std::false_type{});
   for (int u = u_mine; u < u_end; ++u) turn(u);
-  finish_rows<D, NQT, false>(st, p);
+  finish_rows<D, NQT, HAS_MASK>(st, p);
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     const int r = (tile0 + qt) * 16 + n;
@@ -845,14 +880,14 @@ static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mas
 // and 23 % slower on 3584; from two sequences on this kernel wins at either length.
 // Between two and three tiles the number of rounds the workgroups need decides: a row group of three tiles per
 // wave takes 1.5 times as long as one of two, and a last round that is nearly empty costs as much as a full one.
-static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs, int max_seq_len) {
+static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs, int max_seq_len, bool masked) {
   if (head_dim != 64 && head_dim != 128) return 0;
   if (tiles < 8) return 0;
   const int64_t slots = (int64_t)compute_units() * 2;
   const int64_t least = max_seq_len <= 2048 ? slots / 4 : slots / 2;
   int best = 0;
   double best_cost = 0.;
-  for (int nqt = 3; nqt >= 2; --nqt) {
+  for (int nqt = masked ? 2 : 3; nqt >= 2; --nqt) {  // a mask's values take eight more registers per tile: two tiles then
     const int64_t groups = pairs * ((tiles + 4 * nqt - 1) / (4 * nqt));
     if (groups < least) continue;
     const double cost = (double)((groups + slots - 1) / slots) * nqt * (nqt == 2 ? 1.05 : 1.0);
@@ -864,20 +899,22 @@ static int prefill_tiles_per_wave(int head_dim, int tiles, int64_t pairs, int ma
 template <int D>
 static bool launch_prefill(int nqt, const PagedAttnParams& p, hipStream_t s) {
   if constexpr (D == 64 || D == 128) {
-    const bool rope = p.rope.cos != nullptr;
+    const bool rope = p.rope.cos != nullptr, masked = p.mask != nullptr;  // never both (checked by the caller)
     if (g_name_out) {
-      snprintf(g_name_out, g_name_cap, "pace_kv::paged_prefill_kernel<%d, %d, %s>", D, nqt, rope ? "true" : "false");
+      snprintf(g_name_out, g_name_cap, "pace_kv::paged_prefill_kernel<%d, %d, %s, %s>", D, nqt, rope ? "true" : "false",
+               masked ? "true" : "false");
       return true;
     }
     const dim3 grid((unsigned)p.total_items), block(256);
-    if (nqt == 3) {
-      if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 3, true>), grid, block, 0, s, p);
-      else hipLaunchKernelGGL((paged_prefill_kernel<D, 3, false>), grid, block, 0, s, p);
+    if (nqt == 3 && !masked) {
+      if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 3, true, false>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((paged_prefill_kernel<D, 3, false, false>), grid, block, 0, s, p);
       return true;
     }
     if (nqt == 2) {
-      if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 2, true>), grid, block, 0, s, p);
-      else hipLaunchKernelGGL((paged_prefill_kernel<D, 2, false>), grid, block, 0, s, p);
+      if (masked) hipLaunchKernelGGL((paged_prefill_kernel<D, 2, false, true>), grid, block, 0, s, p);
+      else if (rope) hipLaunchKernelGGL((paged_prefill_kernel<D, 2, true, false>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((paged_prefill_kernel<D, 2, false, false>), grid, block, 0, s, p);
       return true;
     }
   }
@@ -977,9 +1014,9 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     max_parts = a->max_parts;
   }
 
-  // Many row groups per KV head, no mask tensor, no fused append: the cooperative kernel, which takes every sequence
+  // Many row groups per KV head, no fused append: the cooperative kernel, which takes every sequence
   // in one piece -- unless the caller asked for a split (an explicit partition_tokens, or a work list that has one).
-  int prefill_nqt = (!a->mask && !a->k_new) ? prefill_tiles_per_wave(pool->head_dim, tiles, (int64_t)a->batch * pool->num_kv_heads, a->max_seq_len) : 0;
+  int prefill_nqt = !a->k_new ? prefill_tiles_per_wave(pool->head_dim, tiles, (int64_t)a->batch * pool->num_kv_heads, a->max_seq_len, a->mask != nullptr) : 0;
   if (prefill_nqt) {
     if (a->work_items ? max_parts != 1 : (a->partition_tokens > 0 && max_parts != 1)) prefill_nqt = 0;
     else max_parts = 1;
@@ -1168,8 +1205,8 @@ extern "C" int pace_paged_attn_plan(const int32_t* seq_lens, const int32_t* bloc
   }
   const int part = max_len > 0 ? resolve_partition(want, max_len, batch, num_kv_heads, rows, head_dim) : 128;
   const int cap = partition_cap(head_dim, tiles);
-  // A launch the cooperative prefill kernel takes (no mask tensor, many row groups) walks every sequence in one piece.
-  const bool one_each = partition_tokens == 0 && !masked && prefill_tiles_per_wave(head_dim, tiles, (int64_t)batch * num_kv_heads, max_len) > 0;
+  // A launch the cooperative prefill kernel takes (many row groups) walks every sequence in one piece.
+  const bool one_each = partition_tokens == 0 && prefill_tiles_per_wave(head_dim, tiles, (int64_t)batch * num_kv_heads, max_len, masked != 0) > 0;
   // Workgroups resident at a time, per (KV head, row group): the launch's slots for (sequence, partition) pairs.
   const int64_t slots = std::max<int64_t>(1, (int64_t)compute_units() * 4 * sh.occ / sh.nw / ((int64_t)num_kv_heads * n_qgroups));
   std::vector<int> n(batch);

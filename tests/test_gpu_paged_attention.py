@@ -383,8 +383,8 @@ def test_prefill_sized_launch_matches_oracle(device, D, S, n_rep):
     assert_attention_close(out, ref, f"prefill-sized S={S} D={D}")
 
 
-def _kernel_of(cache, q, lens, kv_start=None):
-    """Name of the kernel an unmasked, unfused attention call of this shape launches."""
+def _kernel_of(cache, q, lens, mask=None):
+    """Name of the kernel an unfused attention call of this shape launches."""
     import math
 
     from pace_mi355 import _native as nat
@@ -398,6 +398,9 @@ def _kernel_of(cache, q, lens, kv_start=None):
     a.block_table, a.table_stride, a.seq_lens = table.data_ptr(), table.stride(0), lens_dev.data_ptr()
     a.causal, a.batch, a.num_q_heads, a.q_len = 1, B, hq, S
     a.max_seq_len, a.partition_tokens, a.scale = max(lens), 0, 1.0 / math.sqrt(D)
+    if mask is not None:
+        a.causal, a.mask, a.mask_dtype, a.mask_len = 0, mask.data_ptr(), nat.DTYPE_BF16, mask.size(3)
+        a.mask_stride_b, a.mask_stride_s = mask.stride(0), mask.stride(2)
     return nat.kernel_name(cache._desc, a)
 
 
@@ -430,6 +433,30 @@ def test_cooperative_prefill_kernel_long_ragged_and_windowed(device, D, S, n_rep
         assert torch.all(got[empty] == 0)
         assert_attention_close(torch.where(empty, torch.zeros_like(got), got), torch.where(empty, torch.zeros_like(ref), ref),
                                f"cooperative prefill D={D} S={S} window={start is not None}")
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.bfloat16, torch.float32])
+def test_cooperative_prefill_kernel_with_a_mask_tensor(device, mask_dtype):
+    """The same kernel with the additive mask the reference's models pass (llama.py:292-299): ragged lengths through
+    the mask alone, a mask narrower than the longest sequence's block row, one row that is masked everywhere
+    (it must come out as the average of V over the mask's columns, like the reference's softmax of equal values)."""
+    B, hkv, n_rep, D, S = 16, 8, 4, 128, 64
+    rng = np.random.default_rng(5)
+    lens = (rng.integers(S, 900, B)).tolist()
+    lens[0], lens[1] = 900, S
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=91)
+    q = seeded_q(34, B, hkv * n_rep, S, D)
+    qd = q.to(device)
+    L = max(lens)
+    mask = lengths_mask_4d(lens, S, L, mask_dtype).clone()
+    mask[0, :, 5, :] = torch.finfo(mask_dtype).min  # a row with nothing to read, in the sequence that fills the mask
+    md = mask.to(device)
+    if mask_dtype == torch.bfloat16:
+        assert "paged_prefill_kernel<128, 2, false, true>" in _kernel_of(cache, qd, lens, md)
+    out = cache.attend(qd, attention_mask=md)
+    K, V = model.dense(n_rep)
+    ref = sdpa_fp32(q, K[:, :, :L], V[:, :, :L], mask.float())
+    assert_attention_close(out, ref, f"cooperative prefill with a {mask_dtype} mask")
 
 
 def test_prefill_sized_launch_with_rope_rotates_queries(device):
