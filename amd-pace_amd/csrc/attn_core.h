@@ -63,6 +63,10 @@ struct PagedAttnParams {
   // column the row can read whose mask value is above the floor, -1 if there is none (written by
   // mask_row_last_kernel just before the attention launch).
   const int32_t* row_last;
+  // Optional, with row_last: per (sequence, query token) the first column above the floor if the row's mask line is
+  // "plain" -- exactly 0 from there to row_last, at or below the floor everywhere else it can read (a causal or
+  // padding mask) -- and -1 if it is anything else.  A plain row needs its two columns, not its mask line.
+  const int32_t* row_first;
   // Optional rotary embedding (rope.cos == NULL: off): q rows are rotated as they are loaded,
   // the fused append's new keys before they are used and stored.  rotary_dim == D here.
   RopeDev rope;

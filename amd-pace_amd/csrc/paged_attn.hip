@@ -478,7 +478,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
   const int rg = p.n_qgroups - 1 - (int)(rest % (uint32_t)p.n_qgroups);
   const int b = min((int)(rest / (uint32_t)p.n_qgroups), p.batch - 1);
   const int len = max(p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0), 0);
-  const int start = p.kv_start ? min(max(p.kv_start[b], 0), len) : 0;
+  int lo_tok = p.kv_start ? min(max(p.kv_start[b], 0), len) : 0;
+  bool plain = false;  // HAS_MASK: the mask lines of the workgroup's rows are known to be plain (see row_first)
   const int S = p.q_len, R = S * p.n_rep;
   const int tile0 = (rg * NW + wave) * NQT;  // first query tile of this wave
 
@@ -562,7 +563,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     if (__all(mine_real)) wave_end = min(wave_end, __builtin_amdgcn_readfirstlane(mine) + 1);
     if (__all(ours_real)) wg_end = min(wg_end, __builtin_amdgcn_readfirstlane(ours) + 1);
     wave_end = min(wave_end, wg_end);
+    if (p.row_first) {
+      // Every row of the workgroup plain, and from the same first column (a causal mask, padded or not): the rows
+      // are then walked as rows without a mask tensor -- first column, own last column -- and the mask is not read.
+      const int32_t* first_of = p.row_first + (int64_t)b * S;
+      int f_min = 0x7fffffff, f_max = -1;
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) {
+        const int r = rg * (NW * NQT * 16) + qt * 64 + lane;
+        if (r < R) {
+          const int f = first_of[r / p.n_rep];
+          f_min = min(f_min, f), f_max = max(f_max, f);
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < 64; o *= 2) f_min = min(f_min, __shfl_xor(f_min, o, 64)), f_max = max(f_max, __shfl_xor(f_max, o, 64));
+      f_min = __builtin_amdgcn_readfirstlane(f_min), f_max = __builtin_amdgcn_readfirstlane(f_max);
+      plain = f_min >= 0 && f_min == f_max;  // (-1 marks a row that is not plain)
+      if (plain) {
+        lo_tok = max(lo_tok, f_min);
+        min_limit = 0x7fffffff;
+#pragma unroll
+        for (int qt = 0; qt < NQT; ++qt) {
+          if (st.limit[qt] >= 0) {
+            st.limit[qt] = min(st.limit[qt], last_of[row_s[qt]]);
+            min_limit = min(min_limit, st.limit[qt]);
+          }
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o *= 2) min_limit = min(min_limit, __shfl_xor(min_limit, o, 64));
+        min_limit = __builtin_amdgcn_readfirstlane(min_limit);
+      }
+    }
   }
+  const int start = lo_tok;                      // first token any row of the workgroup reads
   const int u0 = start / 32;                     // units before the first readable token are not walked
   const int u_end = max((wg_end + 31) / 32, u0);  // workgroup-uniform: every wave makes the same trips
 
@@ -620,13 +654,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
   const int u_whole_begin = min((start + 31) / 32, u_whole_end);
   // Mask values travel a unit ahead of their use, as K / V do: `coming` holds those of the next unit this wave walks.
   MaskRegs<NQT> coming;
-  if (HAS_MASK && u0 < u_mine) load_mask_regs<NQT>(coming, p, st.mask_off, 32 * u0, g);
-  auto walk = [&](int from, int to, auto whole) {
+  auto walk = [&](int from, int to, auto whole, auto masked) {
+    constexpr bool MASKED = decltype(masked)::value;
     for (int u = from; u < to; ++u) {
       turn(u);
       const int s = (u - u0) & 1, t0 = 32 * u;
       MaskRegs<NQT> mregs;
-      if (HAS_MASK) {
+      if (MASKED) {
         mregs = coming;
         if (u + 1 < u_mine) load_mask_regs<NQT>(coming, p, st.mask_off, t0 + 32, g);
       }
@@ -637,14 +671,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = stage[s][(t * KK + kk) * 64 + lane];
 #pragma unroll
       for (int j = 0; j < MT; ++j) buf.v[j] = stage[s][(MT + j) * 64 + lane];
-      compute_unit_impl<D, NQT, HAS_MASK, decltype(whole)::value>(buf, qreg, st, p, t0, wave_end, start, g, mregs);
+      compute_unit_impl<D, NQT, MASKED, decltype(whole)::value>(buf, qreg, st, p, t0, wave_end, start, g, mregs);
     }
   };
-  walk(u0, u_whole_begin, std::false_type{});
-  walk(u_whole_begin, u_whole_end, std::true_type{});
-  walk(u_whole_end, u_mine, std::false_type{});
+  bool by_mask = false;
+  if constexpr (HAS_MASK) by_mask = !plain;
+  if (by_mask) {
+    if constexpr (HAS_MASK) {
+      if (u0 < u_mine) load_mask_regs<NQT>(coming, p, st.mask_off, 32 * u0, g);
+      walk(u0, u_whole_begin, std::false_type{}, std::true_type{});
+      walk(u_whole_begin, u_whole_end, std::true_type{}, std::true_type{});
+      walk(u_whole_end, u_mine, std::false_type{}, std::true_type{});
+    }
+  } else {
+    walk(u0, u_whole_begin, std::false_type{}, std::false_type{});
+    walk(u_whole_begin, u_whole_end, std::true_type{}, std::false_type{});
+    walk(u_whole_end, u_mine, std::false_type{}, std::false_type{});
+  }
   for (int u = u_mine; u < u_end; ++u) turn(u);
-  finish_rows<D, NQT, HAS_MASK>(st, p);
+  // (the running maximum is in units of the scores the walk used: scaled with a mask, raw without)
+  if (by_mask) finish_rows<D, NQT, true>(st, p);
+  else finish_rows<D, NQT, false>(st, p);
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     const int r = (tile0 + qt) * 16 + n;
@@ -666,13 +713,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 // row can read ([kv_start, len) and inside the mask), that holds a value above the floor; -1 if none.
 // With it a workgroup knows where its rows stop needing the context -- the diagonal of a causal mask
 // -- and whether every row has a real score at all, without walking the mask itself.
-__global__ __launch_bounds__(64) void mask_row_last_kernel(const PagedAttnParams p, int32_t* out) {
+// first_out (optional): the first such column if the line is plain -- exactly 0 on every column from there to the
+// last one, which then are all above the floor -- else -1.
+__global__ __launch_bounds__(64) void mask_row_last_kernel(const PagedAttnParams p, int32_t* out, int32_t* first_out) {
   const int row = blockIdx.x, S = p.q_len, b = row / S, s = row % S, lane = threadIdx.x;
   const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
   const int start = p.kv_start ? p.kv_start[b] : 0;
   const int end = min(len, p.mask_len);
   const int64_t off = (int64_t)b * p.m_sb + (int64_t)s * p.m_ss;
-  int last = -1;
+  int last = -1, first = 0x7fffffff, above = 0;
+  bool zero = true;  // every value above the floor is 0
   for (int c0 = start + 8 * lane; c0 < end; c0 += 8 * 64) {
     float a[8];
     if (c0 + 8 <= end) {
@@ -697,11 +747,24 @@ __global__ __launch_bounds__(64) void mask_row_last_kernel(const PagedAttnParams
     }
 #pragma unroll
     for (int c = 0; c < 8; ++c)
-      if (a[c] > kMaskFloor) last = c0 + c;  // ascending: the largest column wins (NaN compares false: treated as masked)
+      if (a[c] > kMaskFloor) {  // ascending: the largest column wins (NaN compares false: treated as masked)
+        last = c0 + c;
+        first = min(first, c0 + c);
+        above += 1;
+        zero = zero && a[c] == 0.f;
+      }
   }
 #pragma unroll
-  for (int o = 1; o < 64; o *= 2) last = max(last, __shfl_xor(last, o, 64));
-  if (lane == 0) out[row] = last;
+  for (int o = 1; o < 64; o *= 2) {
+    last = max(last, __shfl_xor(last, o, 64));
+    first = min(first, __shfl_xor(first, o, 64));
+    above += __shfl_xor(above, o, 64);
+  }
+  const bool plain = __all(zero) && last >= 0 && above == last - first + 1;
+  if (lane == 0) {
+    out[row] = last;
+    if (first_out) first_out[row] = plain ? first : -1;
+  }
 }
 
 // Merge the partitions of one query row: out = sum_p 2^(m_p - M) o_p / sum_p 2^(m_p - M) l_p.
@@ -1062,16 +1125,21 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     p.part_o = static_cast<float*>(a->workspace);
     p.part_ml = p.part_o + rows_total * max_parts * pool->head_dim;
   }
-  p.row_last = nullptr;
+  p.row_last = nullptr, p.row_first = nullptr;
   int32_t* row_last = nullptr;
+  int32_t* row_first = nullptr;
   if (a->mask && rows > 64) {
-    // room behind the partials for one int per (sequence, query token)?  (pace_paged_attn_workspace_bytes*
+    // room behind the partials for the per-row summary, one int per (sequence, query token)?  (pace_paged_attn_workspace_bytes*
     // asks for it; a caller that sized its workspace otherwise simply goes without)
     const size_t part_bytes = max_parts > 1 ? (size_t)a->batch * a->num_q_heads * a->q_len * max_parts * (pool->head_dim + 2) * sizeof(float) : 0;
     const size_t at = (part_bytes + 15) & ~(size_t)15;
-    if (a->workspace && aligned16(a->workspace) && a->workspace_bytes >= at + (size_t)a->batch * a->q_len * sizeof(int32_t))
+    const size_t per_array = (size_t)a->batch * a->q_len * sizeof(int32_t);
+    if (a->workspace && aligned16(a->workspace) && a->workspace_bytes >= at + per_array)
       row_last = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + at);
     p.row_last = row_last;
+    // and for a second one: the first column of the rows whose mask line is plain (the cooperative kernel's fast walk)
+    if (row_last && prefill_nqt && a->workspace_bytes >= at + 2 * per_array) row_first = row_last + (size_t)a->batch * a->q_len;
+    p.row_first = row_first;
   }
   p.num_kv_heads = pool->num_kv_heads;
   p.items = nullptr;
@@ -1087,7 +1155,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
   const bool has_mask = a->mask != nullptr;
   if (row_last && !g_name_out) {
     PACE_REQUIRE((long long)a->batch * a->q_len < (1ll << 31), "%s: too many query rows", who);
-    hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last);
+    hipLaunchKernelGGL(mask_row_last_kernel, dim3((unsigned)(a->batch * a->q_len)), dim3(64), 0, s, p, row_last, row_first);
     PACE_HIP_CHECK(hipGetLastError());
   }
   bool ok = false;
@@ -1129,11 +1197,11 @@ extern "C" int32_t pace_paged_attn_partition_tokens(int32_t batch, int32_t num_q
 }
 
 // Partials of every (row, partition) when a sequence is cut into several partitions, then (16-byte
-// aligned) one int per (sequence, query token) for launches of more than 64 query rows per KV head:
-// the per-row summary of an explicit mask (mask_row_last_kernel).
+// aligned) two ints per (sequence, query token) for launches of more than 64 query rows per KV head:
+// the per-row summary of an explicit mask (mask_row_last_kernel: last column, first column of a plain line).
 static size_t workspace_need(int batch, int num_q_heads, int q_len, int head_dim, int max_parts, int rows) {
   size_t need = max_parts > 1 ? (size_t)batch * num_q_heads * q_len * max_parts * (head_dim + 2) * sizeof(float) : 0;
-  if (rows > 64) need = ((need + 15) & ~(size_t)15) + (size_t)batch * q_len * sizeof(int32_t);
+  if (rows > 64) need = ((need + 15) & ~(size_t)15) + 2 * (size_t)batch * q_len * sizeof(int32_t);
   return need;
 }
 

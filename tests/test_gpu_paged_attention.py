@@ -450,6 +450,10 @@ def test_cooperative_prefill_kernel_with_a_mask_tensor(device, mask_dtype):
     L = max(lens)
     mask = lengths_mask_4d(lens, S, L, mask_dtype).clone()
     mask[0, :, 5, :] = torch.finfo(mask_dtype).min  # a row with nothing to read, in the sequence that fills the mask
+    # most lines are plain (0 over one stretch of columns: walked without reading the mask); these are not
+    mask[5, :, :, 3:17] -= 1.5                       # finite values that are not 0
+    mask[6, :, :, 10] = torch.finfo(mask_dtype).min  # a masked column inside the stretch
+    mask[7, :, 40:, :4] = torch.finfo(mask_dtype).min  # rows of one row group that start at different columns
     md = mask.to(device)
     if mask_dtype == torch.bfloat16:
         assert "paged_prefill_kernel<128, 2, false, true>" in _kernel_of(cache, qd, lens, md)
