@@ -328,9 +328,11 @@ int pace_paged_attn_kernel_name(const pace_kv_pool_t* pool, const pace_paged_att
 
 /* Scratch bytes the two entry points below need for these sizes (0 = none): the partial results
  * of sequences cut into several partitions and, for launches of more than 64 query rows per KV
- * head, one int32 per (sequence, query token) in which a launch with an explicit mask keeps a
- * summary of the mask (the last column each row can use).  The partials are required; a workspace
- * without room for the summary is accepted and the launch simply walks every column. */
+ * head, two int32 per (sequence, query token) in which a launch with an explicit mask keeps a
+ * summary of the mask (the last column each row can use; the first one, if the row's mask line is
+ * 0 over one stretch of columns and at the floor elsewhere).  The partials are required; a
+ * workspace without room for the summary is accepted: the launch then walks every column (no room
+ * for the first int) or reads the mask values of every unit (no room for the second). */
 size_t pace_paged_attn_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t q_len,
                                        int32_t head_dim, int32_t max_seq_len,
                                        int32_t partition_tokens, int32_t num_kv_heads);
