@@ -186,6 +186,55 @@ __device__ __forceinline__ void load_mask_regs(MaskRegs<NQT>& mr, const PagedAtt
   }
 }
 
+// One wave looks over the columns [start, end) of a mask line (element offset `off` in `mask`): `last` = the last
+// column whose value is above the floor (-1: none; NaN counts as masked), `first_if_plain` = the first such column
+// if the line is plain -- exactly 0 on every column from there to `last`, which then are all above the floor -- and
+// -1 if it is anything else.  Both are the same in every lane on return.
+__device__ __forceinline__ void mask_line_summary(const void* mask, bool is_f32, int64_t off, int start, int end, int lane,
+                                                  int& last_out, int& first_if_plain) {
+  int last = -1, first = 0x7fffffff, above = 0;
+  bool zero = true;  // every value above the floor is 0
+  for (int c0 = start + 8 * lane; c0 < end; c0 += 8 * 64) {
+    float a[8];
+    if (c0 + 8 <= end) {
+      if (is_f32) {
+        const float* line = static_cast<const float*>(mask) + off + c0;
+        const u32x4 lo = load16_unaligned(line), hi = load16_unaligned(line + 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] = __uint_as_float(lo[c]), a[4 + c] = __uint_as_float(hi[c]);
+      } else {
+        const u32x4 raw = load16_unaligned(static_cast<const uint16_t*>(mask) + off + c0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[2 * e] = bf16_bits_to_f32(raw[e] & 0xffffu), a[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        a[c] = kNegInf;
+        if (c0 + c < end)
+          a[c] = is_f32 ? static_cast<const float*>(mask)[off + c0 + c] : bf16_bits_to_f32(static_cast<const uint16_t*>(mask)[off + c0 + c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (a[c] > kMaskFloor) {  // ascending: the largest column wins
+        last = c0 + c;
+        first = min(first, c0 + c);
+        above += 1;
+        zero = zero && a[c] == 0.f;
+      }
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o *= 2) {
+    last = max(last, __shfl_xor(last, o, 64));
+    first = min(first, __shfl_xor(first, o, 64));
+    above += __shfl_xor(above, o, 64);
+  }
+  const bool plain = __all(zero) && last >= 0 && above == last - first + 1;
+  last_out = last;
+  first_if_plain = plain ? first : -1;
+}
+
 // A unit can be left out altogether when it cannot change any row of the wave: every mask value
 // in it is at the floor (weight exactly 0 next to any real score) and every row has already met a
 // real score -- the upper triangle of a causal mask, which is half of a prefill.  Rows that have

@@ -35,8 +35,11 @@ int check_pool(const pace_kv_pool_t* pool, const char* who);
 int compute_units();  // of the current device
 
 // Dense bf16 attention on the matrix cores (dense_attn_mfma.hip); false = shape not handled, nothing launched.
+// workspace (optional): room for the summary of an explicit mask (dense_mfma_workspace_bytes).
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
-                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream);
+                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, void* workspace,
+                       size_t workspace_bytes, hipStream_t stream);
+size_t dense_mfma_workspace_bytes(int S, int H, int mB, int mN, int mS, bool has_mask);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -232,28 +232,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 
 using namespace pace_kv;
 
+extern "C" size_t pace_attn_dense_workspace_bytes(int32_t qkv_dtype, int32_t S, int32_t H, int32_t has_mask, int32_t mB, int32_t mN,
+                                                  int32_t mS) {
+  if (qkv_dtype != PACE_DTYPE_BF16 || S <= 0 || H <= 0 || mB <= 0 || mN <= 0 || mS <= 0) return 0;
+  return dense_mfma_workspace_bytes(S, H, mB, mN, mS, has_mask != 0);
+}
+
 extern "C" int pace_attn_dense(const void* q, const void* k, const void* v, void* out, int32_t qkv_dtype, int32_t B,
                                int32_t N, int32_t S, int32_t L, int32_t H, const void* mask, int32_t mask_dtype,
                                int32_t mB, int32_t mN, int32_t mS, void* stream) {
-  PACE_REQUIRE(qkv_dtype == PACE_DTYPE_F32 || qkv_dtype == PACE_DTYPE_BF16, "pace_attn_dense: bad qkv dtype %d", qkv_dtype);
-  PACE_REQUIRE(B >= 0 && N >= 0 && S >= 0 && L >= 0 && H >= 1, "pace_attn_dense: negative extent");
+  return pace_attn_dense_ws(q, k, v, out, qkv_dtype, B, N, S, L, H, mask, mask_dtype, mB, mN, mS, nullptr, 0, stream);
+}
+
+extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, void* out, int32_t qkv_dtype, int32_t B,
+                                  int32_t N, int32_t S, int32_t L, int32_t H, const void* mask, int32_t mask_dtype,
+                                  int32_t mB, int32_t mN, int32_t mS, void* workspace, size_t workspace_bytes, void* stream) {
+  PACE_REQUIRE(qkv_dtype == PACE_DTYPE_F32 || qkv_dtype == PACE_DTYPE_BF16, "pace_attn_dense*: bad qkv dtype %d", qkv_dtype);
+  PACE_REQUIRE(B >= 0 && N >= 0 && S >= 0 && L >= 0 && H >= 1, "pace_attn_dense*: negative extent");
   if (B == 0 || N == 0 || S == 0) return PACE_KV_OK;
-  PACE_REQUIRE(L >= 1, "pace_attn_dense: empty key/value length");
-  PACE_REQUIRE(H <= 256, "pace_attn_dense: head_dim %d unsupported (max 256)", H);
-  PACE_REQUIRE(q && k && v && out, "pace_attn_dense: NULL tensor pointer");
+  PACE_REQUIRE(L >= 1, "pace_attn_dense*: empty key/value length");
+  PACE_REQUIRE(H <= 256, "pace_attn_dense*: head_dim %d unsupported (max 256)", H);
+  PACE_REQUIRE(q && k && v && out, "pace_attn_dense*: NULL tensor pointer");
   if (mask) {
-    PACE_REQUIRE(mask_dtype == PACE_DTYPE_F32 || mask_dtype == PACE_DTYPE_BF16, "pace_attn_dense: bad mask dtype %d",
+    PACE_REQUIRE(mask_dtype == PACE_DTYPE_F32 || mask_dtype == PACE_DTYPE_BF16, "pace_attn_dense*: bad mask dtype %d",
                  mask_dtype);
     PACE_REQUIRE((mB == 1 || mB == B) && (mN == 1 || mN == N) && (mS == 1 || mS == S),
-                 "pace_attn_dense: mask dims [%d][%d][%d] not broadcastable to [%d][%d][%d]", mB, mN, mS, B, N, S);
+                 "pace_attn_dense*: mask dims [%d][%d][%d] not broadcastable to [%d][%d][%d]", mB, mN, mS, B, N, S);
   }
-  PACE_REQUIRE(B <= 65535 && N <= 65535, "pace_attn_dense: batch / heads exceed grid limits");
+  PACE_REQUIRE(B <= 65535 && N <= 65535, "pace_attn_dense*: batch / heads exceed grid limits");
   hipStream_t s = static_cast<hipStream_t>(stream);
   // bf16 with head_dim 64 / 96 / 128 / 256 runs on the bf16 matrix-core kernels; everything else (fp32,
   // other head sizes) takes the general kernel below.
   if (qkv_dtype == PACE_DTYPE_BF16 &&
       launch_dense_mfma(q, k, v, out, B, N, S, L, H, mask, mask_dtype == PACE_DTYPE_F32, mB, mN, mS,
-                        1.0f / sqrtf((float)H), s)) {
+                        1.0f / sqrtf((float)H), workspace, workspace_bytes, s)) {
     PACE_HIP_CHECK(hipGetLastError());
     return PACE_KV_OK;
   }

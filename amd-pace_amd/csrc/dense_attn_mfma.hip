@@ -20,7 +20,19 @@ struct DenseMfmaParams {
   int32_t B, N, S, L;
   int32_t mB, mN, mS;
   int32_t n_qgroups;
+  // Optional summary of the mask, one entry per mask line ((mb * mN + mn) * mS + ms), written by
+  // dense_mask_lines_kernel just before the attention launch: the last column above the floor (-1: none) and the
+  // first one if the line is plain (see mask_line_summary), else -1.
+  const int32_t* line_last;
+  const int32_t* line_first;
 };
+
+// One wave per mask line.
+__global__ __launch_bounds__(64) void dense_mask_lines_kernel(const void* mask, int is_f32, int L, int32_t* last_out, int32_t* first_out) {
+  int last, first;
+  mask_line_summary(mask, is_f32 != 0, (int64_t)blockIdx.x * L, 0, L, threadIdx.x, last, first);
+  if (threadIdx.x == 0) last_out[blockIdx.x] = last, first_out[blockIdx.x] = first;
+}
 
 // ONCE: one group of query rows per (batch, head), so K / V are read once and fetched non-temporally.
 // Waves per workgroup: four; two with head_dim 256, where a wave has a SIMD (and its 512 registers) to itself
@@ -253,7 +265,8 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   u32x4 pre_k[PER_THREAD], pre_v[PER_THREAD];
   u32x4 pre_m[MASK == 2 ? NQT : 1], cur_m[MASK == 2 ? NQT : 1];  // raw bf16 mask values (MASK == 2)
   MaskRegs<NQT> mnext, mcur;                                      // fp32 values (MASK == 1)
-  auto fetch = [&](int u) {
+  auto fetch = [&](int u, auto with_mask) {
+    constexpr int MODE = decltype(with_mask)::value ? MASK : 0;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
@@ -261,7 +274,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       pre_k[i] = *reinterpret_cast<const u32x4*>(kbase + off);
       pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
     }
-    if (MASK == 2) {
+    if (MODE == 2) {
       const int tok = 32 * u + 8 * g;
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) {
@@ -276,7 +289,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
           }
         }
       }
-    } else if (MASK == 1) {
+    } else if (MODE == 1) {
       const int tok = 32 * u + 8 * g;
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt)
@@ -293,17 +306,18 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
         }
     }
   };
-  auto park = [&](int buf) {
+  auto park = [&](int buf, auto with_mask) {
+    constexpr int MODE = decltype(with_mask)::value ? MASK : 0;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
       *reinterpret_cast<u32x4*>(&stage[buf][r * KROW + (r >= 16 ? KHALF : 0) + ch * 8]) = pre_k[i];
       *reinterpret_cast<u32x4*>(&stage[buf][KSTAGE + r * VROW + ch * 8]) = pre_v[i];
     }
-    if (MASK == 2) {
+    if (MODE == 2) {
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) cur_m[qt] = pre_m[qt];
-    } else if (MASK == 1) {
+    } else if (MODE == 1) {
       mcur = mnext;
     }
   };
@@ -318,13 +332,16 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // queued behind the accumulator of the instruction before it fetches its A / B operands late) is a
   // write-after-read hazard that neither the hardware nor the compiler's wait-state insertion covers; with
   // the two operand sets disjoint inside a unit, and a workgroup barrier between units, it cannot occur.
-  auto unit = [&](int cur, int t0, auto full_tag) {
+  // by_mask: the unit's mask values decide (all of [0, L) is walked); else the rows' own limits and `first` do
+  // (plain mask lines, see below), and the mask values are not looked at.
+  auto unit = [&](int cur, int t0, auto full_tag, auto by_mask, int tok_end, int first) {
     constexpr bool FULL = decltype(full_tag)::value;
-    if (MASK == 2) {
+    constexpr bool BY_MASK = decltype(by_mask)::value && HAS_MASK;
+    if (BY_MASK && MASK == 2) {
 #pragma unroll
       for (int qt = 0; qt < NQT; ++qt) mask_line_from_bf16x8(cur_m[qt], mcur.a[qt]);
     }
-    if (HAS_MASK && unit_is_masked_out<D, NQT>(mcur, st)) return;  // e.g. above the diagonal of a causal mask
+    if (BY_MASK && unit_is_masked_out<D, NQT>(mcur, st)) return;  // e.g. above the diagonal of a causal mask
     u32x4 kop[2][KK], vop[MT];
     // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g ..
     const int r0 = 8 * (n >> 2) + (n & 3);
@@ -351,7 +368,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) asm volatile("" ::"v"(kop[t][kk]));  // K operands live up to here
     __builtin_amdgcn_sched_barrier(0);
-    softmax_and_output<D, NQT, HAS_MASK, FULL>(sc, vop, st, p, t0, L, 0, g, mcur);
+    softmax_and_output<D, NQT, BY_MASK, FULL>(sc, vop, st, p, t0, tok_end, first, g, mcur);
   };
   // Units past the last one that matters to any row of the workgroup are not walked at all: with a
   // bf16 mask every wave first looks from the end of its rows' mask lines backwards for the last
@@ -359,8 +376,37 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // row that shows none (masked everywhere: it ends as the average of V) keeps every unit.  What lies
   // past the workgroup's last such unit weighs exactly 0 for rows that have all met a real score by
   // then: the upper triangle of a causal mask, half of a prefill.
+  // Summary of the mask (optional): per mask line the last column above the floor and, if the line is plain (0 from
+  // a first column to that last one, at the floor elsewhere: a causal mask, padded or not), the first one.  When every
+  // row of the workgroup has a plain line and all start at the same column, the rows are walked like rows without a
+  // mask tensor -- that first column, their own last column -- and the mask is not read (`plain`).
+  bool plain = false;
+  int f_min = 0x7fffffff, f_max = -1, wg_last = -1, l_min = 0x7fffffff;
+  const bool summarised = HAS_MASK && dp.line_last && dp.line_first;
+  const int64_t line0 = ((dp.mB == 1 ? 0 : (int64_t)b) * dp.mN + (dp.mN == 1 ? 0 : head)) * dp.mS;
+  if (summarised) {
+#pragma unroll
+    for (int i = 0; i < NQT; ++i) {
+      const int r = rg * (kCoopWaves * NQT * 16) + i * 64 + lane;
+      if (r < S) {
+        const int64_t line = line0 + (dp.mS == 1 ? 0 : r);
+        const int f = dp.line_first[line], l = dp.line_last[line];
+        f_min = min(f_min, f), f_max = max(f_max, f), wg_last = max(wg_last, l), l_min = min(l_min, l);
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o *= 2) {
+      f_min = min(f_min, __shfl_xor(f_min, o, 64)), f_max = max(f_max, __shfl_xor(f_max, o, 64));
+      wg_last = max(wg_last, __shfl_xor(wg_last, o, 64)), l_min = min(l_min, __shfl_xor(l_min, o, 64));
+    }
+    f_min = __builtin_amdgcn_readfirstlane(f_min), f_max = __builtin_amdgcn_readfirstlane(f_max);
+    wg_last = __builtin_amdgcn_readfirstlane(wg_last), l_min = __builtin_amdgcn_readfirstlane(l_min);
+    plain = f_min >= 0 && f_min == f_max;  // (-1 marks a line that is not plain)
+  }
   int units = (L + 31) / 32;
-  if (MASK == 2) {
+  if (summarised) {
+    if (l_min >= 0) units = min(units, wg_last / 32 + 1);  // every row has a real score: nothing past the last of them counts
+  } else if (MASK == 2) {
     __shared__ int last_needed[kCoopWaves];
     constexpr int ROUND = 4;  // units looked at per round trip (16 measured slower: the volume counts, not the trips)
     int mine = -1;            // last unit in which this lane's columns of a (real) row hold a value above the floor
@@ -418,21 +464,66 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     for (int w = 1; w < kCoopWaves; ++w) wg_last = max(wg_last, last_needed[w]);
     units = __builtin_amdgcn_readfirstlane(min(units, wg_last + 1));
   }
-  // Whole units in the loop, the partial last one (if any) after it: the loop body has one shape.
-  const int whole = min(L / 32, units);
-  fetch(0);
-  park(0);
-  __syncthreads();
-  for (int u = 0; u < whole; ++u) {
-    const int cur = u & 1;
-    fetch(min(u + 1, units - 1));  // unconditional: no branch between a load and the wait for it
-    if (wave_has_rows) {
-      unit(cur, 32 * u, std::true_type{});
+  // One loop per kind of unit -- masked before the rows' whole units, whole, masked after them, needed by other waves
+  // only -- so that the accumulators have one path through each loop body.
+  if (plain) {
+    {
+      int min_limit = 0x7fffffff, mine = -1;
+#pragma unroll
+      for (int qt = 0; qt < NQT; ++qt) {
+        if (st.limit[qt] >= 0) {
+          st.limit[qt] = dp.line_last[line0 + (dp.mS == 1 ? 0 : row_s[qt])];
+          min_limit = min(min_limit, st.limit[qt]);
+          mine = max(mine, st.limit[qt]);
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < 64; o *= 2) min_limit = min(min_limit, __shfl_xor(min_limit, o, 64)), mine = max(mine, __shfl_xor(mine, o, 64));
+      min_limit = __builtin_amdgcn_readfirstlane(min_limit);
+      const int first = f_min;
+      const int wave_end = wave_has_rows ? __builtin_amdgcn_readfirstlane(mine) + 1 : 0;
+      const int u0 = first / 32;
+      const int u_end = max(wg_last / 32 + 1, u0 + 1);  // (every line has a column: u_end > u0)
+      const int u_mine = min(max((wave_end + 31) / 32, u0), u_end);
+      const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
+      const int u_whole_begin = min((first + 31) / 32, u_whole_end);
+      fetch(u0, std::false_type{});
+      park(0, std::false_type{});
+      __syncthreads();
+      auto walk = [&](int from, int to, auto kind) {  // kind: 0 masked unit, 1 whole unit, 2 nothing to compute
+        constexpr int KIND = decltype(kind)::value;
+        for (int u = from; u < to; ++u) {
+          const int cur = (u - u0) & 1;
+          fetch(min(u + 1, u_end - 1), std::false_type{});
+          if (KIND == 0) unit(cur, 32 * u, std::false_type{}, std::false_type{}, wave_end, first);
+          if (KIND == 1) unit(cur, 32 * u, std::true_type{}, std::false_type{}, wave_end, first);
+          park(cur ^ 1, std::false_type{});
+          __syncthreads();
+        }
+      };
+      walk(u0, u_whole_begin, std::integral_constant<int, 0>{});
+      walk(u_whole_begin, u_whole_end, std::integral_constant<int, 1>{});
+      walk(u_whole_end, u_mine, std::integral_constant<int, 0>{});
+      walk(u_mine, u_end, std::integral_constant<int, 2>{});
     }
-    park(cur ^ 1);
-    __syncthreads();
   }
-  if (whole < units && wave_has_rows) unit(whole & 1, 32 * whole, std::false_type{});
+  if (!plain) {
+    // Whole units in the loop, the partial last one (if any) after it: the loop body has one shape.
+    const int whole = min(L / 32, units);
+    fetch(0, std::true_type{});
+    park(0, std::true_type{});
+    __syncthreads();
+    for (int u = 0; u < whole; ++u) {
+      const int cur = u & 1;
+      fetch(min(u + 1, units - 1), std::true_type{});  // unconditional: no branch between a load and the wait for it
+      if (wave_has_rows) {
+        unit(cur, 32 * u, std::true_type{}, std::true_type{}, L, 0);
+      }
+      park(cur ^ 1, std::true_type{});
+      __syncthreads();
+    }
+    if (whole < units && wave_has_rows) unit(whole & 1, 32 * whole, std::false_type{}, std::true_type{}, L, 0);
+  }
 
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
@@ -453,8 +544,10 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 }
 
 // Launches the dense bf16 kernel; returns false when the shape is not one it handles.
+// workspace (optional): room for the summary of the mask, two ints per mask line (dense_mfma_workspace_bytes).
 bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
-                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, hipStream_t stream) {
+                       const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, void* workspace,
+                       size_t workspace_bytes, hipStream_t stream) {
   if ((H != 64 && H != 96 && H != 128 && H != 256) || L < 1) return false;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(out) & 7u)) return false;
   DenseMfmaParams dp = {};
@@ -482,6 +575,13 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
     const long long cblocks = pairs8 * dp.n_qgroups;
     if (cblocks >= (1ll << 31)) return false;
     const dim3 cgrid((unsigned)cblocks), cblock(64 * kCoopWaves);
+    const size_t lines = mask ? (size_t)mB * mN * mS : 0;
+    if (mask && workspace && (reinterpret_cast<uintptr_t>(workspace) & 3u) == 0 && lines < (1u << 31) &&
+        workspace_bytes >= 2 * lines * sizeof(int32_t)) {
+      int32_t* last = static_cast<int32_t*>(workspace);
+      hipLaunchKernelGGL(dense_mask_lines_kernel, dim3((unsigned)lines), dim3(64), 0, stream, mask, mask_is_f32 ? 1 : 0, L, last, last + lines);
+      dp.line_last = last, dp.line_first = last + lines;
+    }
 #define PACE_COOP(D_, Q_, M_) hipLaunchKernelGGL((dense_attn_coop_kernel<D_, Q_, M_>), cgrid, cblock, 0, stream, dp)
 #define PACE_COOP_M(D_, Q_) \
   do { if (mode == 0) PACE_COOP(D_, Q_, 0); else if (mode == 1) PACE_COOP(D_, Q_, 1); else PACE_COOP(D_, Q_, 2); } while (0)
@@ -513,6 +613,14 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
 #undef PACE_DENSE1
 #undef PACE_DENSE
   return true;
+}
+
+// Scratch the dense bf16 path can use for these sizes (0: none): the summary of an explicit mask on prefill-sized
+// launches.
+size_t dense_mfma_workspace_bytes(int S, int H, int mB, int mN, int mS, bool has_mask) {
+  const int tiles = (S + 15) / 16;
+  if (!has_mask || tiles <= 4 || (H != 64 && H != 128)) return 0;
+  return 2 * (size_t)mB * mN * mS * sizeof(int32_t);
 }
 
 }  // namespace pace_kv

@@ -719,51 +719,11 @@ __global__ __launch_bounds__(64) void mask_row_last_kernel(const PagedAttnParams
   const int row = blockIdx.x, S = p.q_len, b = row / S, s = row % S, lane = threadIdx.x;
   const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
   const int start = p.kv_start ? p.kv_start[b] : 0;
-  const int end = min(len, p.mask_len);
-  const int64_t off = (int64_t)b * p.m_sb + (int64_t)s * p.m_ss;
-  int last = -1, first = 0x7fffffff, above = 0;
-  bool zero = true;  // every value above the floor is 0
-  for (int c0 = start + 8 * lane; c0 < end; c0 += 8 * 64) {
-    float a[8];
-    if (c0 + 8 <= end) {
-      if (p.mask_is_f32) {
-        const float* line = static_cast<const float*>(p.mask) + off + c0;
-        const u32x4 lo = load16_unaligned(line), hi = load16_unaligned(line + 4);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) a[c] = __uint_as_float(lo[c]), a[4 + c] = __uint_as_float(hi[c]);
-      } else {
-        const u32x4 raw = load16_unaligned(static_cast<const uint16_t*>(p.mask) + off + c0);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) a[2 * e] = bf16_bits_to_f32(raw[e] & 0xffffu), a[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        a[c] = kNegInf;
-        if (c0 + c < end)
-          a[c] = p.mask_is_f32 ? static_cast<const float*>(p.mask)[off + c0 + c]
-                               : bf16_bits_to_f32(static_cast<const uint16_t*>(p.mask)[off + c0 + c]);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < 8; ++c)
-      if (a[c] > kMaskFloor) {  // ascending: the largest column wins (NaN compares false: treated as masked)
-        last = c0 + c;
-        first = min(first, c0 + c);
-        above += 1;
-        zero = zero && a[c] == 0.f;
-      }
-  }
-#pragma unroll
-  for (int o = 1; o < 64; o *= 2) {
-    last = max(last, __shfl_xor(last, o, 64));
-    first = min(first, __shfl_xor(first, o, 64));
-    above += __shfl_xor(above, o, 64);
-  }
-  const bool plain = __all(zero) && last >= 0 && above == last - first + 1;
+  int last, first;
+  mask_line_summary(p.mask, p.mask_is_f32 != 0, (int64_t)b * p.m_sb + (int64_t)s * p.m_ss, start, min(len, p.mask_len), lane, last, first);
   if (lane == 0) {
     out[row] = last;
-    if (first_out) first_out[row] = plain ? first : -1;
+    if (first_out) first_out[row] = first;
   }
 }
 

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 10
+ABI_VERSION = 11
 STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
@@ -40,6 +40,8 @@ EXPORTED_SYMBOLS = (
     "pace_paged_attn_verify",
     "pace_paged_attn_verify_static",
     "pace_attn_dense",
+    "pace_attn_dense_ws",
+    "pace_attn_dense_workspace_bytes",
 )
 
 
@@ -217,6 +219,13 @@ def load() -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
     ]
+    lib.pace_attn_dense_ws.restype = ctypes.c_int
+    lib.pace_attn_dense_ws.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+        c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, ctypes.c_size_t, c_void_p,
+    ]
+    lib.pace_attn_dense_workspace_bytes.restype = ctypes.c_size_t
+    lib.pace_attn_dense_workspace_bytes.argtypes = [c_int32] * 7
     got = int(lib.pace_kv_abi_version())
     if got != ABI_VERSION:
         raise ImportError(f"{_LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")

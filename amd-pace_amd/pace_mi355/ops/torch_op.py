@@ -61,10 +61,15 @@ def _attention(input_Q, input_K, input_V, input_mask: Optional[torch.Tensor] = N
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     dt = nat.DTYPE_F32 if q.dtype == torch.float32 else nat.DTYPE_BF16
     mdt = nat.DTYPE_F32 if m.dtype == torch.float32 else nat.DTYPE_BF16
+    lib = nat.load()
+    # scratch for the library's look over the mask (prefill-sized bf16 calls; 0 bytes otherwise)
+    ws_bytes = int(lib.pace_attn_dense_workspace_bytes(dt, S, H, 1, m.shape[0], m.shape[1], m.shape[2]))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     nat.check(
-        nat.load().pace_attn_dense(
+        lib.pace_attn_dense_ws(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dt, B, N, S, L, H,
-            m.data_ptr(), mdt, m.shape[0], m.shape[1], m.shape[2], nat.current_stream_ptr(),
+            m.data_ptr(), mdt, m.shape[0], m.shape[1], m.shape[2],
+            ws.data_ptr() if ws is not None else None, ws_bytes, nat.current_stream_ptr(),
         )
     )
     return out

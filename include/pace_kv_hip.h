@@ -385,6 +385,22 @@ int pace_attn_dense(const void* q, const void* k, const void* v, void* out,
                     const void* mask, int32_t mask_dtype, int32_t mB, int32_t mN, int32_t mS,
                     void* stream);
 
+/*
+ * The same op (csrc/ops/attention.cpp:18-108) with scratch memory of the caller's: `workspace` (4-byte
+ * aligned, pace_attn_dense_workspace_bytes() of these sizes, device memory) lets a prefill-sized bf16 launch
+ * with a mask look over the mask once before the attention kernel -- where its lines are 0 over one stretch
+ * of columns and at the floor elsewhere (a causal mask, padded or not) the rows are then walked by that
+ * stretch and the mask is not read again.  Results are the same up to rounding (the weights of such rows
+ * are formed as exp2((qk - max) * scale * log2 e) instead of exp2((qk * scale + 0 - max) * log2 e)).
+ * A NULL or short workspace is accepted: the call is then pace_attn_dense.
+ */
+size_t pace_attn_dense_workspace_bytes(int32_t qkv_dtype, int32_t S, int32_t H, int32_t has_mask,
+                                       int32_t mB, int32_t mN, int32_t mS);
+int pace_attn_dense_ws(const void* q, const void* k, const void* v, void* out,
+                       int32_t qkv_dtype, int32_t B, int32_t N, int32_t S, int32_t L, int32_t H,
+                       const void* mask, int32_t mask_dtype, int32_t mB, int32_t mN, int32_t mS,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -201,3 +201,13 @@ def test_dense_prefill_is_bit_identical_from_call_to_call(device):
         out = torch.ops.pace.attention(qd, kd, vd, md, 0)
         differing += int(not torch.equal(out.view(torch.int16), first.view(torch.int16)))
     assert differing == 0
+    # the same through the walk that plain mask lines take (a causal mask: the mask values are not read)
+    causal = torch.zeros(B, 1, S, L, dtype=torch.bfloat16).masked_fill(
+        torch.arange(L)[None, :] > torch.arange(S)[:, None] // 4, torch.finfo(torch.bfloat16).min)
+    cd = causal.to(device)
+    first = torch.ops.pace.attention(qd, kd, vd, cd, 0)
+    assert_attention_close(first, sdpa_fp32(q, k, v, causal), "prefill, causal mask")
+    for _ in range(1000):
+        out = torch.ops.pace.attention(qd, kd, vd, cd, 0)
+        differing += int(not torch.equal(out.view(torch.int16), first.view(torch.int16)))
+    assert differing == 0

@@ -463,6 +463,31 @@ def test_cooperative_prefill_kernel_with_a_mask_tensor(device, mask_dtype):
     assert_attention_close(out, ref, f"cooperative prefill with a {mask_dtype} mask")
 
 
+@pytest.mark.parametrize("masked", [False, True])
+def test_cooperative_prefill_kernel_gives_the_same_bits_every_call(device, masked):
+    """Operands come out of LDS into registers that matrix instructions of the unit before were issued from, and
+    the stage a unit is read from is refilled by loads that bypass the registers: every call must give the same
+    bits (a barrier per unit and the waits before it are what orders the two)."""
+    B, hkv, n_rep, D, S = 16, 8, 4, 128, 64
+    rng = np.random.default_rng(17)
+    lens = (rng.integers(S, 400, B)).tolist()
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=93)
+    q = seeded_q(35, B, hkv * n_rep, S, D)
+    qd = q.to(device)
+    md = None
+    if masked:  # values that have to be read (not a plain causal mask)
+        mask = lengths_mask_4d(lens, S, max(lens), torch.bfloat16).clone()
+        mask[:, :, :, 1:9] -= 0.75
+        md = mask.to(device)
+    assert "paged_prefill_kernel" in _kernel_of(cache, qd, lens, md)
+    first = cache.attend(qd, attention_mask=md)
+    differing = 0
+    for _ in range(1000):
+        out = cache.attend(qd, attention_mask=md)
+        differing += int(not torch.equal(out.view(torch.int16), first.view(torch.int16)))
+    assert differing == 0
+
+
 def test_prefill_sized_launch_with_rope_rotates_queries(device):
     from oracle import rope_ref
     from pace_mi355.llm import PagedKVCache
