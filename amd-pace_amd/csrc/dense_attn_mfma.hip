@@ -487,17 +487,21 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const int u_mine = min(max((wave_end + 31) / 32, u0), u_end);
       const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
       const int u_whole_begin = min((first + 31) / 32, u_whole_end);
+      // A unit is parked in LDS a whole turn before it is read: turn u parks unit u + 1 (fetched during turn u - 1)
+      // into the stage unit u - 1 was read from, fetches unit u + 2 into the registers that freed, and then works on
+      // unit u; the barrier at its end finds the next unit long written.
       fetch(u0, std::false_type{});
       park(0, std::false_type{});
+      fetch(min(u0 + 1, u_end - 1), std::false_type{});
       __syncthreads();
       auto walk = [&](int from, int to, auto kind) {  // kind: 0 masked unit, 1 whole unit, 2 nothing to compute
         constexpr int KIND = decltype(kind)::value;
         for (int u = from; u < to; ++u) {
           const int cur = (u - u0) & 1;
-          fetch(min(u + 1, u_end - 1), std::false_type{});
+          park(cur ^ 1, std::false_type{});
+          fetch(min(u + 2, u_end - 1), std::false_type{});
           if (KIND == 0) unit(cur, 32 * u, std::false_type{}, std::false_type{}, wave_end, first);
           if (KIND == 1) unit(cur, 32 * u, std::true_type{}, std::false_type{}, wave_end, first);
-          park(cur ^ 1, std::false_type{});
           __syncthreads();
         }
       };
