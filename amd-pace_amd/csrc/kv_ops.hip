@@ -469,3 +469,32 @@ extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool
   PACE_HIP_CHECK(hipGetLastError());
   return PACE_KV_OK;
 }
+
+extern "C" int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, int32_t n_pools, const int32_t* block_table,
+                                          int32_t table_stride, const int64_t* n_blocks, int32_t batch, int32_t* moves_host,
+                                          int32_t capacity, int32_t* moves_dev, void* stream) {
+  const char* who = "pace_kv_compact_blocks";
+  if (!pools || n_pools < 1 || !moves_host || !moves_dev) {
+    set_error("%s: NULL pools / moves_host / moves_dev or no pool", who);
+    return PACE_KV_EINVAL;
+  }
+  for (int i = 0; i < n_pools; ++i) {
+    if (int rc = check_pool(pools[i], who)) return rc;
+    if (pools[i]->num_blocks != pools[0]->num_blocks) {
+      set_error("%s: pools of one table must have the same number of blocks", who);
+      return PACE_KV_EINVAL;
+    }
+  }
+  // the plan reads the table only (apply = 0): the caller rewrites it with pace_kv_apply_moves while the copies run
+  const int32_t n = pace_kv_plan_compaction(const_cast<int32_t*>(block_table), table_stride, n_blocks, batch, pools[0]->num_blocks,
+                                            moves_host, capacity, 0, nullptr);
+  if (n <= 0) return n;
+  if (hipMemcpyAsync(moves_dev, moves_host, (size_t)n * 2 * sizeof(int32_t), hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)) !=
+      hipSuccess) {
+    set_error("%s: upload of the moves failed: %s", who, hipGetErrorString(hipGetLastError()));
+    return PACE_KV_EHIP;
+  }
+  for (int i = 0; i < n_pools; ++i)
+    if (int rc = pace_kv_copy_blocks(pools[i], pools[i], moves_dev, n, stream)) return rc;
+  return n;
+}

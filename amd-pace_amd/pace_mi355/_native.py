@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "pace_paged_attn_decode",
     "pace_paged_attn_verify",
     "pace_paged_attn_verify_static",
+    "pace_kv_compact_blocks",
     "pace_attn_dense",
     "pace_attn_dense_ws",
     "pace_attn_dense_workspace_bytes",
@@ -219,6 +220,8 @@ def load() -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
     ]
+    lib.pace_kv_compact_blocks.restype = c_int32
+    lib.pace_kv_compact_blocks.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.pace_attn_dense_ws.restype = ctypes.c_int
     lib.pace_attn_dense_ws.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,

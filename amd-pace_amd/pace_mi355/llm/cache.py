@@ -383,13 +383,9 @@ class PagedKVCache(KVCacheBase):
         for p in self._shared.get("layers", [self]):
             if p.pool is not None:
                 p._flush()
-        moves = self.state.plan_compaction()
+        # one library call plans the moves, uploads them and starts the copies of every layer's pool
+        moves = self.state.compact_blocks([self._describe(pool) for pool in self.state.pools])
         if len(moves):
-            pairs = self.state.upload_pairs(moves)
-            lib = nat.load()
-            for pool in self.state.pools:
-                desc = self._describe(pool)
-                nat.check(lib.pace_kv_copy_blocks(ctypes.byref(desc), ctypes.byref(desc), pairs.data_ptr(), len(moves), nat.current_stream_ptr()))
             self.state.apply_moves(moves)  # the table rewrite runs on the host while the GPU copies
         return len(moves)
 

@@ -140,6 +140,7 @@ class PagedState:
         self._pairs_host: Optional[torch.Tensor] = None
         self._pairs_dev: Optional[torch.Tensor] = None
         self._pairs_copied = None
+        self._pairs_event = None
         self._n_items, self._max_parts, self._plan_ws = 0, 1, 0
 
     # -- capacity ---------------------------------------------------------------
@@ -331,6 +332,31 @@ class PagedState:
         self._pairs_copied = torch.cuda.Event()
         self._pairs_copied.record()
         return self._pairs_dev[:n]
+
+    def compact_blocks(self, descs) -> np.ndarray:
+        """Plan the compaction, upload its moves and start the block copies of every pool in ``descs`` (pool
+        descriptors that share this table) with one library call; returns the moves ``[n][2]`` (a view of the pinned
+        staging buffer: valid until the next upload).  The table is not rewritten here: ``apply_moves`` does
+        that on the host while the copies run."""
+        cap = self.allocator.num_blocks
+        if self._pairs_host is None or self._pairs_host.shape[0] < cap:
+            self._pairs_copied = None
+            self._pairs_host = torch.empty((cap, 2), dtype=torch.int32, pin_memory=True)
+            self._pairs_dev = torch.empty((cap, 2), dtype=torch.int32, device=self.device)
+        if self._pairs_copied is not None:
+            self._pairs_copied.synchronize()  # the upload before this one has read the staging buffer
+        ptrs = (ctypes.c_void_p * len(descs))(*[ctypes.addressof(d) for d in descs])
+        n = int(nat.load().pace_kv_compact_blocks(
+            ptrs, len(descs), self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch,
+            self._pairs_host.data_ptr(), cap, self._pairs_dev.data_ptr(), nat.current_stream_ptr()))
+        if n < 0:
+            nat.check(n)
+        if n:
+            if self._pairs_event is None:
+                self._pairs_event = torch.cuda.Event()
+            self._pairs_event.record()
+            self._pairs_copied = self._pairs_event
+        return self._pairs_host.numpy()[:n]
 
     def workspace(self, nbytes: int) -> Optional[torch.Tensor]:
         if nbytes == 0:

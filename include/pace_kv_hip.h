@@ -155,6 +155,19 @@ int pace_kv_apply_moves(int32_t* block_table, int32_t table_stride, const int64_
                         int32_t num_blocks, const int32_t* moves, int32_t n_moves, int32_t* refs);
 
 /*
+ * Compaction in one call: pace_kv_plan_compaction (apply = 0) into moves_host [capacity][2], the upload of the
+ * moves to moves_dev (device memory for as many pairs) and pace_kv_copy_blocks for each of the n_pools pools that
+ * share the table (the layers of a model), all on `stream`.  Returns the number of moves or a negative code.
+ * Afterwards the caller rewrites its table with pace_kv_apply_moves(moves_host, returned count) -- on the host,
+ * while the copies run.  moves_host should be pinned memory (else the upload waits for the stream) and must stay
+ * untouched until the upload has run.  Like compaction as a whole, this has no counterpart in the reference, whose
+ * caches are dense tensors (pace/llm/cache.py:161-167 is its only copy between cache rows).
+ */
+int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, int32_t n_pools, const int32_t* block_table,
+                               int32_t table_stride, const int64_t* n_blocks, int32_t batch, int32_t* moves_host,
+                               int32_t capacity, int32_t* moves_dev, void* stream);
+
+/*
  * Rotary position embedding, the step the models run on q and k right before the
  * append (pace/llm/models/llama.py:147-158; operator pace/ops/rotary_embedding.py:370-474).
  * cos / sin: device tables [table_rows][rotary_dim/2] as RotaryEmbedding builds them
