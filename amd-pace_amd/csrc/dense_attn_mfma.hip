@@ -204,6 +204,87 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
 // ---------------------------------------------------------------------------------
 constexpr int kCoopWaves = 4;
 
+// One turn of the walk that keeps its units in LDS by direct loads (dense_attn_coop_kernel, plain mask lines): send
+// this wave's share of a coming unit into stage `nxt` and take the operands of the unit at hand out of stage `cur`
+// (K in operand order, V row-major with swizzled 32-byte pieces through the transposing read), with the score
+// products between the K and the V reads.
+// The LDS reads are written as instructions, with their own wait: before an LDS read the compiler sees, it waits for
+// every outstanding direct-to-LDS load (it cannot tell that the read does not touch what they write) -- the full
+// memory latency of the unit just sent, every turn (measured: more than half of the wave cycles).  The reads here
+// are of a stage whose loads the caller has waited for (vmcnt, barrier), the loads in flight write other stages.
+struct CoopSend {
+  const uint16_t* kp;   // this lane's K piece of the coming unit (second load: 64 bytes on)
+  const uint16_t* vp;   // this lane's V piece (second load: four rows on, or vp2 where rows are clamped)
+  const uint16_t* vp2;
+  bool on, whole;       // wave-uniform
+};
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+template <int D, int NQT>
+__device__ __forceinline__ void coop_stage_turn(const u32x4* cur, u32x4* nxt, const CoopSend& sd, int k_first, int lane, int v_at,
+                                                const u32x4 (&qreg)[NQT][D / 32], f32x4 (&sc)[NQT][2], u32x4 (&vop)[D / 16]) {
+  constexpr int KK = D / 32, MT = D / 16, PER = MT / kCoopWaves, ROW_BYTES = D * 2;
+  typedef const __attribute__((address_space(1))) void* gptr;
+  typedef __attribute__((address_space(3))) void* lptr;
+  static_assert(PER == 1 || PER == 2, "one or two loads per operand and wave");
+  static_assert(KK == 2 || KK == 4, "head_dim 64 or 128");
+  if (sd.on) {
+    u32x4* const ks = nxt + k_first * 64;
+    __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 0, 0);
+    // (the immediate offset moves the address in memory and the one in LDS alike: 64 bytes on in the row, 1024 in the stage)
+    if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)(ks + 60), 16, 64, 0);
+    u32x4* const vs = nxt + (MT + k_first) * 64;
+    __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 0, 0);
+    if (PER == 2) {
+      if (sd.whole) {  // four rows on: 1024 bytes in memory and in the stage, the same swizzle
+        __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 4 * ROW_BYTES, 0);
+      } else {
+        __builtin_amdgcn_global_load_lds((gptr)sd.vp2, (lptr)(vs + 64), 16, 0, 0);
+      }
+    }
+  }
+  u32x4 kop[2][KK];
+  const uint32_t k_at = lds_address(cur) + lane * 16;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kop[t][kk]) : "v"(k_at), "n"((t * KK + kk) * 1024) : "memory");
+  if constexpr (KK == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(kop[0][0]), "+v"(kop[0][1]), "+v"(kop[0][2]), "+v"(kop[0][3]), "+v"(kop[1][0]), "+v"(kop[1][1]), "+v"(kop[1][2]),
+                   "+v"(kop[1][3]));
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kop[0][0]), "+v"(kop[0][1]), "+v"(kop[1][0]), "+v"(kop[1][1]));
+  }
+  score_products<D, NQT>(kop, qreg, sc);
+  __builtin_amdgcn_sched_barrier(0);  // the products above are issued before any read below
+  const uint32_t v_base = lds_address(cur) + v_at;
+  u32x2 lo[MT], hi[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const uint32_t at = v_base ^ (j << 5);
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo[j]) : "v"(at) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi[j]) : "v"(at), "n"(4 * ROW_BYTES) : "memory");
+  }
+  if constexpr (MT == 8) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(lo[4]), "+v"(lo[5]), "+v"(lo[6]), "+v"(lo[7]), "+v"(hi[0]),
+                   "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]), "+v"(hi[4]), "+v"(hi[5]), "+v"(hi[6]), "+v"(hi[7]));
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
+  }
+#pragma unroll
+  for (int j = 0; j < MT; ++j) vop[j] = u32x4{lo[j][0], lo[j][1], hi[j][0], hi[j][1]};
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) asm volatile("" ::"v"(kop[t][kk]));  // K operands live up to here (see the kernel)
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int D, int NQT, int MASK>
 __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_coop_kernel(
     const DenseMfmaParams dp) {
@@ -218,7 +299,10 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   constexpr int PER_THREAD = 32 * CH / (64 * kCoopWaves);
   constexpr bool HAS_MASK = MASK != 0;
   static_assert(PER_THREAD >= 1 && (32 * CH) % (64 * kCoopWaves) == 0, "unit does not divide over the workgroup");
-  __shared__ __attribute__((aligned(16))) uint16_t stage[2][STAGE];
+  // (the walk over plain mask lines keeps three units of 2 * MT KiB in the same memory, see below)
+  constexpr int STAGE_ELEMS = 2 * STAGE > 3 * MT * 1024 ? 2 * STAGE : 3 * MT * 1024;
+  __shared__ __attribute__((aligned(256))) uint16_t stage_mem[STAGE_ELEMS];
+  uint16_t(*stage)[STAGE] = reinterpret_cast<uint16_t(*)[STAGE]>(stage_mem);
   const PagedAttnParams& p = dp.base;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, g = lane >> 4;
   // Workgroups are dealt to the eight XCDs in turn: keep all row groups of one (batch, head) on
@@ -487,22 +571,77 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const int u_mine = min(max((wave_end + 31) / 32, u0), u_end);
       const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
       const int u_whole_begin = min((first + 31) / 32, u_whole_end);
-      // A unit is parked in LDS a whole turn before it is read: turn u parks unit u + 1 (fetched during turn u - 1)
-      // into the stage unit u - 1 was read from, fetches unit u + 2 into the registers that freed, and then works on
-      // unit u; the barrier at its end finds the next unit long written.
-      fetch(u0, std::false_type{});
-      park(0, std::false_type{});
-      fetch(min(u0 + 1, u_end - 1), std::false_type{});
-      __syncthreads();
+      // In this walk K / V go from memory straight into LDS (global_load_lds_dwordx4: lane l of a load lands at
+      // base + 16 l), two units ahead of their use (three stages), the stage laid out for the reads that follow: K in
+      // operand order (load (t, kk): lane (n, g) fetches the 16 bytes it will read back), V row-major with the 32-byte
+      // pieces of row r stored at piece index (piece ^ sw(r)), so that the sixteen rows one transposing read touches
+      // fall on different banks (the padding the register-staged layout uses cannot be had inside a 1 KiB load).
+      constexpr int UNIT_CHUNKS = 2 * MT * 64;  // 16-byte pieces of a unit: K, then V
+      constexpr int PER = MT / kCoopWaves;      // K loads and V loads per wave and unit
+      constexpr int ROWS_PER_LOAD = 64 / CH, ROW_BYTES = D * 2;
+      static_assert(3 * UNIT_CHUNKS * 16 <= STAGE_ELEMS * 2, "the three stages of this walk fit the kernel's LDS");
+      u32x4* const dstage = reinterpret_cast<u32x4*>(stage_mem);
+      auto sw = [](int r) { return D == 128 ? 2 * (r >> 3) + ((r & 3) >> 1) : (r >> 3) & 3; };  // < 32-byte pieces per row
+      const int k_first = wave * PER;
+      const int k_tok = 8 * (n >> 2) + 4 * (k_first / KK) + (n & 3), k_col = 32 * (k_first % KK) + 8 * g;
+      const int v_row = k_first * ROWS_PER_LOAD + lane / CH;
+      const int v_col = 8 * ((((lane % CH) >> 1) ^ sw(v_row)) * 2 + (lane & 1));
+      auto sending = [&](int u, bool on) {  // the loads of unit u (rows past the end are clamped, and masked later)
+        CoopSend sd;
+        sd.on = on, sd.whole = 32 * (u + 1) <= L;
+        sd.kp = kbase + (int64_t)min(32 * u + k_tok, L - 1) * D + k_col;
+        sd.vp = vbase + (int64_t)min(32 * u + v_row, L - 1) * D + v_col;
+        sd.vp2 = vbase + (int64_t)min(32 * u + v_row + ROWS_PER_LOAD, L - 1) * D + v_col;
+        return sd;
+      };
+      // byte offset (inside a stage) of this lane's first transposing read: row 8g + n/4, piece n%4 of 32-byte slot
+      // (0 ^ sw); slot j is one exclusive-or away, the rows four on one immediate offset
+      const int v_r0 = 8 * g + (n >> 2);
+      const int v_at = (MT * 64 * 16 + v_r0 * ROW_BYTES + (n & 3) * 8) ^ (sw(v_r0) << 5);
+      // Two units ahead: a unit's loads take longer than a unit's arithmetic here.  Unit u is complete in its stage
+      // once every wave's loads of it are back -- all but the newest unit's, counted, then the barrier; the same
+      // barrier says that every wave has taken unit u - 1 out of the stage the next loads reuse.  (Wait and barrier
+      // are written out: the library barrier waits for every outstanding load.)
+      auto send_only = [&](int u, int s) {  // prologue: nothing to read yet
+        const CoopSend sd = sending(u, true);
+        typedef const __attribute__((address_space(1))) void* gptr;
+        typedef __attribute__((address_space(3))) void* lptr;
+        u32x4* const nxt = dstage + s * UNIT_CHUNKS;
+        u32x4* const ks = nxt + k_first * 64;
+        __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 0, 0);
+        if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)(ks + 60), 16, 64, 0);
+        u32x4* const vs = nxt + (MT + k_first) * 64;
+        __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 0, 0);
+        if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.vp2, (lptr)(vs + 64), 16, 0, 0);
+      };
+      // (a wait the compiler sees, for the query rows' loads: its own wait for them would otherwise land inside the
+      // loop, at count 0, behind the direct-to-LDS loads of the coming units)
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      send_only(u0, 0);
+      if (u0 + 1 < u_end) send_only(u0 + 1, 1);
+      int cur = 0;  // stage of the unit at hand: (u - u0) % 3
       auto walk = [&](int from, int to, auto kind) {  // kind: 0 masked unit, 1 whole unit, 2 nothing to compute
         constexpr int KIND = decltype(kind)::value;
         for (int u = from; u < to; ++u) {
-          const int cur = (u - u0) & 1;
-          park(cur ^ 1, std::false_type{});
-          fetch(min(u + 2, u_end - 1), std::false_type{});
-          if (KIND == 0) unit(cur, 32 * u, std::false_type{}, std::false_type{}, wave_end, first);
-          if (KIND == 1) unit(cur, 32 * u, std::true_type{}, std::false_type{}, wave_end, first);
-          __syncthreads();
+          if (u + 1 < u_end) {
+            if (PER == 2) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+            else __builtin_amdgcn_s_waitcnt(0x0072);           // vmcnt(2) lgkmcnt(0)
+          } else {
+            __builtin_amdgcn_s_waitcnt(0x0070);                // vmcnt(0) lgkmcnt(0)
+          }
+          asm volatile("s_barrier" ::: "memory");
+          const int nxt = cur == 0 ? 2 : cur - 1;
+          const CoopSend sd = sending(u + 2, u + 2 < u_end);
+          if (KIND == 2) {
+            if (sd.on) send_only(u + 2, nxt);
+          } else {
+            f32x4 sc[NQT][2];
+            u32x4 vop[MT];
+            coop_stage_turn<D, NQT>(dstage + cur * UNIT_CHUNKS, dstage + nxt * UNIT_CHUNKS, sd, k_first, lane, v_at, qreg, sc, vop);
+            if (KIND == 0) softmax_and_output<D, NQT, false, false>(sc, vop, st, p, 32 * u, wave_end, first, g);
+            if (KIND == 1) softmax_and_output<D, NQT, false, true>(sc, vop, st, p, 32 * u, wave_end, first, g);
+          }
+          cur = cur == 2 ? 0 : cur + 1;
         }
       };
       walk(u0, u_whole_begin, std::integral_constant<int, 0>{});

@@ -105,6 +105,30 @@ def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     assert_attention_close(out, sdpa_fp32(q, k, v, m), f"prefill {B}x{N}x{S}x{H}x{L} {mask}")
 
 
+@pytest.mark.parametrize("B,N,S,H,L,pad,mdt,mB", [
+    (2, 32, 512, 128, 512, 0, torch.bfloat16, 2),     # the plain causal mask of a prompt
+    (2, 32, 300, 128, 333, 45, torch.bfloat16, 2),    # left-padded by 45 columns, a partial last unit, rows before the keys' end
+    (1, 40, 256, 64, 256, 0, torch.float32, 1),       # head_dim 64, fp32 mask, one mask for the whole batch
+    (2, 32, 260, 64, 203, 32, torch.bfloat16, 2),     # padding that ends on a unit, a last row group that is partly filled
+    (3, 16, 512, 128, 1100, 7, torch.bfloat16, 1),    # a chunk on top of a longer context (rows start at column 588)
+])
+def test_dense_prefill_with_plain_mask_lines(device, B, N, S, H, L, pad, mdt, mB):
+    """Masks whose lines are 0 over one stretch of columns and finfo.min elsewhere (causal, with or without left
+    padding): the op looks over the mask once and walks such rows by their first and last column, fetching K / V
+    straight into LDS.  One sequence's lines are made unplain (a bias; a hole) so that both walks run in one call."""
+    k, v = seeded_kv(31, B, N, L, H)
+    q = seeded_q(32, B, N, S, H)
+    past = L - S if L >= S else 0
+    cols, rows = torch.arange(L)[None, :], torch.arange(S)[:, None]
+    allowed = (cols <= rows + past) & (cols >= pad)
+    m = torch.zeros(mB, 1, S, L, dtype=mdt).masked_fill(~allowed[None, None], torch.finfo(mdt).min)
+    if mB > 1:
+        m[1, :, : S // 2, pad] -= 0.5                      # finite and not 0: these lines are read
+        m[1, :, S // 2 :, pad + 1] = torch.finfo(mdt).min  # a hole inside the stretch
+    out = torch.ops.pace.attention(q.to(device), k.to(device), v.to(device), m.to(device), 0)
+    assert_attention_close(out, sdpa_fp32(q, k, v, m), f"plain mask lines {B}x{N}x{S}x{H}x{L} pad {pad}")
+
+
 def test_dense_op_with_bmc_padded_buffers_and_finfo_min_mask(device):
     """BMC returns padded buffers and pads the mask with finfo.min (cache.py:195-222); the padded
     columns must not contribute."""
