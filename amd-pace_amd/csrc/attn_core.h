@@ -332,8 +332,12 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
           // when out of range, and propagates (like the reference) when in range.
         }
     }
-    const float mx_lane = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                                fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    const float top = st.m_top[qt];
+    bool above = false;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) above = above || s[t][i] > top;
     // exponent = (score - reference) * c with c = log2(e) (masked: natural units) or scale * log2(e).
     // The reference st.m follows the row's maximum lazily: it moves (and the accumulators are rescaled) only when
     // a score exceeds it by more than 2^kLazyLog2 in weight, for any row of the wave; until then weights may
@@ -343,8 +347,9 @@ __device__ __forceinline__ void softmax_and_output(const f32x4 (&sc)[NQT][2], co
     const float c = HAS_MASK ? kLog2e : p.scale_log2;
     // (a row's four lanes hold the same threshold: some lane's own maximum exceeds it exactly when the row's does,
     // so the maximum over the row's lanes is only formed when the reference moves)
-    if (__any(mx_lane > st.m_top[qt])) {  // m_top = -inf at first: the first real score always moves the reference
-      const float mx = row_max4(mx_lane);
+    if (__any(above)) {  // m_top = -inf at first: the first real score always moves the reference
+      const float mx = row_max4(fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                                      fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3]))));
       const float m_old = st.m[qt];
       const float m_new = fmaxf(m_old, mx);
       const float m_use = (m_new == kNegInf) ? 0.f : m_new;
