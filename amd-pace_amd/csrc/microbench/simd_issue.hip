@@ -32,6 +32,9 @@ enum Mode {
   kMfmaThenFma,   // 8 x (matrix instruction, multiply-add that reads its result)
   kSplit,         // first half of the waves: kMfmaChain; second half: kFma
   kInterleaved,   // every wave: 8 x (matrix instruction, 3 multiply-adds that do not depend on it)
+  kExpFma,        // 16 x (exp2, multiply-add that does not depend on it)
+  kSplitExp,      // first half of the waves: kMfmaChain; second half: kExp
+  kMfmaExp,       // every wave: 8 x (matrix instruction, 2 exp2 that do not depend on it)
 };
 
 template <int MODE, int WAVES>
@@ -74,6 +77,27 @@ __global__ __launch_bounds__(64 * WAVES) void issue_kernel(float* out, int iters
         for (int r = 0; r < 2; ++r)
 #pragma unroll
           for (int i = 0; i < 16; ++i) x[i] = __builtin_fmaf(x[i], 1.0001f, 0.5f);
+      }
+    } else if (MODE == kExpFma) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        x[i] = __builtin_amdgcn_exp2f(x[i]);
+        acc[i & 7][i >> 3] = __builtin_fmaf(acc[i & 7][i >> 3], 1.0001f, 0.5f);
+      }
+    } else if (MODE == kSplitExp) {
+      if (first_half) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) MFMA(acc[0]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]);
+      }
+    } else if (MODE == kMfmaExp) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        MFMA(acc[0]);
+        x[2 * i] = __builtin_amdgcn_exp2f(x[2 * i]);
+        x[2 * i + 1] = __builtin_amdgcn_exp2f(x[2 * i + 1]);
       }
     } else if (MODE == kInterleaved) {
 #pragma unroll
@@ -167,6 +191,11 @@ int main() {
   issue<kMfmaThenFma, 8>(out, it, "8 x (MFMA, FMA on its result)", 8);
   issue<kSplit, 8>(out, it, "one wave: 8 MFMA per turn, the other: 32 FMA per turn", 0);
   issue<kInterleaved, 8>(out, it, "each wave: 8 x (MFMA, 3 independent FMA) per turn", 0);
+  issue<kExpFma, 4>(out, it, "16 x (exp2, independent FMA)", 16);
+  issue<kExpFma, 8>(out, it, "16 x (exp2, independent FMA)", 16);
+  issue<kSplitExp, 8>(out, it, "one wave: 8 MFMA per turn, the other: 16 exp2 per turn", 0);
+  issue<kMfmaExp, 4>(out, it, "each wave: 8 x (MFMA, 2 independent exp2) per turn", 0);
+  issue<kMfmaExp, 8>(out, it, "each wave: 8 x (MFMA, 2 independent exp2) per turn", 0);
   lds<16>(out, 5000);
   lds<8>(out, 5000);
   lds<4>(out, 5000);
