@@ -67,6 +67,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
     const DenseParams p) {
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
   constexpr int MTL = HP / 16;  // 16-dim output tiles
+  constexpr int VG = MTL >= 4 ? 4 : MTL;  // output tiles whose dims of a lane are neighbours (see the V loads)
   constexpr int ROW_F = HP + 2;
   __shared__ float merge_buf[2 * 16 * ROW_F];
   const int H = p.H, L = p.L, S = p.S;
@@ -119,11 +120,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   auto fetch = [&](int tile, float (&kx)[KS], float (&vx)[MTL][4], float (&mx4)[4]) {
     const int t0 = tile * 16;
     load_run(kbase + (int64_t)min(L - 1, t0 + n) * H, kx);  // rows past the end are masked below
+    // V: output tile j of lane n stands for dim v_dim(j, n) = 16 VG (j / VG) + VG n + j % VG, so that the VG values a
+    // lane needs of one token for VG neighbouring tiles are one contiguous run: a quarter of the load instructions
+    // that one value per load takes, and every load of a wave covers whole 256-byte stretches of four rows.
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const T* vr = vbase + (int64_t)min(L - 1, t0 + 4 * g + i) * H + n;
+      const T* vr = vbase + (int64_t)min(L - 1, t0 + 4 * g + i) * H;
 #pragma unroll
-      for (int j = 0; j < MTL; ++j) vx[j][i] = (16 * j + n < H) ? load_f32<T>(vr + 16 * j) : 0.f;
+      for (int jj = 0; jj < MTL; jj += VG) {
+        const int d = 16 * jj + VG * n;
+        if (VEC && VG == 4 && d + 4 <= H) {
+          const f32x4 t = load4_f32(vr + d);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vx[jj + e][i] = t[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < VG; ++e) vx[jj + e][i] = (d + e < H) ? load_f32<T>(vr + d + e) : 0.f;
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -215,15 +229,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   if (ls != 0 || !valid) return;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   T* orow = static_cast<T*>(p.out) + (pair * S + row) * H;
+  // o[j][c] of lane (row, g) is the output at dim v_dim(j, 4 g + c)
 #pragma unroll
-  for (int j = 0; j < MTL; ++j) {
-    const int d = 16 * j + 4 * g;
-    if (VEC && d + 4 <= H) {
-      store4_out(orow + d, o[j] * inv);
-    } else {
+  for (int jj = 0; jj < MTL; jj += VG) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (d + c < H) store_out(orow + d + c, o[j][c] * inv);
+    for (int c = 0; c < 4; ++c) {
+      const int d = 16 * jj + VG * (4 * g + c);
+      if (VEC && VG == 4 && d + 4 <= H) {
+        store4_out(orow + d, f32x4{o[jj][c], o[jj + (1 % VG)][c], o[jj + (2 % VG)][c], o[jj + (3 % VG)][c]} * inv);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VG; ++e)
+          if (d + e < H) store_out(orow + d + e, o[jj + e][c] * inv);
+      }
     }
   }
 }
