@@ -62,15 +62,17 @@ struct DenseParams {
 // AHEAD: the operands of the next tile are fetched while this one is computed (a second set of registers: one
 // wave per SIMD at head size 128).  It pays where the launch is bound by memory (few query rows: +8 % on an fp32
 // decode step) and costs 10 % where it is bound by the matrix cores, so the launcher picks.
-template <typename T, typename MT, int HP, bool VEC, bool AHEAD>
+// EXACT: H == HP (and VEC): no bound on a dim is checked anywhere, which is a third of the vector instructions of a tile.
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_kernel(
     const DenseParams p) {
+  static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
   constexpr int MTL = HP / 16;  // 16-dim output tiles
   constexpr int VG = MTL >= 4 ? 4 : MTL;  // output tiles whose dims of a lane are neighbours (see the V loads)
   constexpr int ROW_F = HP + 2;
   __shared__ float merge_buf[2 * 16 * ROW_F];
-  const int H = p.H, L = p.L, S = p.S;
+  const int H = EXACT ? HP : p.H, L = p.L, S = p.S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int split = p.l_split;
   const int head = blockIdx.y, b = blockIdx.z;
@@ -174,14 +176,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
       pr[i] = expf(val[i] - m_use);
       sum += pr[i];
     }
-    l_run = l_run * alpha + sum;
-    m_run = m_new;
+    // (no row of the wave has a new maximum: alpha is exactly 1 in every lane, and the products with it are skipped)
+    if (__any(m_new != m_run)) {
+      l_run = l_run * alpha + sum;
 #pragma unroll
-    for (int j = 0; j < MTL; ++j) {
-      o[j] *= alpha;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j][i], pr[i], o[j], 0, 0, 0);
+      for (int j = 0; j < MTL; ++j) o[j] *= alpha;
+    } else {
+      l_run += sum;
     }
+    m_run = m_new;
+    // token quarter by token quarter over all output tiles: neighbouring matrix instructions write different
+    // accumulators (per tile the order of the four is unchanged)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < MTL; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j][i], pr[i], o[j], 0, 0, 0);
     if constexpr (AHEAD) {
       if (more) {
 #pragma unroll
@@ -306,10 +315,12 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
   do { \
     constexpr bool kAheadBuilt = HP_ <= 128; /* at 256 the second set of registers does not fit */ \
     if (ahead && kAheadBuilt) { \
-      if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt>), grid, dim3(256), 0, s, p); \
-      else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, kAheadBuilt>), grid, dim3(256), 0, s, p); \
-    } else if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, false>), grid, dim3(256), 0, s, p); \
-    else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, false>), grid, dim3(256), 0, s, p); \
+      if (vec && H == HP_) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt, true>), grid, dim3(256), 0, s, p); \
+      else if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt, false>), grid, dim3(256), 0, s, p); \
+      else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, kAheadBuilt, false>), grid, dim3(256), 0, s, p); \
+    } else if (vec && H == HP_) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, false, true>), grid, dim3(256), 0, s, p); \
+    else if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, false, false>), grid, dim3(256), 0, s, p); \
+    else hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, false, false, false>), grid, dim3(256), 0, s, p); \
   } while (0)
 #define PACE_DENSE_HP(T_, MT_) \
   do { \

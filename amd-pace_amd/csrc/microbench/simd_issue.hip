@@ -35,6 +35,8 @@ enum Mode {
   kExpFma,        // 16 x (exp2, multiply-add that does not depend on it)
   kSplitExp,      // first half of the waves: kMfmaChain; second half: kExp
   kMfmaExp,       // every wave: 8 x (matrix instruction, 2 exp2 that do not depend on it)
+  kMfmaF32,       // 8 fp32 matrix instructions (16x16x4) on eight accumulators
+  kMfmaF32Chain,  // 8 fp32 matrix instructions on one accumulator
 };
 
 template <int MODE, int WAVES>
@@ -99,6 +101,12 @@ __global__ __launch_bounds__(64 * WAVES) void issue_kernel(float* out, int iters
         x[2 * i] = __builtin_amdgcn_exp2f(x[2 * i]);
         x[2 * i + 1] = __builtin_amdgcn_exp2f(x[2 * i + 1]);
       }
+    } else if (MODE == kMfmaF32) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[i], x[i + 8], acc[i], 0, 0, 0);
+    } else if (MODE == kMfmaF32Chain) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[i], x[i + 8], acc[0], 0, 0, 0);
     } else if (MODE == kInterleaved) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -196,6 +204,10 @@ int main() {
   issue<kSplitExp, 8>(out, it, "one wave: 8 MFMA per turn, the other: 16 exp2 per turn", 0);
   issue<kMfmaExp, 4>(out, it, "each wave: 8 x (MFMA, 2 independent exp2) per turn", 0);
   issue<kMfmaExp, 8>(out, it, "each wave: 8 x (MFMA, 2 independent exp2) per turn", 0);
+  issue<kMfmaF32, 4>(out, it, "8 MFMA 16x16x4 f32 on eight accumulators", 8);
+  issue<kMfmaF32, 8>(out, it, "8 MFMA 16x16x4 f32 on eight accumulators", 8);
+  issue<kMfmaF32Chain, 4>(out, it, "8 MFMA 16x16x4 f32 on one accumulator", 8);
+  issue<kMfmaF32Chain, 8>(out, it, "8 MFMA 16x16x4 f32 on one accumulator", 8);
   lds<16>(out, 5000);
   lds<8>(out, 5000);
   lds<4>(out, 5000);
