@@ -141,10 +141,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
         }
       }
     }
+    // the lane's four mask values: one load where the four columns exist (mask lines start wherever L puts them;
+    // the hardware takes unaligned multi-dword loads), element by element at the end of a line
+    const int t = t0 + 4 * g;
+    if (!mrow) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int t = t0 + 4 * g + i;
-      mx4[i] = (mrow && t < L) ? load_f32<MT>(mrow + t) : 0.f;
+      for (int i = 0; i < 4; ++i) mx4[i] = 0.f;
+    } else if (t + 4 <= L) {
+      if constexpr (sizeof(MT) == 4) {
+        u32x4 raw;
+        __builtin_memcpy(&raw, mrow + t, 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx4[i] = __uint_as_float(raw[i]);
+      } else {
+        u32x2 raw;
+        __builtin_memcpy(&raw, mrow + t, 8);
+        mx4[0] = __uint_as_float(raw[0] << 16), mx4[1] = __uint_as_float(raw[0] & 0xffff0000u);
+        mx4[2] = __uint_as_float(raw[1] << 16), mx4[3] = __uint_as_float(raw[1] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx4[i] = (t + i < L) ? load_f32<MT>(mrow + t + i) : 0.f;
     }
   };
   if (AHEAD && has_rows && tile_lo < tile_hi) fetch(tile_lo, kf, vf, mv);
