@@ -42,6 +42,14 @@ __device__ __forceinline__ f32x4 load4_f32(const uint16_t* p) {
   return f32x4{bf16_bits_to_f32(w[0] & 0xffffu), __uint_as_float(w[0] & 0xffff0000u), bf16_bits_to_f32(w[1] & 0xffffu),
                __uint_as_float(w[1] & 0xffff0000u)};
 }
+// Two consecutive elements (p 8- resp. 4-byte aligned).
+__device__ __forceinline__ f32x2 load2_f32(const float* p) { return *reinterpret_cast<const f32x2*>(p); }
+__device__ __forceinline__ f32x2 load2_f32(const uint16_t* p) {
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+  return f32x2{bf16_bits_to_f32(w & 0xffffu), __uint_as_float(w & 0xffff0000u)};
+}
+__device__ __forceinline__ void store2_out(float* p, f32x2 v) { *reinterpret_cast<f32x2*>(p) = v; }
+__device__ __forceinline__ void store2_out(uint16_t* p, f32x2 v) { *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(v[0], v[1]); }
 __device__ __forceinline__ void store4_out(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
 __device__ __forceinline__ void store4_out(uint16_t* p, f32x4 v) {
   *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
@@ -73,7 +81,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
   constexpr int MTL = HP / 16;  // 16-dim output tiles
-  constexpr int VG = MTL >= 4 ? 4 : MTL;  // output tiles whose dims of a lane are neighbours (see the V loads)
+  constexpr int VG = MTL % 4 == 0 ? 4 : 2;  // output tiles whose dims of a lane are neighbours (see the V loads)
+  static_assert(MTL % VG == 0, "head sizes built: multiples of 32");
   constexpr int ROW_F = HP + 2;
   __shared__ float merge_buf[2 * 16 * ROW_F];
   const int H = EXACT ? HP : p.H, L = p.L, S = p.S;
@@ -98,8 +107,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 #pragma unroll
     for (int s4 = 0; s4 < KS; s4 += 4) {
       const int d = d0 + s4;
-      if (VEC && d + 4 <= H) {
-        const f32x4 t = load4_f32(r + d);
+      if (VEC) {  // H is a multiple of 4: the four dims exist together or not at all
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        if (d + 4 <= H) t = load4_f32(r + d);
         x[s4] = t[0], x[s4 + 1] = t[1], x[s4 + 2] = t[2], x[s4 + 3] = t[3];
       } else {
 #pragma unroll
@@ -135,10 +145,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 #pragma unroll
       for (int jj = 0; jj < MTL; jj += VG) {
         const int d = 16 * jj + VG * n;
-        if (VEC && VG == 4 && d + 4 <= H) {
-          const f32x4 t = load4_f32(vr + d);
+        if (VEC && VG == 4) {
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          if (d + 4 <= H) t = load4_f32(vr + d);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) vx[jj + e][i] = t[e];
+          for (int e = 0; e < 4; ++e) vx[jj + (e % VG)][i] = t[e];
+        } else if (VEC && VG == 2) {
+          f32x2 t = {0.f, 0.f};
+          if (d + 2 <= H) t = load2_f32(vr + d);
+          vx[jj][i] = t[0], vx[jj + (1 % VG)][i] = t[1];
         } else {
 #pragma unroll
           for (int e = 0; e < VG; ++e) vx[jj + e][i] = (d + e < H) ? load_f32<T>(vr + d + e) : 0.f;
@@ -265,8 +280,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int d = 16 * jj + VG * (4 * g + c);
-      if (VEC && VG == 4 && d + 4 <= H) {
-        store4_out(orow + d, f32x4{o[jj][c], o[jj + (1 % VG)][c], o[jj + (2 % VG)][c], o[jj + (3 % VG)][c]} * inv);
+      if (VEC && VG == 4) {
+        if (d + 4 <= H) store4_out(orow + d, f32x4{o[jj][c], o[jj + (1 % VG)][c], o[jj + (2 % VG)][c], o[jj + (3 % VG)][c]} * inv);
+      } else if (VEC && VG == 2) {
+        if (d + 2 <= H) store2_out(orow + d, f32x2{o[jj][c], o[jj + (1 % VG)][c]} * inv);
       } else {
 #pragma unroll
         for (int e = 0; e < VG; ++e)
@@ -347,6 +364,7 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
   do { \
     if (H <= 32) PACE_DENSE_GO(T_, MT_, 32); \
     else if (H <= 64) PACE_DENSE_GO(T_, MT_, 64); \
+    else if (H <= 96) PACE_DENSE_GO(T_, MT_, 96); \
     else if (H <= 128) PACE_DENSE_GO(T_, MT_, 128); \
     else PACE_DENSE_GO(T_, MT_, 256); \
   } while (0)
