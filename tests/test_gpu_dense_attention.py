@@ -20,6 +20,8 @@ CASES = [
     (1, 1, 1, 1, 1), (1, 16, 128, 64, 512), (32, 1, 1, 128, 2048), (2, 32, 512, 128, 1), (3, 2, 17, 1, 33),
     (2, 16, 1, 64, 2048), (96, 1, 1, 64, 1), (1, 1, 128, 128, 512), (2, 3, 5, 80, 70), (1, 2, 33, 256, 40),
     (2, 4, 1, 96, 700), (1, 3, 100, 96, 333), (2, 2, 1, 256, 900), (1, 2, 70, 256, 130), (1, 2, 9, 100, 50),
+    # head sizes off every built one: not a multiple of 4 (element by element), 30 (the 32 build), 80 over several tiles
+    (1, 2, 40, 50, 90), (1, 2, 20, 30, 45), (1, 2, 64, 80, 300),
 ]
 
 
