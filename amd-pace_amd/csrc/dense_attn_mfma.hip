@@ -206,15 +206,17 @@ constexpr int kCoopWaves = 4;
 
 // One turn of the walk that keeps its units in LDS by direct loads (dense_attn_coop_kernel, plain mask lines): send
 // this wave's share of a coming unit into stage `nxt` and take the operands of the unit at hand out of stage `cur`
-// (K in operand order, V row-major with swizzled 32-byte pieces through the transposing read), with the score
-// products between the K and the V reads.
+// (both row-major as in memory, so that every load is 1 KiB of contiguous rows; K with its 16-byte chunks swizzled by
+// row for the operand reads, V with swizzled 32-byte pieces for the transposing read), with the score products
+// between the K and the V reads.
 // The LDS reads are written as instructions, with their own wait: before an LDS read the compiler sees, it waits for
 // every outstanding direct-to-LDS load (it cannot tell that the read does not touch what they write) -- the full
 // memory latency of the unit just sent, every turn (measured: more than half of the wave cycles).  The reads here
 // are of a stage whose loads the caller has waited for (vmcnt, barrier), the loads in flight write other stages.
 struct CoopSend {
-  const uint16_t* kp;   // this lane's K piece of the coming unit (second load: 64 bytes on)
-  const uint16_t* vp;   // this lane's V piece (second load: four rows on, or vp2 where rows are clamped)
+  const uint16_t* kp;   // this lane's K piece of the coming unit (second load: four rows on, or kp2 where rows are clamped)
+  const uint16_t* kp2;
+  const uint16_t* vp;   // this lane's V piece (likewise)
   const uint16_t* vp2;
   bool on, whole;       // wave-uniform
 };
@@ -222,7 +224,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
 template <int D, int NQT>
-__device__ __forceinline__ void coop_stage_turn(const u32x4* cur, u32x4* nxt, const CoopSend& sd, int k_first, int lane, int v_at,
+__device__ __forceinline__ void coop_stage_turn(const u32x4* cur, u32x4* nxt, const CoopSend& sd, int k_first, int k_at, int v_at,
                                                 const u32x4 (&qreg)[NQT][D / 32], f32x4 (&sc)[NQT][2], u32x4 (&vop)[D / 16]) {
   constexpr int KK = D / 32, MT = D / 16, PER = MT / kCoopWaves, ROW_BYTES = D * 2;
   typedef const __attribute__((address_space(1))) void* gptr;
@@ -231,26 +233,30 @@ __device__ __forceinline__ void coop_stage_turn(const u32x4* cur, u32x4* nxt, co
   static_assert(KK == 2 || KK == 4, "head_dim 64 or 128");
   if (sd.on) {
     u32x4* const ks = nxt + k_first * 64;
-    __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 0, 0);
-    // (the immediate offset moves the address in memory and the one in LDS alike: 64 bytes on in the row, 1024 in the stage)
-    if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)(ks + 60), 16, 64, 0);
     u32x4* const vs = nxt + (MT + k_first) * 64;
+    __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 0, 0);
     __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 0, 0);
     if (PER == 2) {
-      if (sd.whole) {  // four rows on: 1024 bytes in memory and in the stage, the same swizzle
+      if (sd.whole) {  // four rows on: 1024 bytes in memory and in the stage (the immediate offset moves both), the same swizzle
+        __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 4 * ROW_BYTES, 0);
         __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 4 * ROW_BYTES, 0);
       } else {
+        __builtin_amdgcn_global_load_lds((gptr)sd.kp2, (lptr)(ks + 64), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((gptr)sd.vp2, (lptr)(vs + 64), 16, 0, 0);
       }
     }
   }
+  // K: rows of token tile t lie four rows on (an immediate offset); the chunk of contraction step kk is one
+  // exclusive-or away from that of step 0 (the swizzle key sits in the same bits)
   u32x4 kop[2][KK];
-  const uint32_t k_at = lds_address(cur) + lane * 16;
+  const uint32_t k_base = lds_address(cur) + k_at;
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int kk = 0; kk < KK; ++kk) {
+    const uint32_t at = k_base ^ (kk << 6);
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kop[t][kk]) : "v"(k_at), "n"((t * KK + kk) * 1024) : "memory");
+    for (int t = 0; t < 2; ++t)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kop[t][kk]) : "v"(at), "n"(t * 4 * ROW_BYTES) : "memory");
+  }
   if constexpr (KK == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(kop[0][0]), "+v"(kop[0][1]), "+v"(kop[0][2]), "+v"(kop[0][3]), "+v"(kop[1][0]), "+v"(kop[1][1]), "+v"(kop[1][2]),
@@ -572,10 +578,12 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       const int u_whole_end = min(max((min(wave_end - 1, min_limit) + 1) / 32, u0), u_mine);
       const int u_whole_begin = min((first + 31) / 32, u_whole_end);
       // In this walk K / V go from memory straight into LDS (global_load_lds_dwordx4: lane l of a load lands at
-      // base + 16 l), two units ahead of their use (three stages), the stage laid out for the reads that follow: K in
-      // operand order (load (t, kk): lane (n, g) fetches the 16 bytes it will read back), V row-major with the 32-byte
-      // pieces of row r stored at piece index (piece ^ sw(r)), so that the sixteen rows one transposing read touches
-      // fall on different banks (the padding the register-staged layout uses cannot be had inside a 1 KiB load).
+      // base + 16 l), two units ahead of their use (three stages).  Both operands stay row-major, so that a load is 1 KiB of
+      // contiguous rows, and are swizzled for the reads that follow (the padding the register-staged layout uses cannot
+      // be had inside a 1 KiB load): K with the 16-byte chunks of row r at chunk index (chunk ^ kw(r)), V with the
+      // 32-byte pieces of row r at piece index (piece ^ sw(r)), so that the sixteen rows one operand read or one
+      // transposing read touches fall on different banks.  (K fetched in operand order instead -- lane (n, g) of load
+      // (t, kk) the 16 bytes it reads back: sixteen 64-byte runs per load -- measured 2.6 % slower.)
       constexpr int UNIT_CHUNKS = 2 * MT * 64;  // 16-byte pieces of a unit: K, then V
       constexpr int PER = MT / kCoopWaves;      // K loads and V loads per wave and unit
       constexpr int ROWS_PER_LOAD = 64 / CH, ROW_BYTES = D * 2;
@@ -583,19 +591,27 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
       u32x4* const dstage = reinterpret_cast<u32x4*>(stage_mem);
       auto sw = [](int r) { return D == 128 ? 2 * (r >> 3) + ((r & 3) >> 1) : (r >> 3) & 3; };  // < 32-byte pieces per row
       const int k_first = wave * PER;
-      const int k_tok = 8 * (n >> 2) + 4 * (k_first / KK) + (n & 3), k_col = 32 * (k_first % KK) + 8 * g;
+      // (the sixteen rows of one K operand read are 8a + b + 4t, a and b below 4: kw tells them apart and is the same
+      // four rows on, so that a wave's second load is the first one's lane addresses plus an immediate offset)
+      auto kw = [](int r) { return D == 128 ? ((r >> 3) << 2) | (r & 3) : 2 * (r >> 3) + ((r & 3) >> 1); };
+      const int k_row = k_first * ROWS_PER_LOAD + lane / CH;
+      const int k_col = 8 * ((lane % CH) ^ kw(k_row));
       const int v_row = k_first * ROWS_PER_LOAD + lane / CH;
       const int v_col = 8 * ((((lane % CH) >> 1) ^ sw(v_row)) * 2 + (lane & 1));
       auto sending = [&](int u, bool on) {  // the loads of unit u (rows past the end are clamped, and masked later)
         CoopSend sd;
         sd.on = on, sd.whole = 32 * (u + 1) <= L;
-        sd.kp = kbase + (int64_t)min(32 * u + k_tok, L - 1) * D + k_col;
+        sd.kp = kbase + (int64_t)min(32 * u + k_row, L - 1) * D + k_col;
+        sd.kp2 = kbase + (int64_t)min(32 * u + k_row + ROWS_PER_LOAD, L - 1) * D + k_col;
         sd.vp = vbase + (int64_t)min(32 * u + v_row, L - 1) * D + v_col;
         sd.vp2 = vbase + (int64_t)min(32 * u + v_row + ROWS_PER_LOAD, L - 1) * D + v_col;
         return sd;
       };
       // byte offset (inside a stage) of this lane's first transposing read: row 8g + n/4, piece n%4 of 32-byte slot
       // (0 ^ sw); slot j is one exclusive-or away, the rows four on one immediate offset
+      // byte offset of this lane's K read of token tile 0, contraction step 0: row 8 (n / 4) + n % 4, chunk g
+      const int k_r0 = 8 * (n >> 2) + (n & 3);
+      const int k_at = k_r0 * ROW_BYTES + ((g ^ kw(k_r0)) << 4);
       const int v_r0 = 8 * g + (n >> 2);
       const int v_at = (MT * 64 * 16 + v_r0 * ROW_BYTES + (n & 3) * 8) ^ (sw(v_r0) << 5);
       // Two units ahead: a unit's loads take longer than a unit's arithmetic here.  Unit u is complete in its stage
@@ -609,7 +625,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
         u32x4* const nxt = dstage + s * UNIT_CHUNKS;
         u32x4* const ks = nxt + k_first * 64;
         __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)ks, 16, 0, 0);
-        if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.kp, (lptr)(ks + 60), 16, 64, 0);
+        if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.kp2, (lptr)(ks + 64), 16, 0, 0);
         u32x4* const vs = nxt + (MT + k_first) * 64;
         __builtin_amdgcn_global_load_lds((gptr)sd.vp, (lptr)vs, 16, 0, 0);
         if (PER == 2) __builtin_amdgcn_global_load_lds((gptr)sd.vp2, (lptr)(vs + 64), 16, 0, 0);
@@ -637,7 +653,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
           } else {
             f32x4 sc[NQT][2];
             u32x4 vop[MT];
-            coop_stage_turn<D, NQT>(dstage + cur * UNIT_CHUNKS, dstage + nxt * UNIT_CHUNKS, sd, k_first, lane, v_at, qreg, sc, vop);
+            coop_stage_turn<D, NQT>(dstage + cur * UNIT_CHUNKS, dstage + nxt * UNIT_CHUNKS, sd, k_first, k_at, v_at, qreg, sc, vop);
             if (KIND == 0) softmax_and_output<D, NQT, false, false>(sc, vop, st, p, 32 * u, wave_end, first, g);
             if (KIND == 1) softmax_and_output<D, NQT, false, true>(sc, vop, st, p, 32 * u, wave_end, first, g);
           }
