@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
                                                               const RopeDev rope) {
   constexpr int CHUNKS = D / 8;
   constexpr int BT = PACE_KV_BLOCK_TOKENS;
-  __shared__ uint16_t ks[BT * D];
-  __shared__ uint16_t vs[BT * (D + 8)];  // padded rows: column reads hit different banks
+  __shared__ uint16_t ks[ROPE ? BT * D : 8];  // keys pass through LDS only where they are rotated on the way
+  __shared__ uint16_t vs[BT * (D + 8)];       // padded rows: column reads hit different banks
   const int h = blockIdx.y, b = blockIdx.z;
   const int64_t pos0 = (int64_t)dest.seq_lens[b] + dest.pos_offset;  // position of new token 0
   if (pos0 < 0) return;
@@ -108,20 +108,31 @@ __global__ __launch_bounds__(256) void kv_append_block_kernel(pace_kv_pool_t poo
     for (int c = threadIdx.x; c < n_here * CHUNKS; c += 256) {
       const int r = c / CHUNKS, ch = c % CHUNKS;
       const int64_t src = (int64_t)(t_lo + r) * st + ch * 8;
-      *reinterpret_cast<u32x4*>(&ks[(off_lo + r) * D + ch * 8]) = load16_stream(kin + src);
       *reinterpret_cast<u32x4*>(&vs[(off_lo + r) * (D + 8) + ch * 8]) = load16_stream(vin + src);
     }
   }
-  __syncthreads();
   uint16_t* kslab = reinterpret_cast<uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
   uint16_t* vslab = reinterpret_cast<uint16_t*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
   const bool whole = (n_here == BT);
-  // K: slab chunk c = (tile, dim chunk, slot) holds dims 8*chunk.. of token tok(tile, slot).
-  for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
-    const int tile = c / (CHUNKS * 8), chunk = (c / 8) % CHUNKS, slot = c % 8;
-    const int tok = ((slot >> 2) << 3) | (tile << 2) | (slot & 3);
-    if (tok >= off_lo && tok < off_lo + n_here)
-      store16_stream(kslab + c * 8, *reinterpret_cast<const u32x4*>(&ks[tok * D + chunk * 8]));
+  // K: slab chunk c = (tile, dim chunk, slot) holds dims 8*chunk.. of token tok(tile, slot).  Keys that are not
+  // rotated need no staging: the chunk goes from its row to its slab place through a register (a wave reads eight
+  // 128-byte runs and writes 1 KiB in one piece), before the barrier, so that it travels along with the V loads.
+  if (!ROPE) {
+    for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
+      const int tile = c / (CHUNKS * 8), chunk = (c / 8) % CHUNKS, slot = c % 8;
+      const int tok = ((slot >> 2) << 3) | (tile << 2) | (slot & 3);
+      if (tok >= off_lo && tok < off_lo + n_here)
+        store16_stream(kslab + c * 8, load16_stream(kin + (int64_t)(t_lo + tok - off_lo) * st + chunk * 8));
+    }
+  }
+  __syncthreads();
+  if (ROPE) {
+    for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
+      const int tile = c / (CHUNKS * 8), chunk = (c / 8) % CHUNKS, slot = c % 8;
+      const int tok = ((slot >> 2) << 3) | (tile << 2) | (slot & 3);
+      if (tok >= off_lo && tok < off_lo + n_here)
+        store16_stream(kslab + c * 8, *reinterpret_cast<const u32x4*>(&ks[tok * D + chunk * 8]));
+    }
   }
   // V: slab chunk c = (dim tile, token half, dim) holds tokens 8*half..+7 of one dim.
   for (int c = threadIdx.x; c < BT * CHUNKS; c += 256) {
