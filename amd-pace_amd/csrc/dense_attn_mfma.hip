@@ -306,7 +306,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   constexpr bool HAS_MASK = MASK != 0;
   static_assert(PER_THREAD >= 1 && (32 * CH) % (64 * kCoopWaves) == 0, "unit does not divide over the workgroup");
   // (the walk over plain mask lines keeps three units of 2 * MT KiB in the same memory, see below)
-  constexpr int STAGE_ELEMS = 2 * STAGE > 3 * MT * 1024 ? 2 * STAGE : 3 * MT * 1024;
+  // (at head_dim 256 three such units would leave room for one workgroup per compute unit: that walk is not built)
+  constexpr bool DIRECT_WALK = D <= 128;
+  constexpr int STAGE_ELEMS = (!DIRECT_WALK || 2 * STAGE > 3 * MT * 1024) ? 2 * STAGE : 3 * MT * 1024;
   __shared__ __attribute__((aligned(256))) uint16_t stage_mem[STAGE_ELEMS];
   uint16_t(*stage)[STAGE] = reinterpret_cast<uint16_t(*)[STAGE]>(stage_mem);
   const PagedAttnParams& p = dp.base;
@@ -424,7 +426,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // the two operand sets disjoint inside a unit, and a workgroup barrier between units, it cannot occur.
   // by_mask: the unit's mask values decide (all of [0, L) is walked); else the rows' own limits and `first` do
   // (plain mask lines, see below), and the mask values are not looked at.
-  auto unit = [&](int cur, int t0, auto full_tag, auto by_mask, int tok_end, int first) {
+  // before_weights(): called once the unit's operands are in their registers and the score products are issued (not
+  // at all for a unit that is skipped) -- the place for loads whose registers should not be alive next to the K operands.
+  auto unit = [&](int cur, int t0, auto full_tag, auto by_mask, int tok_end, int first, auto before_weights) {
     constexpr bool FULL = decltype(full_tag)::value;
     constexpr bool BY_MASK = decltype(by_mask)::value && HAS_MASK;
     if (BY_MASK && MASK == 2) {
@@ -458,6 +462,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) asm volatile("" ::"v"(kop[t][kk]));  // K operands live up to here
     __builtin_amdgcn_sched_barrier(0);
+    before_weights();
     softmax_and_output<D, NQT, BY_MASK, FULL>(sc, vop, st, p, t0, tok_end, first, g, mcur);
   };
   // Units past the last one that matters to any row of the workgroup are not walked at all: with a
@@ -472,7 +477,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   // mask tensor -- that first column, their own last column -- and the mask is not read (`plain`).
   bool plain = false;
   int f_min = 0x7fffffff, f_max = -1, wg_last = -1, l_min = 0x7fffffff;
-  const bool summarised = HAS_MASK && dp.line_last && dp.line_first;
+  const bool summarised = DIRECT_WALK && HAS_MASK && dp.line_last && dp.line_first;
   const int64_t line0 = ((dp.mB == 1 ? 0 : (int64_t)b) * dp.mN + (dp.mN == 1 ? 0 : head)) * dp.mS;
   if (summarised) {
 #pragma unroll
@@ -556,7 +561,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   }
   // One loop per kind of unit -- masked before the rows' whole units, whole, masked after them, needed by other waves
   // only -- so that the accumulators have one path through each loop body.
-  if (plain) {
+  if constexpr (DIRECT_WALK) if (plain) {
     {
       int min_limit = 0x7fffffff, mine = -1;
 #pragma unroll
@@ -674,14 +679,25 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     __syncthreads();
     for (int u = 0; u < whole; ++u) {
       const int cur = u & 1;
-      fetch(min(u + 1, units - 1), std::true_type{});  // unconditional: no branch between a load and the wait for it
-      if (wave_has_rows) {
-        unit(cur, 32 * u, std::true_type{}, std::true_type{}, L, 0);
+      if constexpr (D <= 128) {
+        fetch(min(u + 1, units - 1), std::true_type{});  // unconditional: no branch between a load and the wait for it
+        if (wave_has_rows) unit(cur, 32 * u, std::true_type{}, std::true_type{}, L, 0, [] {});
+      } else {
+        // head_dim 256: the next unit's loads are issued behind the score products, when the K operands' 64 registers
+        // are free again -- with them issued first, about 90 registers spill
+        bool sent = false;
+        if (wave_has_rows) {
+          unit(cur, 32 * u, std::true_type{}, std::true_type{}, L, 0, [&] {
+            fetch(min(u + 1, units - 1), std::true_type{});
+            sent = true;
+          });
+        }
+        if (!sent) fetch(min(u + 1, units - 1), std::true_type{});
       }
       park(cur ^ 1, std::true_type{});
       __syncthreads();
     }
-    if (whole < units && wave_has_rows) unit(whole & 1, 32 * whole, std::false_type{}, std::true_type{}, L, 0);
+    if (whole < units && wave_has_rows) unit(whole & 1, 32 * whole, std::false_type{}, std::true_type{}, L, 0, [] {});
   }
 
 #pragma unroll
@@ -718,11 +734,11 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
-  const bool coop_built = H == 64 || H == 128;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
+  const bool coop_built = H == 64 || H == 128 || H == 256;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
   if (tiles > 4 && coop_built) {
     // prefill-sized: rows of a head share its K / V through LDS
     const int mode = !mask ? 0 : (mask_is_f32 ? 1 : 2);
-    int cnqt = 2;
+    int cnqt = H == 256 ? 1 : 2;  // (two tiles of head_dim 256 do not fit the register file)
     dp.n_qgroups = (tiles + kCoopWaves * cnqt - 1) / (kCoopWaves * cnqt);
     // too few workgroups: halve their rows; so does the element-wise mask path at head_dim 128, whose
     // two-tile form does not fit the register file
@@ -744,7 +760,8 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
 #define PACE_COOP(D_, Q_, M_) hipLaunchKernelGGL((dense_attn_coop_kernel<D_, Q_, M_>), cgrid, cblock, 0, stream, dp)
 #define PACE_COOP_M(D_, Q_) \
   do { if (mode == 0) PACE_COOP(D_, Q_, 0); else if (mode == 1) PACE_COOP(D_, Q_, 1); else PACE_COOP(D_, Q_, 2); } while (0)
-    if (H == 128) { if (cnqt == 2) PACE_COOP_M(128, 2); else PACE_COOP_M(128, 1); }
+    if (H == 256) PACE_COOP_M(256, 1);
+    else if (H == 128) { if (cnqt == 2) PACE_COOP_M(128, 2); else PACE_COOP_M(128, 1); }
     else { if (cnqt == 2) PACE_COOP_M(64, 2); else PACE_COOP_M(64, 1); }
 #undef PACE_COOP_M
 #undef PACE_COOP

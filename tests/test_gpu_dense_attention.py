@@ -73,6 +73,14 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     (1, 4, 100, 64, 41, "causal-short-f32"),
     (2, 3, 20, 64, 8, "causal-short-bf16"),
     (1, 2, 40, 128, 70, "rows-masked-bf16"),
+    # head_dim 256: rows of a head share K / V through LDS here too, one tile per wave, in every mask form
+    (1, 3, 200, 256, 333, "causal-bf16"),
+    (2, 4, 130, 256, 264, "causal-bf16"),
+    (1, 2, 100, 256, 96, "causal-f32"),
+    (1, 2, 100, 256, 50, None),
+    (1, 5, 300, 256, 96, "heads-bf16"),
+    (1, 2, 90, 256, 41, "causal-short-bf16"),
+    (1, 2, 80, 256, 70, "rows-masked-bf16"),
 ])
 def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     from oracle.attention_ref import causal_mask_4d
@@ -235,5 +243,18 @@ def test_dense_prefill_is_bit_identical_from_call_to_call(device):
     assert_attention_close(first, sdpa_fp32(q, k, v, causal), "prefill, causal mask")
     for _ in range(1000):
         out = torch.ops.pace.attention(qd, kd, vd, cd, 0)
+        differing += int(not torch.equal(out.view(torch.int16), first.view(torch.int16)))
+    assert differing == 0
+    # head_dim 256: the next unit's loads are issued right behind the score products there
+    B, N, S, H, L = 2, 16, 256, 256, 128
+    k, v = seeded_kv(24, B, N, L, H)
+    q = seeded_q(25, B, N, S, H)
+    band = (torch.arange(L)[None, :] + torch.arange(S)[:, None]) % 3 == 0
+    m = torch.zeros(B, 1, S, L, dtype=torch.bfloat16).masked_fill(band, torch.finfo(torch.bfloat16).min)
+    qd, kd, vd, md = q.to(device), k.to(device), v.to(device), m.to(device)
+    first = torch.ops.pace.attention(qd, kd, vd, md, 0)
+    assert_attention_close(first, sdpa_fp32(q, k, v, m), "prefill, head_dim 256")
+    for _ in range(500):
+        out = torch.ops.pace.attention(qd, kd, vd, md, 0)
         differing += int(not torch.equal(out.view(torch.int16), first.view(torch.int16)))
     assert differing == 0
