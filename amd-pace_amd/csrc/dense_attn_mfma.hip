@@ -302,12 +302,13 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   constexpr int KSTAGE = 32 * KROW + KHALF;
   constexpr int STAGE = KSTAGE + 32 * VROW;
   constexpr int CH = D / 8;          // 16-byte chunks per row
-  constexpr int PER_THREAD = 32 * CH / (64 * kCoopWaves);
+  constexpr int PER_THREAD = (32 * CH + 64 * kCoopWaves - 1) / (64 * kCoopWaves);
+  constexpr bool WHOLE_ROUNDS = (32 * CH) % (64 * kCoopWaves) == 0;  // every thread has a chunk in every round
   constexpr bool HAS_MASK = MASK != 0;
-  static_assert(PER_THREAD >= 1 && (32 * CH) % (64 * kCoopWaves) == 0, "unit does not divide over the workgroup");
   // (the walk over plain mask lines keeps three units of 2 * MT KiB in the same memory, see below)
-  // (at head_dim 256 three such units would leave room for one workgroup per compute unit: that walk is not built)
-  constexpr bool DIRECT_WALK = D <= 128;
+  // (at head_dim 256 three such units would leave room for one workgroup per compute unit, and a unit of head_dim 96
+  // does not divide into whole loads per wave: that walk is not built for them)
+  constexpr bool DIRECT_WALK = D == 64 || D == 128;
   constexpr int STAGE_ELEMS = (!DIRECT_WALK || 2 * STAGE > 3 * MT * 1024) ? 2 * STAGE : 3 * MT * 1024;
   __shared__ __attribute__((aligned(256))) uint16_t stage_mem[STAGE_ELEMS];
   uint16_t(*stage)[STAGE] = reinterpret_cast<uint16_t(*)[STAGE]>(stage_mem);
@@ -362,6 +363,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
+      if (!WHOLE_ROUNDS && c >= 32 * CH) break;
       const int64_t off = (int64_t)min(L - 1, 32 * u + r) * D + ch * 8;  // rows past the end are masked later
       pre_k[i] = *reinterpret_cast<const u32x4*>(kbase + off);
       pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
@@ -403,6 +405,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
+      if (!WHOLE_ROUNDS && c >= 32 * CH) break;
       *reinterpret_cast<u32x4*>(&stage[buf][r * KROW + (r >= 16 ? KHALF : 0) + ch * 8]) = pre_k[i];
       *reinterpret_cast<u32x4*>(&stage[buf][KSTAGE + r * VROW + ch * 8]) = pre_v[i];
     }
@@ -734,7 +737,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
-  const bool coop_built = H == 64 || H == 128 || H == 256;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
+  const bool coop_built = H == 64 || H == 96 || H == 128 || H == 256;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
   if (tiles > 4 && coop_built) {
     // prefill-sized: rows of a head share its K / V through LDS
     const int mode = !mask ? 0 : (mask_is_f32 ? 1 : 2);
@@ -742,7 +745,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
     dp.n_qgroups = (tiles + kCoopWaves * cnqt - 1) / (kCoopWaves * cnqt);
     // too few workgroups: halve their rows; so does the element-wise mask path at head_dim 128, whose
     // two-tile form does not fit the register file
-    if ((long long)B * N * dp.n_qgroups < compute_units() || (mode == 1 && H == 128)) {
+    if ((long long)B * N * dp.n_qgroups < compute_units() || (mode == 1 && (H == 128 || H == 96))) {
       cnqt = 1;
       dp.n_qgroups = (tiles + kCoopWaves - 1) / kCoopWaves;
     }
@@ -761,6 +764,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
 #define PACE_COOP_M(D_, Q_) \
   do { if (mode == 0) PACE_COOP(D_, Q_, 0); else if (mode == 1) PACE_COOP(D_, Q_, 1); else PACE_COOP(D_, Q_, 2); } while (0)
     if (H == 256) PACE_COOP_M(256, 1);
+    else if (H == 96) { if (cnqt == 2) PACE_COOP_M(96, 2); else PACE_COOP_M(96, 1); }
     else if (H == 128) { if (cnqt == 2) PACE_COOP_M(128, 2); else PACE_COOP_M(128, 1); }
     else { if (cnqt == 2) PACE_COOP_M(64, 2); else PACE_COOP_M(64, 1); }
 #undef PACE_COOP_M

@@ -81,6 +81,12 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     (1, 5, 300, 256, 96, "heads-bf16"),
     (1, 2, 90, 256, 41, "causal-short-bf16"),
     (1, 2, 80, 256, 70, "rows-masked-bf16"),
+    # head_dim 96 (a unit's chunks do not divide evenly over the workgroup's threads)
+    (1, 3, 200, 96, 333, "causal-bf16"),
+    (2, 32, 512, 96, 72, "causal-bf16"),
+    (1, 2, 100, 96, 96, "causal-f32"),
+    (2, 32, 300, 96, 50, None),
+    (1, 2, 90, 96, 41, "causal-short-bf16"),
 ])
 def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     from oracle.attention_ref import causal_mask_4d
