@@ -738,7 +738,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
   const bool coop_built = H == 64 || H == 96 || H == 128 || H == 256;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
-  if (tiles > 4 && coop_built) {
+  if ((tiles > 4 || (H == 256 && tiles > 1)) && coop_built) {
     // prefill-sized: rows of a head share its K / V through LDS
     const int mode = !mask ? 0 : (mask_is_f32 ? 1 : 2);
     int cnqt = H == 256 ? 1 : 2;  // (two tiles of head_dim 256 do not fit the register file)
