@@ -40,8 +40,11 @@ __global__ __launch_bounds__(64) void dense_mask_lines_kernel(const void* mask, 
 template <int D>
 constexpr int dense_split_waves() { return D > 128 ? 2 : 4; }
 
-template <int D, int NQT, bool HAS_MASK, bool ONCE>
-__global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : 2))) void dense_attn_mfma_kernel(
+// OCC: waves per SIMD the registers are budgeted for.  At head_dim 256 a wave with a SIMD to itself (OCC 1) spills
+// nothing and is the faster form while the launch has no more workgroups than fit at that rate; a launch with more
+// (decode steps of a batch) is bound by the loads in flight and gains from a second wave per SIMD.
+template <int D, int NQT, bool HAS_MASK, bool ONCE, int OCC = (D > 128 ? 1 : 2)>
+__global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_waves_per_eu(OCC))) void dense_attn_mfma_kernel(
     const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
   constexpr int MT = D / 16;
@@ -778,7 +781,13 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   const dim3 grid((unsigned)blocks), block(H > 128 ? 128 : 256);
   const bool m = mask != nullptr;
   const bool once = dp.n_qgroups == 1;
-#define PACE_DENSE1(D_, Q_, M_, O_) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_>), grid, block, 0, stream, dp)
+  // (head_dim 256: two waves per SIMD once there are more workgroups than compute units hold at one wave per SIMD)
+  const bool packed = H == 256 && blocks > 2ll * compute_units();
+#define PACE_DENSE1(D_, Q_, M_, O_)                                                                              \
+  do {                                                                                                          \
+    if (D_ == 256 && packed) hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_, 2>), grid, block, 0, stream, dp); \
+    else hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_>), grid, block, 0, stream, dp);                \
+  } while (0)
 #define PACE_DENSE(D_, Q_, M_) do { if (once) PACE_DENSE1(D_, Q_, M_, true); else PACE_DENSE1(D_, Q_, M_, false); } while (0)
   for_head_dim(H, [&](auto d) {
     constexpr int DIM = decltype(d)::value;
