@@ -186,6 +186,53 @@ __device__ __forceinline__ void load_mask_regs(MaskRegs<NQT>& mr, const PagedAtt
   }
 }
 
+// The same values as fetched, for a caller that fetches a unit ahead: converting them where they are loaded would
+// make the wave wait for the load there.  bf16: eight values in w[qt][0]; fp32: in w[qt][0], w[qt][1].  Columns the mask
+// does not have come as -inf.
+template <int NQT>
+struct MaskRaw {
+  u32x4 w[NQT][2];
+};
+template <int NQT>
+__device__ __forceinline__ void load_mask_raw(MaskRaw<NQT>& raw, const PagedAttnParams& p, const int64_t (&mask_off)[NQT], int t0, int g) {
+  const int base = t0 + 8 * g;
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    if (p.mask_is_f32) {
+      const float* line = static_cast<const float*>(p.mask) + mask_off[qt] + base;
+      if (base + 8 <= p.mask_len) {
+        raw.w[qt][0] = load16_unaligned(line), raw.w[qt][1] = load16_unaligned(line + 4);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) raw.w[qt][c >> 2][c & 3] = base + c < p.mask_len ? __float_as_uint(line[c]) : 0xff800000u;
+      }
+    } else {
+      const uint16_t* line = static_cast<const uint16_t*>(p.mask) + mask_off[qt] + base;
+      if (base + 8 <= p.mask_len) {
+        raw.w[qt][0] = load16_unaligned(line);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t lo = base + 2 * e < p.mask_len ? line[2 * e] : 0xff80u, hi = base + 2 * e + 1 < p.mask_len ? line[2 * e + 1] : 0xff80u;
+          raw.w[qt][0][e] = lo | (hi << 16);
+        }
+      }
+    }
+  }
+}
+template <int NQT>
+__device__ __forceinline__ void mask_regs_from_raw(MaskRegs<NQT>& mr, const MaskRaw<NQT>& raw, const PagedAttnParams& p) {
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    if (p.mask_is_f32) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) mr.a[qt][c] = fmaxf(__uint_as_float(raw.w[qt][c >> 2][c & 3]), kMaskFloor);
+    } else {
+      mask_line_from_bf16x8(raw.w[qt][0], mr.a[qt]);
+    }
+  }
+}
+
 // One wave looks over the columns [start, end) of a mask line (element offset `off` in `mask`): `last` = the last
 // column whose value is above the floor (-1: none; NaN counts as masked), `first_if_plain` = the first such column
 // if the line is plain -- exactly 0 on every column from there to `last`, which then are all above the floor -- and

@@ -97,25 +97,68 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
   const int n_units = min(units, u_begin + per_wave) - u_begin;
   UnitRegs<D> buf;
   MaskRegs<NQT> mregs;
-  for (int uu = 0; uu < n_units; ++uu) {
-    const int t0 = 32 * (u_begin + uu);
-    if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
-    // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g.. (clamped rows are masked later).
+  constexpr int CH = D / 8;            // chunks per row
+  constexpr int VCH = 32 * CH / 64;    // V chunks of a unit per lane
+  // A wave that has a SIMD to itself has the registers to fetch a unit ahead: its loads then travel while the unit
+  // before is worked on, instead of every unit waiting out its own memory latency with nothing else in flight.
+  constexpr bool AHEAD = OCC == 1;
+  // K: token 8*(n/4) + 4*tile + n%4 of the unit, dims 32*kk + 8g.. (clamped rows are masked later).
+  auto fetch_k = [&](int t0, u32x4 (&kx)[2][KK]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int tok = min(L - 1, t0 + 8 * (n >> 2) + 4 * t + (n & 3));
       const uint16_t* kp = kbase + (int64_t)tok * D + 8 * g;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = ONCE ? load16_stream(kp + kk * 32) : *reinterpret_cast<const u32x4*>(kp + kk * 32);
+      for (int kk = 0; kk < KK; ++kk) kx[t][kk] = ONCE ? load16_stream(kp + kk * 32) : *reinterpret_cast<const u32x4*>(kp + kk * 32);
     }
-    // V: the unit's 32 rows go to this wave's LDS stage (coalesced 16-byte chunks) ...
-    constexpr int CH = D / 8;  // chunks per row
+  };
+  // V: the unit's 32 rows, coalesced 16-byte chunks
+  auto fetch_v = [&](int t0, u32x4 (&vx)[VCH]) {
 #pragma unroll
-    for (int i = 0; i < 32 * CH / 64; ++i) {
+    for (int i = 0; i < VCH; ++i) {
       const int c = i * 64 + lane, r = c / CH, ch = c % CH;
-      const int tok = min(L - 1, t0 + r);
-      const uint16_t* vp = vbase + (int64_t)tok * D + ch * 8;
-      *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = ONCE ? load16_stream(vp) : *reinterpret_cast<const u32x4*>(vp);
+      const uint16_t* vp = vbase + (int64_t)min(L - 1, t0 + r) * D + ch * 8;
+      vx[i] = ONCE ? load16_stream(vp) : *reinterpret_cast<const u32x4*>(vp);
+    }
+  };
+  u32x4 k_next[AHEAD ? 2 : 1][AHEAD ? KK : 1], v_next[AHEAD ? VCH : 1];
+  MaskRaw<NQT> m_next;
+  if constexpr (AHEAD) {
+    if (n_units > 0) {
+      if (HAS_MASK) load_mask_raw<NQT>(m_next, p, st.mask_off, 32 * u_begin, g);
+      fetch_k(32 * u_begin, k_next);
+      fetch_v(32 * u_begin, v_next);
+    }
+  }
+  for (int uu = 0; uu < n_units; ++uu) {
+    const int t0 = 32 * (u_begin + uu);
+    // ... V goes to this wave's LDS stage ...
+    if constexpr (AHEAD) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) buf.k[t][kk] = k_next[t][kk];
+      if (HAS_MASK) mask_regs_from_raw<NQT>(mregs, m_next, p);
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int c = i * 64 + lane, r = c / CH, ch = c % CH;
+        *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = v_next[i];
+      }
+      if (uu + 1 < n_units) {
+        if (HAS_MASK) load_mask_raw<NQT>(m_next, p, st.mask_off, t0 + 32, g);
+        fetch_k(t0 + 32, k_next);
+        fetch_v(t0 + 32, v_next);
+      }
+    } else {
+      if (HAS_MASK) load_mask_regs<NQT>(mregs, p, st.mask_off, t0, g);  // travels with the unit's K / V
+      fetch_k(t0, buf.k);
+      u32x4 vx[VCH];
+      fetch_v(t0, vx);
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int c = i * 64 + lane, r = c / CH, ch = c % CH;
+        *reinterpret_cast<u32x4*>(stage + r * VROW + ch * 8) = vx[i];
+      }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
     __builtin_amdgcn_wave_barrier();
