@@ -876,6 +876,77 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
 #undef PACE_GO
 }
 
+// The same merge for rows cut into many partitions (a few long sequences spread over the whole GPU): the loop above
+// waits out a memory round trip per partition, twice.  Here a lane fetches the (max, sum) pair of partition
+// base + lane, so 64 pairs arrive together, and the partial outputs are fetched eight partitions at a time; the
+// sums are taken in the same order as above, from the same terms: the same bits.
+template <int D>
+__global__ __launch_bounds__(64) void paged_attn_merge_wide_kernel(const PagedAttnParams p) {
+  const int64_t row = blockIdx.x;  // (b, hq, s)
+  const int S = p.q_len;
+  const int s = (int)(row % S);
+  const int hq = (int)((row / S) % p.num_q_heads);
+  const int b = (int)(row / ((int64_t)S * p.num_q_heads));
+  const int lane = threadIdx.x;
+  int n_parts;
+  if (p.seq_parts) {
+    n_parts = p.seq_parts[b];
+  } else {
+    const int len = p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0);
+    n_parts = partition_count(len, p.part_tokens);
+  }
+  n_parts = min(max(n_parts, 1), p.max_parts);  // the workspace holds max_parts partials per row
+  const float* ml = p.part_ml + row * p.max_parts * 2;
+  const float* po = p.part_o + row * p.max_parts * D;
+  float M = kNegInf;
+  for (int base = 0; base < n_parts; base += 64) {
+    const float m_i = base + lane < n_parts ? ml[2 * (base + lane)] : kNegInf;
+    M = fmaxf(M, m_i);
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o *= 2) M = fmaxf(M, __shfl_xor(M, o, 64));
+  const float m_use = (M == kNegInf) ? 0.f : M;
+  constexpr int PASSES = (D + 127) / 128;  // a lane owns the dim pairs 2 * lane + 128 * pass that exist
+  float acc[PASSES][2];
+#pragma unroll
+  for (int e = 0; e < PASSES; ++e) acc[e][0] = acc[e][1] = 0.f;
+  float L = 0.f;
+  const int d0 = 2 * lane;
+  for (int base = 0; base < n_parts; base += 64) {
+    const bool mine = base + lane < n_parts;
+    const u32x2 pair = mine ? *reinterpret_cast<const u32x2*>(ml + 2 * (base + lane)) : u32x2{0xff800000u, 0u};
+    const float w_mine = __builtin_amdgcn_exp2f(__uint_as_float(pair[0]) - m_use), l_mine = __uint_as_float(pair[1]);
+    const int here = min(64, n_parts - base);
+    for (int j0 = 0; j0 < here; j0 += 8) {
+      u32x2 v[8][PASSES];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < PASSES; ++e) {
+          v[j][e] = u32x2{0u, 0u};
+          if (j0 + j < here && d0 + 128 * e < D) v[j][e] = *reinterpret_cast<const u32x2*>(po + (int64_t)(base + j0 + j) * D + d0 + 128 * e);
+        }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (j0 + j < here) {  // uniform
+          const float w = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w_mine), j0 + j));
+          const float l = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(l_mine), j0 + j));
+          L += w * l;
+#pragma unroll
+          for (int e = 0; e < PASSES; ++e) {
+            acc[e][0] += w * __uint_as_float(v[j][e][0]);
+            acc[e][1] += w * __uint_as_float(v[j][e][1]);
+          }
+        }
+      }
+    }
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + d0;
+#pragma unroll
+  for (int e = 0; e < PASSES; ++e)
+    if (d0 + 128 * e < D) *reinterpret_cast<uint32_t*>(op + 128 * e) = pack_bf16x2(acc[e][0] * inv, acc[e][1] * inv);
+}
 template <int D>
 static bool launch_shape(const Shape& sh, const PagedAttnParams& p, bool has_mask, hipStream_t s) {
 #define PACE_TRY(NQT_, NW_, OCC_, MAX_)                                          \
@@ -1137,7 +1208,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
     PACE_REQUIRE(rows_total < ((size_t)1 << 31), "%s: too many query rows", who);
     for_head_dim(pool->head_dim, [&](auto d) {
-      hipLaunchKernelGGL(paged_attn_merge_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+      if (p.max_parts > 8) hipLaunchKernelGGL(paged_attn_merge_wide_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+      else hipLaunchKernelGGL(paged_attn_merge_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
     });
     PACE_HIP_CHECK(hipGetLastError());
   }
