@@ -878,16 +878,20 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
 
 // The same merge for rows cut into many partitions (a few long sequences spread over the whole GPU): the loop above
 // waits out a memory round trip per partition, twice.  Here a lane fetches the (max, sum) pair of partition
-// base + lane, so 64 pairs arrive together, and the partial outputs are fetched eight partitions at a time; the
-// sums are taken in the same order as above, from the same terms: the same bits.
+// base + lane, so 64 pairs arrive together, the partial outputs are fetched eight partitions at a time, and the
+// four waves of the workgroup take those groups of eight in turn; wave 0 adds the four partial results in wave
+// order.  (The sum is therefore taken in another order than above: same result to rounding, the same bits from
+// call to call.)
 template <int D>
-__global__ __launch_bounds__(64) void paged_attn_merge_wide_kernel(const PagedAttnParams p) {
+__global__ __launch_bounds__(256) void paged_attn_merge_wide_kernel(const PagedAttnParams p) {
+  constexpr int PASSES = (D + 127) / 128;  // a lane owns the dim pairs 2 * lane + 128 * pass that exist
+  __shared__ float part_sum[3][64][2 * PASSES + 1];
   const int64_t row = blockIdx.x;  // (b, hq, s)
   const int S = p.q_len;
   const int s = (int)(row % S);
   const int hq = (int)((row / S) % p.num_q_heads);
   const int b = (int)(row / ((int64_t)S * p.num_q_heads));
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int n_parts;
   if (p.seq_parts) {
     n_parts = p.seq_parts[b];
@@ -906,7 +910,6 @@ __global__ __launch_bounds__(64) void paged_attn_merge_wide_kernel(const PagedAt
 #pragma unroll
   for (int o = 1; o < 64; o *= 2) M = fmaxf(M, __shfl_xor(M, o, 64));
   const float m_use = (M == kNegInf) ? 0.f : M;
-  constexpr int PASSES = (D + 127) / 128;  // a lane owns the dim pairs 2 * lane + 128 * pass that exist
   float acc[PASSES][2];
 #pragma unroll
   for (int e = 0; e < PASSES; ++e) acc[e][0] = acc[e][1] = 0.f;
@@ -917,7 +920,7 @@ __global__ __launch_bounds__(64) void paged_attn_merge_wide_kernel(const PagedAt
     const u32x2 pair = mine ? *reinterpret_cast<const u32x2*>(ml + 2 * (base + lane)) : u32x2{0xff800000u, 0u};
     const float w_mine = __builtin_amdgcn_exp2f(__uint_as_float(pair[0]) - m_use), l_mine = __uint_as_float(pair[1]);
     const int here = min(64, n_parts - base);
-    for (int j0 = 0; j0 < here; j0 += 8) {
+    for (int j0 = 8 * wave; j0 < here; j0 += 32) {
       u32x2 v[8][PASSES];
 #pragma unroll
       for (int j = 0; j < 8; ++j)
@@ -940,6 +943,19 @@ __global__ __launch_bounds__(64) void paged_attn_merge_wide_kernel(const PagedAt
         }
       }
     }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < PASSES; ++e) part_sum[wave - 1][lane][2 * e] = acc[e][0], part_sum[wave - 1][lane][2 * e + 1] = acc[e][1];
+    part_sum[wave - 1][lane][2 * PASSES] = L;
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+#pragma unroll
+    for (int e = 0; e < PASSES; ++e) acc[e][0] += part_sum[w][lane][2 * e], acc[e][1] += part_sum[w][lane][2 * e + 1];
+    L += part_sum[w][lane][2 * PASSES];
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   uint16_t* op = p.out + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)s * p.o_ss + d0;
@@ -1208,7 +1224,7 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     const size_t rows_total = (size_t)a->batch * a->num_q_heads * a->q_len;
     PACE_REQUIRE(rows_total < ((size_t)1 << 31), "%s: too many query rows", who);
     for_head_dim(pool->head_dim, [&](auto d) {
-      if (p.max_parts > 8) hipLaunchKernelGGL(paged_attn_merge_wide_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
+      if (p.max_parts > 8) hipLaunchKernelGGL(paged_attn_merge_wide_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(256), 0, s, p);
       else hipLaunchKernelGGL(paged_attn_merge_kernel<decltype(d)::value>, dim3((unsigned)rows_total), dim3(64), 0, s, p);
     });
     PACE_HIP_CHECK(hipGetLastError());
