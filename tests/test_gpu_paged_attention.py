@@ -526,6 +526,32 @@ def test_very_long_context_single_sequence(device):
     assert_attention_close(cache.attend(q3.to(device)), model.attention(q3, 4), "70k verify")
 
 
+@pytest.mark.parametrize("D,hkv,n_rep,lens,partition,S", [
+    (128, 2, 4, [4100, 900], 64, 1),     # 65 partitions: more than one round of 64 (max, sum) pairs
+    (128, 1, 8, [833], 64, 1),           # 14 partitions: a last group of fewer than eight
+    (64, 2, 7, [3000], 128, 1),          # head_dim 64: half the lanes own dims
+    (256, 2, 2, [2500, 64], 128, 1),     # head_dim 256: two dim pairs per lane; a sequence of one partition beside it
+    (128, 2, 4, [2000, 1500], 128, 5),   # several query tokens per row group
+])
+def test_rows_cut_into_many_partitions(device, D, hkv, n_rep, lens, partition, S):
+    """More than eight partitions per row: the merge that fetches the partials in groups, four waves per row."""
+    B = len(lens)
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=sum(lens) + D, partition=partition)
+    if S == 1:
+        q = seeded_q(31, B, hkv * n_rep, 1, D)
+        out, ref = cache.attend(q.to(device)), model.attention(q, n_rep)
+    else:
+        k1, v1 = seeded_kv(32, B, hkv, S, D)
+        q = seeded_q(33, B, hkv * n_rep, S, D)
+        cache.update_cache(k1.to(device), v1.to(device), 2)
+        model.append(k1, v1)
+        out, ref = cache.attend(q.to(device)), model.attention(q, n_rep)
+    assert_attention_close(out, ref, f"many partitions D={D} lens={lens}")
+    again = cache.attend(q.to(device)) if S == 1 else None
+    if again is not None:
+        assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+
+
 @pytest.mark.parametrize("seed", range(5))
 def test_paged_attention_random_batches_masks_and_partitions(device, seed):
     """Seeded sweep: ragged lengths, query lengths on both sides of the kernel's tile limits, forced
