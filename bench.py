@@ -575,7 +575,7 @@ def wl_dense_prefill(torch, dev, args):
     every (row, key) pair is computed: 4*B*N*S*L*H flop."""
     import pace_mi355.ops  # noqa: F401  (defines the op)
 
-    B, N, S, L, H = 8, 32, 2048, 2048, 128
+    B, N, S, L, H = args.batch or 8, args.heads or 32, args.queries or 2048, args.context or 2048, args.head_dim or 128
     g = torch.Generator(device=dev).manual_seed(10)
     q, k, v = (_randn_bf16(torch, (B, N, n, H), g, dev) for n in (S, L, L))
     mask = torch.zeros(B, 1, S, L, device=dev, dtype=torch.bfloat16)
@@ -598,9 +598,10 @@ def wl_dense_prefill(torch, dev, args):
     once = 2 * (q.numel() * 2 + k.numel() + v.numel()) + B * S * L * 2  # q, out, K, V and the mask read once
     tflops = flops / (attn_ms * 1e-3) / 1e12
     return result_line(
-        args, "dense op at a prefill shape: batch 8, 32 heads, 2048 queries x 2048 keys, head_dim 128, additive causal mask "
+        args, f"dense op at a prefill shape: batch {B}, {N} heads, {S} queries x {L} keys, head_dim {H}, additive causal mask "
         "[B,1,S,L]; step = one torch.ops.pace.attention call (output allocation included)", once, B * S, dt,
-        {"bound": "mfma", "kernel": "dense_attn_coop_kernel<128,2,2>", "achieved": round(tflops, 1),
+        {"bound": "mfma", "kernel": "dense_attn_coop_kernel<128,2,2>" if (H, S) == (128, 2048) else f"bf16 dense op, head_dim {H}, {S} query rows",
+         "achieved": round(tflops, 1),
          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5),
          "tflops_if_all_pairs_counted": round(all_pairs / (attn_ms * 1e-3) / 1e12, 1)})
@@ -774,6 +775,9 @@ def main() -> int:
                          "MultiHeadAttention; graph: the api calls captured once into a HIP graph and replayed per step")
     ap.add_argument("--batch", type=int, default=0, help="decode and prefill workloads: override the batch size (latency studies)")
     ap.add_argument("--context", type=int, default=0, help="decode and prefill workloads: override the context length (prefill: the cached tokens)")
+    ap.add_argument("--heads", type=int, default=0, help="dense-prefill: number of heads (default 32)")
+    ap.add_argument("--head-dim", type=int, default=0, dest="head_dim", help="dense-prefill: head size (default 128)")
+    ap.add_argument("--queries", type=int, default=0, help="dense-prefill: query rows per head (default 2048; --context gives the keys)")
     ap.add_argument("--layers", type=int, default=4,
                     help="decode workloads: distinct layer pools (own block permutation each) the timed steps rotate over; "
                          "4 x 1.07 GB is 16 times the last-level cache, 1 re-reads one pool every step")
