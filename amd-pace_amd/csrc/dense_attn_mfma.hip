@@ -18,6 +18,7 @@ struct DenseMfmaParams {
   const uint16_t* k;
   const uint16_t* v;
   int32_t B, N, S, L;
+  int32_t H;  // the tensors' head size: the kernel's D, or less (a multiple of 8) where the kernel is built PADDED
   int32_t mB, mN, mS;
   int32_t n_qgroups;
   // Optional summary of the mask, one entry per mask line ((mb * mN + mn) * mS + ms), written by
@@ -43,7 +44,9 @@ constexpr int dense_split_waves() { return D > 128 ? 2 : 4; }
 // OCC: waves per SIMD the registers are budgeted for.  At head_dim 256 a wave with a SIMD to itself (OCC 1) spills
 // nothing and is the faster form while the launch has no more workgroups than fit at that rate; a launch with more
 // (decode steps of a batch) is bound by the loads in flight and gains from a second wave per SIMD.
-template <int D, int NQT, bool HAS_MASK, bool ONCE, int OCC = (D > 128 ? 1 : 2)>
+// PADDED: the tensors' head size is dp.H < D, a multiple of 8: rows are dp.H elements apart, the 16-byte chunks past
+// dp.H read as zero (they change neither a score nor an output dim that exists) and are not written.
+template <int D, int NQT, bool HAS_MASK, bool ONCE, int OCC = (D > 128 ? 1 : 2), bool PADDED = false>
 __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_waves_per_eu(OCC))) void dense_attn_mfma_kernel(
     const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
@@ -60,8 +63,9 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
   const int head = (blockIdx.x / dp.n_qgroups) % dp.N;
   const int b = blockIdx.x / (dp.n_qgroups * dp.N);
   const int L = dp.L, S = dp.S;
-  const uint16_t* kbase = dp.k + ((int64_t)b * dp.N + head) * (int64_t)L * D;
-  const uint16_t* vbase = dp.v + ((int64_t)b * dp.N + head) * (int64_t)L * D;
+  const int RS = PADDED ? dp.H : D;  // row stride of the tensors, in elements
+  const uint16_t* kbase = dp.k + ((int64_t)b * dp.N + head) * (int64_t)L * RS;
+  const uint16_t* vbase = dp.v + ((int64_t)b * dp.N + head) * (int64_t)L * RS;
   uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + wave * STAGE;
 
   u32x4 qreg[NQT][KK];
@@ -81,11 +85,11 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
     }
     st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
-    const uint16_t* qp = p.q + (((int64_t)b * dp.N + head) * S + (valid ? s : 0)) * D + 8 * g;
+    const uint16_t* qp = p.q + (((int64_t)b * dp.N + head) * S + (valid ? s : 0)) * RS + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       u32x4 z = {0u, 0u, 0u, 0u};
-      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
+      qreg[qt][kk] = (valid && (!PADDED || 32 * kk + 8 * g < dp.H)) ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
     }
 #pragma unroll
     for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -107,9 +111,12 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int tok = min(L - 1, t0 + 8 * (n >> 2) + 4 * t + (n & 3));
-      const uint16_t* kp = kbase + (int64_t)tok * D + 8 * g;
+      const uint16_t* kp = kbase + (int64_t)tok * RS + 8 * g;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kx[t][kk] = ONCE ? load16_stream(kp + kk * 32) : *reinterpret_cast<const u32x4*>(kp + kk * 32);
+      for (int kk = 0; kk < KK; ++kk) {
+        kx[t][kk] = u32x4{0u, 0u, 0u, 0u};
+        if (!PADDED || 32 * kk + 8 * g < dp.H) kx[t][kk] = ONCE ? load16_stream(kp + kk * 32) : *reinterpret_cast<const u32x4*>(kp + kk * 32);
+      }
     }
   };
   // V: the unit's 32 rows, coalesced 16-byte chunks
@@ -117,8 +124,9 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
       const int c = i * 64 + lane, r = c / CH, ch = c % CH;
-      const uint16_t* vp = vbase + (int64_t)min(L - 1, t0 + r) * D + ch * 8;
-      vx[i] = ONCE ? load16_stream(vp) : *reinterpret_cast<const u32x4*>(vp);
+      const uint16_t* vp = vbase + (int64_t)min(L - 1, t0 + r) * RS + ch * 8;
+      vx[i] = u32x4{0u, 0u, 0u, 0u};
+      if (!PADDED || ch * 8 < dp.H) vx[i] = ONCE ? load16_stream(vp) : *reinterpret_cast<const u32x4*>(vp);
     }
   };
   u32x4 k_next[AHEAD ? 2 : 1][AHEAD ? KK : 1], v_next[AHEAD ? VCH : 1];
@@ -227,13 +235,13 @@ __global__ __launch_bounds__(64 * dense_split_waves<D>()) __attribute__((amdgpu_
     if (row_s[qt] >= S) continue;
     const float l = st.l[qt];
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* op = p.out + (((int64_t)b * dp.N + head) * S + row_s[qt]) * D + 4 * g;
+    uint16_t* op = p.out + (((int64_t)b * dp.N + head) * S + row_s[qt]) * RS + 4 * g;
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       u32x2 w;
       w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
       w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
-      *reinterpret_cast<u32x2*>(op + 16 * j) = w;
+      if (!PADDED || 16 * j + 4 * g < dp.H) *reinterpret_cast<u32x2*>(op + 16 * j) = w;
     }
   }
 }
@@ -337,7 +345,7 @@ __device__ __forceinline__ void coop_stage_turn(const u32x4* cur, u32x4* nxt, co
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int D, int NQT, int MASK>
+template <int D, int NQT, int MASK, bool PADDED = false>
 __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu(2))) void dense_attn_coop_kernel(
     const DenseMfmaParams dp) {
   constexpr int KK = D / 32;
@@ -369,8 +377,9 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
   if (pair >= dp.B * dp.N) return;  // uniform over the workgroup
   const int b = pair / dp.N, head = pair % dp.N;
   const int L = dp.L, S = dp.S;
-  const uint16_t* kbase = dp.k + (int64_t)pair * L * D;
-  const uint16_t* vbase = dp.v + (int64_t)pair * L * D;
+  const int RS = PADDED ? dp.H : D;  // row stride of the tensors, in elements (PADDED: see dense_attn_mfma_kernel)
+  const uint16_t* kbase = dp.k + (int64_t)pair * L * RS;
+  const uint16_t* vbase = dp.v + (int64_t)pair * L * RS;
   const int row0 = (rg * kCoopWaves + wave) * (NQT * 16);
   const bool wave_has_rows = row0 < S;
 
@@ -391,11 +400,11 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     }
     st.m[qt] = kNegInf, st.m_top[qt] = kNegInf, st.m_neg[qt] = 0.f;
     st.l[qt] = 0.f;
-    const uint16_t* qp = p.q + ((int64_t)pair * S + (valid ? s : 0)) * D + 8 * g;
+    const uint16_t* qp = p.q + ((int64_t)pair * S + (valid ? s : 0)) * RS + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       const u32x4 z = {0u, 0u, 0u, 0u};
-      qreg[qt][kk] = valid ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
+      qreg[qt][kk] = (valid && (!PADDED || 32 * kk + 8 * g < dp.H)) ? *reinterpret_cast<const u32x4*>(qp + kk * 32) : z;
     }
 #pragma unroll
     for (int j = 0; j < MT; ++j) st.o[qt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -410,9 +419,12 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + i * 64 * kCoopWaves, r = c / CH, ch = c % CH;
       if (!WHOLE_ROUNDS && c >= 32 * CH) break;
-      const int64_t off = (int64_t)min(L - 1, 32 * u + r) * D + ch * 8;  // rows past the end are masked later
-      pre_k[i] = *reinterpret_cast<const u32x4*>(kbase + off);
-      pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
+      const int64_t off = (int64_t)min(L - 1, 32 * u + r) * RS + ch * 8;  // rows past the end are masked later
+      pre_k[i] = pre_v[i] = u32x4{0u, 0u, 0u, 0u};
+      if (!PADDED || ch * 8 < dp.H) {
+        pre_k[i] = *reinterpret_cast<const u32x4*>(kbase + off);
+        pre_v[i] = *reinterpret_cast<const u32x4*>(vbase + off);
+      }
     }
     if (MODE == 2) {
       const int tok = 32 * u + 8 * g;
@@ -756,22 +768,26 @@ __global__ __launch_bounds__(64 * kCoopWaves) __attribute__((amdgpu_waves_per_eu
     l += xor_lanes(l, 32);
     if (row_s[qt] >= S) continue;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* op = p.out + ((int64_t)pair * S + row_s[qt]) * D + 4 * g;
+    uint16_t* op = p.out + ((int64_t)pair * S + row_s[qt]) * RS + 4 * g;
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       u32x2 w;
       w[0] = pack_bf16x2(st.o[qt][j][0] * inv, st.o[qt][j][1] * inv);
       w[1] = pack_bf16x2(st.o[qt][j][2] * inv, st.o[qt][j][3] * inv);
-      *reinterpret_cast<u32x2*>(op + 16 * j) = w;
+      if (!PADDED || 16 * j + 4 * g < dp.H) *reinterpret_cast<u32x2*>(op + 16 * j) = w;
     }
   }
 }
 
 // Launches the dense bf16 kernel; returns false when the shape is not one it handles.
 // workspace (optional): room for the summary of the mask, two ints per mask line (dense_mfma_workspace_bytes).
-bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H,
+bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, int B, int N, int S, int L, int H_real,
                        const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, void* workspace,
                        size_t workspace_bytes, hipStream_t stream) {
+  // Head sizes between 64 and 96 that are a multiple of 8 (OPT-2.7B's 80) run in the 96 build, their rows read as if
+  // padded with zeros (PADDED); `scale` is the caller's, of the real head size.
+  const bool padded = H_real > 64 && H_real < 96 && H_real % 8 == 0;
+  const int H = padded ? 96 : H_real;
   if ((H != 64 && H != 96 && H != 128 && H != 256) || L < 1) return false;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(out) & 7u)) return false;
   DenseMfmaParams dp = {};
@@ -781,7 +797,7 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
   dp.base.scale_log2 = scale * kLog2e;
   dp.base.scale = scale;
   dp.k = static_cast<const uint16_t*>(k), dp.v = static_cast<const uint16_t*>(v);
-  dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.mB = mB, dp.mN = mN, dp.mS = mS;
+  dp.B = B, dp.N = N, dp.S = S, dp.L = L, dp.H = H_real, dp.mB = mB, dp.mN = mN, dp.mS = mS;
   const int tiles = (S + 15) / 16;
   const bool coop_built = H == 64 || H == 96 || H == 128 || H == 256;  // other head sizes: the split-L kernel, one launch of as many row groups as it takes
   if ((tiles > 4 || (H == 256 && tiles > 1)) && coop_built) {
@@ -810,6 +826,12 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
 #define PACE_COOP_M(D_, Q_) \
   do { if (mode == 0) PACE_COOP(D_, Q_, 0); else if (mode == 1) PACE_COOP(D_, Q_, 1); else PACE_COOP(D_, Q_, 2); } while (0)
     if (H == 256) PACE_COOP_M(256, 1);
+    else if (padded) {
+#define PACE_COOP_P(Q_, M_) hipLaunchKernelGGL((dense_attn_coop_kernel<96, Q_, M_, true>), cgrid, cblock, 0, stream, dp)
+      if (cnqt == 2) { if (mode == 0) PACE_COOP_P(2, 0); else if (mode == 1) PACE_COOP_P(2, 1); else PACE_COOP_P(2, 2); }
+      else { if (mode == 0) PACE_COOP_P(1, 0); else if (mode == 1) PACE_COOP_P(1, 1); else PACE_COOP_P(1, 2); }
+#undef PACE_COOP_P
+    }
     else if (H == 96) { if (cnqt == 2) PACE_COOP_M(96, 2); else PACE_COOP_M(96, 1); }
     else if (H == 128) { if (cnqt == 2) PACE_COOP_M(128, 2); else PACE_COOP_M(128, 1); }
     else { if (cnqt == 2) PACE_COOP_M(64, 2); else PACE_COOP_M(64, 1); }
@@ -832,6 +854,17 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
     else hipLaunchKernelGGL((dense_attn_mfma_kernel<D_, Q_, M_, O_>), grid, block, 0, stream, dp);                \
   } while (0)
 #define PACE_DENSE(D_, Q_, M_) do { if (once) PACE_DENSE1(D_, Q_, M_, true); else PACE_DENSE1(D_, Q_, M_, false); } while (0)
+  if (padded) {
+#define PACE_DENSE_P(Q_, M_)                                                                                              \
+  do {                                                                                                                    \
+    if (once) hipLaunchKernelGGL((dense_attn_mfma_kernel<96, Q_, M_, true, 2, true>), grid, block, 0, stream, dp);         \
+    else hipLaunchKernelGGL((dense_attn_mfma_kernel<96, Q_, M_, false, 2, true>), grid, block, 0, stream, dp);             \
+  } while (0)
+    if (nqt == 2) { if (m) PACE_DENSE_P(2, true); else PACE_DENSE_P(2, false); }
+    else { if (m) PACE_DENSE_P(1, true); else PACE_DENSE_P(1, false); }
+#undef PACE_DENSE_P
+    return true;
+  }
   for_head_dim(H, [&](auto d) {
     constexpr int DIM = decltype(d)::value;
     if constexpr (DIM != 256) {

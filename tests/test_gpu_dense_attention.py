@@ -87,6 +87,14 @@ def test_dense_op_mask_broadcast_and_mixed_dtypes(device, mshape):
     (1, 2, 100, 96, 96, "causal-f32"),
     (2, 32, 300, 96, 50, None),
     (1, 2, 90, 96, 41, "causal-short-bf16"),
+    # head sizes between 64 and 96 (OPT-2.7B's 80): the 96 build reading the rows as if padded with zeros
+    (1, 3, 200, 80, 333, "causal-bf16"),
+    (2, 4, 130, 72, 264, "causal-bf16"),
+    (1, 2, 100, 88, 96, "causal-f32"),
+    (2, 32, 300, 80, 50, None),
+    (1, 2, 90, 80, 41, "causal-short-bf16"),
+    (2, 3, 40, 80, 700, "rows-bf16"),          # few query rows: the kernel that splits the keys
+    (2, 3, 1, 88, 333, "rows-bf16"),
 ])
 def test_dense_prefill_shapes(device, B, N, S, H, L, mask):
     from oracle.attention_ref import causal_mask_4d
