@@ -36,21 +36,26 @@ class BlockAllocator:
         self._n_free = self.num_blocks
         self._is_free = np.ones(self.num_blocks, dtype=bool)
         self.refs = np.zeros(self.num_blocks, dtype=np.int32)
+        self._order = np.zeros(self.num_blocks, dtype=np.int32)  # scratch of free_in_turn
 
     @property
     def num_free(self) -> int:
         return self._n_free
 
     def allocate(self, n: int) -> List[int]:
+        return self.allocate_array(n).tolist()
+
+    def allocate_array(self, n: int) -> np.ndarray:
+        """``n`` blocks off the top of the stack, in the order ``n`` single allocations would hand them out."""
         if n > self._n_free:
             raise MemoryError(f"KV block pool exhausted: need {n} blocks, {self._n_free} free of {self.num_blocks}")
         if n == 0:
-            return []
+            return np.zeros(0, dtype=np.int32)
         out = self._stack[self._n_free - n:self._n_free][::-1].copy()
         self._n_free -= n
         self._is_free[out] = False
         self.refs[out] = 1
-        return out.tolist()
+        return out
 
     def share(self, ids: Iterable[int]) -> None:
         """One more owner for each of ``ids`` (an id may occur several times)."""
@@ -78,6 +83,35 @@ class BlockAllocator:
             self._stack[self._n_free:self._n_free + gone.size] = gone
             self._n_free += gone.size
 
+    def free_in_turn(self, arr: np.ndarray) -> None:
+        """``free`` of each id of ``arr`` one after the other, in one go: a block that loses several owners here
+        returns to the free list where its last owner drops it."""
+        arr = np.asarray(arr, dtype=np.int64)
+        if not arr.size:
+            return
+        if self._is_free[arr].any():
+            raise ValueError(f"block {int(arr[self._is_free[arr]][0])} freed twice")
+        if (self.refs[arr] == 1).all():
+            # no block here has another owner (the usual case: no forked sequences): each returns as it is listed.
+            # An id listed twice would be a block freed twice: the second write of its position shows it.
+            self._order[arr] = np.arange(arr.size, dtype=np.int32)
+            if (self._order[arr] != np.arange(arr.size, dtype=np.int32)).any():
+                raise ValueError("a block with one owner freed twice")
+            self.refs[arr] = 0
+            gone = arr
+        else:
+            np.subtract.at(self.refs, arr, 1)
+            if (self.refs[arr] < 0).any():
+                raise ValueError(f"block {int(arr[self.refs[arr] < 0][0])} freed twice")
+            gone = arr[self.refs[arr] == 0]
+            if gone.size:
+                _, last = np.unique(gone[::-1], return_index=True)  # an id listed twice is pushed once, where it occurs last
+                gone = gone[np.sort(gone.size - 1 - last)]
+        if gone.size:
+            self._is_free[gone] = True
+            self._stack[self._n_free:self._n_free + gone.size] = gone
+            self._n_free += gone.size
+
     def take(self, ids: Iterable[int]) -> None:
         """Mark specific ids as used (compaction destinations)."""
         want = np.unique(np.asarray(list(ids), dtype=np.int64))
@@ -100,6 +134,15 @@ class BlockAllocator:
 
     def free_ids(self) -> np.ndarray:
         return np.nonzero(self._is_free)[0]
+
+
+def _ragged_cells(first: np.ndarray, count: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """Row and column indices of cells ``first[b] .. first[b] + count[b] - 1`` of every row ``b``, row by row."""
+    count = np.asarray(count, dtype=np.int64)
+    rows = np.repeat(np.arange(count.size), count)
+    starts = np.cumsum(count) - count
+    cols = np.arange(int(count.sum())) - np.repeat(starts, count) + np.repeat(np.asarray(first, dtype=np.int64), count)
+    return rows, cols
 
 
 class PagedState:
@@ -161,23 +204,26 @@ class PagedState:
         """Give every sequence enough blocks to hold ``lens[b]`` tokens."""
         need = (lens + BLOCK - 1) // BLOCK
         self._grow_table(int(need.max(initial=0)))
-        for b in np.nonzero(need > self.n_blocks)[0]:
-            have, want = int(self.n_blocks[b]), int(need[b])
-            self.table[b, have:want] = self.allocator.allocate(want - have)
-            self.n_blocks[b] = want
+        grow = np.maximum(need - self.n_blocks, 0)
+        total = int(grow.sum())
+        if total:
+            # every sequence's new blocks in one allocation, in the order one allocation per sequence would give them
+            rows, cols = _ragged_cells(self.n_blocks, grow)
+            self.table[rows, cols] = self.allocator.allocate_array(total)
+            self.n_blocks = np.maximum(self.n_blocks, need).astype(self.n_blocks.dtype)
             self._table_dirty = True
         self.min_capacity = self._min_blocks() * BLOCK
 
     def release_beyond(self, lens: np.ndarray) -> int:
         """Free the blocks no token of ``lens`` touches any more; returns how many."""
         need = (lens + BLOCK - 1) // BLOCK
-        freed = 0
-        for b in np.nonzero(need < self.n_blocks)[0]:
-            have, want = int(self.n_blocks[b]), int(need[b])
-            self.allocator.free(self.table[b, want:have].tolist())
-            self.table[b, want:have] = 0
-            self.n_blocks[b] = want
-            freed += have - want
+        drop = np.maximum(self.n_blocks - need, 0)
+        freed = int(drop.sum())
+        if freed:
+            rows, cols = _ragged_cells(np.minimum(self.n_blocks, need), drop)
+            self.allocator.free_in_turn(self.table[rows, cols])
+            self.table[rows, cols] = 0
+            self.n_blocks = np.minimum(self.n_blocks, need).astype(self.n_blocks.dtype)
             self._table_dirty = True
         if freed:
             self.table_version += 1

@@ -207,6 +207,59 @@ def test_capacity_release_and_slots():
         st.ensure_capacity(np.array([16, 16, 2000]))
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_capacity_changes_over_the_batch_match_one_sequence_at_a_time(seed):
+    """ensure_capacity / release_beyond handle the whole batch in one allocation / one release: the block ids every
+    sequence ends up with, the reference counts and the order of the free list are those of taking the sequences
+    one by one (one allocate() or free() per sequence, in batch order), forks included."""
+    rng = np.random.default_rng(seed)
+    B = 7
+    st = PagedState(B, 64, 400, torch.device("cpu"))
+    ref = PagedState(B, 64, 400, torch.device("cpu"))
+
+    def grow_one_by_one(state, lens):
+        need = (lens + 15) // 16
+        state._grow_table(int(need.max(initial=0)))
+        for b in range(B):
+            have, want = int(state.n_blocks[b]), int(need[b])
+            if want > have:
+                state.table[b, have:want] = state.allocator.allocate(want - have)
+                state.n_blocks[b] = want
+
+    def shrink_one_by_one(state, lens):
+        need = (lens + 15) // 16
+        for b in range(B):
+            have, want = int(state.n_blocks[b]), int(need[b])
+            if want < have:
+                state.allocator.free(state.table[b, want:have].tolist())
+                state.table[b, want:have] = 0
+                state.n_blocks[b] = want
+
+    lens = np.zeros(B, dtype=np.int64)
+    for step in range(60):
+        kind = rng.integers(0, 4)
+        if kind <= 1:  # some sequences grow
+            lens = lens + rng.integers(0, 90, size=B) * (rng.random(B) < 0.7)
+            st.ensure_capacity(lens)
+            grow_one_by_one(ref, lens)
+        elif kind == 2:  # some shrink (rollback, or a sequence that ends)
+            lens = (lens * rng.choice([0.0, 0.5, 1.0], size=B)).astype(np.int64)
+            st.release_beyond(lens)
+            shrink_one_by_one(ref, lens)
+        else:  # beam step: every row continues some source row (blocks shared until written)
+            src = rng.integers(0, B, size=B).tolist()
+            st.fork(src)
+            ref.fork(src)
+            lens = lens[src]
+        n = st.allocator.num_free
+        assert n == ref.allocator.num_free
+        assert st.allocator._stack[:n].tolist() == ref.allocator._stack[:n].tolist()
+        assert st.allocator.refs.tolist() == ref.allocator.refs.tolist()
+        assert st.n_blocks.tolist() == ref.n_blocks.tolist()
+        for b in range(B):
+            assert st.table[b, : st.n_blocks[b]].tolist() == ref.table[b, : ref.n_blocks[b]].tolist()
+
+
 def test_table_grows_on_demand():
     st = PagedState(1, 16, 300, torch.device("cpu"))
     st.ensure_capacity(np.array([16 * 200]))
