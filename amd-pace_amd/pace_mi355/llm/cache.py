@@ -272,12 +272,12 @@ class PagedKVCache(KVCacheBase):
             if rope is not None:
                 raise NotImplementedError("rotary embedding with a zero-padded head size")
             k, v = (torch.nn.functional.pad(t, (0, self.head_dim - self.model_dim)) for t in (k, v))
-        if k.stride(3) != 1 or v.stride(3) != 1 or k.stride() != v.stride() or any(s % 8 for s in k.stride()[:3]):
+        ks = k.stride()
+        if ks[3] != 1 or ks != v.stride() or ks[0] % 8 or ks[1] % 8 or ks[2] % 8:
             k, v = k.contiguous(), v.contiguous()
         head_step = h_in // self.num_kv_heads  # de-duplicate a repeat_kv-expanded input
         st = self.state
         lib = nat.load()
-        stream = nat.current_stream_ptr()
         if self._graph is not None and counts is None and self.fuse_append and T <= 32 and self._pending is None:
             # a step of a decode graph: blocks and table were prepared for every step; the append rides in the
             # attention launch, and the lengths advance on the device
@@ -308,7 +308,7 @@ class PagedKVCache(KVCacheBase):
             nat.check(
                 lib.pace_kv_append(
                     ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
-                    B, T, slots.data_ptr(), stream,
+                    B, T, slots.data_ptr(), nat.current_stream_ptr(),
                 )
             )
         self.lens = new_lens
@@ -488,8 +488,10 @@ class PagedKVCache(KVCacheBase):
             raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.model_dim}]")
         if self.head_dim != self.model_dim:
             query, D = torch.nn.functional.pad(query, (0, self.head_dim - self.model_dim)), self.head_dim
-        if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
+        qs = query.stride()
+        if qs[3] != 1 or qs[0] % 8 or qs[1] % 8 or qs[2] % 8 or query.data_ptr() % 16:
             query = query.contiguous()
+            qs = query.stride()
         rope, self._query_rope = self._query_rope, None
         rope_desc = None
         if rope is not None:
@@ -500,6 +502,7 @@ class PagedKVCache(KVCacheBase):
                 # cases the attention launch does not fold in: rotate the queries (and a held-back append) first
                 self._flush()
                 query, _ = rope(query, None)
+                qs = query.stride()
                 rope_desc = None
         out = torch.empty((B, hq, S, D), dtype=torch.bfloat16, device=query.device)
         st = self.state
@@ -523,8 +526,8 @@ class PagedKVCache(KVCacheBase):
             a.seq_len_bias, a.seq_len_bias_ptr = graph.new_tokens, graph.counter.data_ptr()
             max_len = int(graph.base.max()) + graph.new_tokens * graph.max_steps
         ws = st.workspace(ws_bytes)
-        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = query.data_ptr(), query.stride(0), query.stride(1), query.stride(2)
-        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = query.data_ptr(), qs[0], qs[1], qs[2]
+        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), hq * S * D, S * D, D  # (allocated above: contiguous)
         a.block_table, a.table_stride = table.data_ptr(), table.stride(0)
         a.seq_lens = lens_dev.data_ptr()
         a.kv_start = None if kv_start is None else kv_start.data_ptr()
@@ -558,8 +561,9 @@ class PagedKVCache(KVCacheBase):
             if (k_rope is None) != (rope_desc is None) or k.shape[2] != S and rope_desc is not None:
                 raise RuntimeError("a held-back append and the attention call disagree about the rotary embedding")
             self._pending = None  # this launch stores them into the pool
+            ks = k.stride()
             a.k_new, a.v_new, a.n_new = k.data_ptr(), v.data_ptr(), k.shape[2]
-            a.new_stride_b, a.new_stride_h, a.new_stride_t = k.stride(0), k.stride(1) * head_step, k.stride(2)
+            a.new_stride_b, a.new_stride_h, a.new_stride_t = ks[0], ks[1] * head_step, ks[2]
         fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
         nat.check(fn(ctypes.byref(self._desc), ctypes.byref(a), nat.current_stream_ptr()))
         return out if self.head_dim == self.model_dim else out[..., : self.model_dim].contiguous()
