@@ -31,7 +31,9 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
     }                                                                             \
   } while (0)
 
-int check_pool(const pace_kv_pool_t* pool, const char* who);
+// f32_ok: the entry point also takes pools of fp32 rows (elem_bytes 4); otherwise such a pool is refused.
+int check_pool(const pace_kv_pool_t* pool, const char* who, bool f32_ok = false);
+inline bool pool_is_f32(const pace_kv_pool_t* pool) { return pool->elem_bytes == 4; }
 int compute_units();  // of the current device
 
 // Dense bf16 attention on the matrix cores (dense_attn_mfma.hip); false = shape not handled, nothing launched.
@@ -40,6 +42,8 @@ bool launch_dense_mfma(const void* q, const void* k, const void* v, void* out, i
                        const void* mask, bool mask_is_f32, int mB, int mN, int mS, float scale, void* workspace,
                        size_t workspace_bytes, hipStream_t stream);
 size_t dense_mfma_workspace_bytes(int S, int H, int mB, int mN, int mS, bool has_mask);
+// Attention over a pool of fp32 rows (dense_attn.hip); pool and args are already checked.
+int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, const char* who, hipStream_t stream);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

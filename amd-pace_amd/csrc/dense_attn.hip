@@ -67,6 +67,16 @@ struct DenseParams {
   int32_t mB, mN, mS;
   int32_t l_split;  // waves of a workgroup that share one row group and split its keys: 1, 2 or 4
   float scale;
+  // PAGED (attn_paged_f32_kernel): K / V rows come out of a pool of fp32 rows through a block table (one 16-token
+  // tile is one block), N counts KV heads, the query rows of a KV head are those of its n_rep query heads one
+  // after the other (row r: head r / S of the group, token r % S), q / out / mask are addressed by strides, the
+  // length is the sequence's own and L is unused.
+  const int32_t* table;
+  const int32_t* seq_lens;
+  const int32_t* len_bias_dev;
+  const int32_t* kv_start;
+  int64_t k_bs, k_hs, v_bs, v_hs, q_sb, q_sh, q_ss, o_sb, o_sh, o_ss, m_sb, m_ss;
+  int32_t table_stride, len_bias, num_blocks, n_rep, causal, mask_len;
 };
 
 // HP: head size rounded up to the next size built (dims >= H read as zero).  VEC: H is a multiple
@@ -75,32 +85,51 @@ struct DenseParams {
 // wave per SIMD at head size 128).  It pays where the launch is bound by memory (few query rows: +8 % on an fp32
 // decode step) and costs 10 % where it is bound by the matrix cores, so the launcher picks.
 // EXACT: H == HP (and VEC): no bound on a dim is checked anywhere, which is a third of the vector instructions of a tile.
-template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_kernel(
-    const DenseParams p) {
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED>
+__device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
+  static_assert(!PAGED || (VEC && sizeof(T) == 4), "pools of rows hold fp32 with head sizes that are multiples of 4");
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
   constexpr int MTL = HP / 16;  // 16-dim output tiles
   constexpr int VG = MTL % 4 == 0 ? 4 : 2;  // output tiles whose dims of a lane are neighbours (see the V loads)
   static_assert(MTL % VG == 0, "head sizes built: multiples of 32");
   constexpr int ROW_F = HP + 2;
   __shared__ float merge_buf[2 * 16 * ROW_F];
-  const int H = EXACT ? HP : p.H, L = p.L, S = p.S;
+  const int H = EXACT ? HP : p.H, S = p.S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int split = p.l_split;
-  const int head = blockIdx.y, b = blockIdx.z;
+  const int head = blockIdx.y, b = blockIdx.z;  // PAGED: the KV head
   const int rowgroup = blockIdx.x * (4 / split) + wave / split, ls = wave % split;
   const int row = rowgroup * 16 + n;
-  const bool valid = row < S;
+  // L: keys of this (batch, head); R: its query rows; [start, L) can be read, by this lane's row up to `limit`;
+  // mcols: columns of a mask line.  Without PAGED these are the launch's constants.
+  int L = p.L, R = S, start = 0, mcols = p.L;
+  if constexpr (PAGED) {
+    L = max(0, p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0));
+    if (p.mask) L = min(L, p.mask_len);  // columns the mask does not have are masked
+    start = p.kv_start ? min(max(p.kv_start[b], 0), L) : 0;
+    R = S * p.n_rep, mcols = p.mask_len;
+  }
+  const bool valid = row < R;
+  const int vrow = valid ? row : 0;
+  const int row_s = PAGED ? vrow % S : vrow;                         // token of the row
+  const int qhead = PAGED ? head * p.n_rep + vrow / S : head;        // its query head
   const int64_t pair = (int64_t)b * p.N + head;
-  const T* qrow = static_cast<const T*>(p.q) + (pair * S + (valid ? row : 0)) * H;
-  const T* kbase = static_cast<const T*>(p.k) + pair * (int64_t)L * H;
-  const T* vbase = static_cast<const T*>(p.v) + pair * (int64_t)L * H;
+  const T* qrow = PAGED ? static_cast<const T*>(p.q) + b * p.q_sb + qhead * p.q_sh + row_s * p.q_ss
+                        : static_cast<const T*>(p.q) + (pair * S + vrow) * H;
+  const T* kbase = PAGED ? static_cast<const T*>(p.k) + head * p.k_hs : static_cast<const T*>(p.k) + pair * (int64_t)L * H;
+  const T* vbase = PAGED ? static_cast<const T*>(p.v) + head * p.v_hs : static_cast<const T*>(p.v) + pair * (int64_t)L * H;
   const MT* mrow = nullptr;
   if (p.mask) {
-    const int64_t mb = p.mB == 1 ? 0 : b, mn = p.mN == 1 ? 0 : head, ms = p.mS == 1 ? 0 : (valid ? row : 0);
-    mrow = static_cast<const MT*>(p.mask) + ((mb * p.mN + mn) * p.mS + ms) * (int64_t)L;
+    if constexpr (PAGED) {
+      mrow = static_cast<const MT*>(p.mask) + b * p.m_sb + row_s * p.m_ss;  // (strides of broadcast dims are 0)
+    } else {
+      const int64_t mb = p.mB == 1 ? 0 : b, mn = p.mN == 1 ? 0 : head, ms = p.mS == 1 ? 0 : vrow;
+      mrow = static_cast<const MT*>(p.mask) + ((mb * p.mN + mn) * p.mS + ms) * (int64_t)L;
+    }
   }
+  // causal: query token s reads keys <= L - S + s
+  const int limit = (PAGED && p.causal) ? min(L, L - S + row_s + 1) : L;
   // This lane's dims of a row for the first product: d0 .. d0 + KS - 1.
   const int d0 = g * KS;
   auto load_run = [&](const T* r, float (&x)[KS]) {
@@ -128,20 +157,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   for (int j = 0; j < MTL; ++j) o[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = kNegInf, l_run = 0.f;
 
-  // This wave's share of the 16-token tiles.
-  const int tiles = (L + 15) / 16, per = (tiles + split - 1) / split;
-  const int tile_lo = min(tiles, ls * per), tile_hi = min(tiles, tile_lo + per);
-  const bool has_rows = rowgroup * 16 < S;  // wave-uniform
+  // This wave's share of the 16-token tiles that some row of its group reads.
+  int key_end = L, tile_first = 0;  // wave-uniform
+  if constexpr (PAGED) {
+    if (p.causal) {  // the group's last token: its rows lie in one query head, or some row is a head's last token
+      const int s0 = (rowgroup * 16) % S;
+      key_end = max(0, min(L, L - S + (s0 + 15 < S ? s0 + 15 : S - 1) + 1));
+    }
+    tile_first = start / 16;
+  }
+  const int tiles = max(tile_first, (key_end + 15) / 16), per = (tiles - tile_first + split - 1) / split;
+  const int tile_lo = min(tiles, tile_first + ls * per), tile_hi = min(tiles, tile_lo + per);
+  const bool has_rows = rowgroup * 16 < R;  // wave-uniform
   float kf[KS], vf[MTL][4], mv[4];
   auto fetch = [&](int tile, float (&kx)[KS], float (&vx)[MTL][4], float (&mx4)[4]) {
     const int t0 = tile * 16;
-    load_run(kbase + (int64_t)min(L - 1, t0 + n) * H, kx);  // rows past the end are masked below
+    const T* kblock = kbase;
+    const T* vblock = vbase;
+    if constexpr (PAGED) {  // one tile is one block: a scalar look-up; ids are clamped, nothing outside the pool is read
+      const int64_t blk = min(max(p.table[(int64_t)b * p.table_stride + min(tile, p.table_stride - 1)], 0), p.num_blocks - 1);
+      kblock = kbase + blk * p.k_bs - (int64_t)t0 * H, vblock = vbase + blk * p.v_bs - (int64_t)t0 * H;
+    }
+    // rows past the end are masked below (PAGED: the block's 16 rows exist whatever the length is)
+    load_run(kblock + (int64_t)(PAGED ? t0 + n : min(L - 1, t0 + n)) * H, kx);
     // V: output tile j of lane n stands for dim v_dim(j, n) = 16 VG (j / VG) + VG n + j % VG, so that the VG values a
     // lane needs of one token for VG neighbouring tiles are one contiguous run: a quarter of the load instructions
     // that one value per load takes, and every load of a wave covers whole 256-byte stretches of four rows.
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const T* vr = vbase + (int64_t)min(L - 1, t0 + 4 * g + i) * H;
+      const T* vr = vblock + (int64_t)(PAGED ? t0 + 4 * g + i : min(L - 1, t0 + 4 * g + i)) * H;
 #pragma unroll
       for (int jj = 0; jj < MTL; jj += VG) {
         const int d = 16 * jj + VG * n;
@@ -166,7 +210,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
     if (!mrow) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) mx4[i] = 0.f;
-    } else if (t + 4 <= L) {
+    } else if (t + 4 <= mcols) {
       if constexpr (sizeof(MT) == 4) {
         u32x4 raw;
         __builtin_memcpy(&raw, mrow + t, 16);
@@ -180,7 +224,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) mx4[i] = (t + i < L) ? load_f32<MT>(mrow + t + i) : 0.f;
+      for (int i = 0; i < 4; ++i) mx4[i] = (t + i < mcols) ? load_f32<MT>(mrow + t + i) : 0.f;
     }
   };
   if (AHEAD && has_rows && tile_lo < tile_hi) fetch(tile_lo, kf, vf, mv);
@@ -199,7 +243,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
     float val[4], mx = kNegInf;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      val[i] = (t0 + 4 * g + i < L) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
+      const int tk = t0 + 4 * g + i;
+      val[i] = (tk < limit && (!PAGED || tk >= start)) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
       mx = fmaxf(mx, val[i]);
     }
     mx = row_max4(mx);
@@ -273,7 +318,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   }
   if (ls != 0 || !valid) return;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-  T* orow = static_cast<T*>(p.out) + (pair * S + row) * H;
+  T* orow = PAGED ? static_cast<T*>(p.out) + b * p.o_sb + qhead * p.o_sh + row_s * p.o_ss : static_cast<T*>(p.out) + (pair * S + row) * H;
   // o[j][c] of lane (row, g) is the output at dim v_dim(j, 4 g + c)
 #pragma unroll
   for (int jj = 0; jj < MTL; jj += VG) {
@@ -291,6 +336,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
       }
     }
   }
+}
+
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_kernel(
+    const DenseParams p) {
+  attn_dense_body<T, MT, HP, VEC, AHEAD, EXACT, false>(p);
+}
+
+// The same walk over a pool of fp32 rows (pace_kv_pool_t with elem_bytes 4).  No fetch a tile ahead: here the second
+// wave per SIMD hides more than the second set of registers did (decode, batch 64 x 8 KV heads x 4096 tokens of 128
+// dims: 370 us against 460).
+template <typename MT, int HP, bool EXACT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_paged_f32_kernel(
+    const DenseParams p) {
+  attn_dense_body<float, MT, HP, true, false, EXACT, true>(p);
+}
+
+int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, const char* who, hipStream_t stream) {
+  PACE_REQUIRE(a->batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
+  DenseParams p = {};
+  p.q = a->q, p.k = pool->k, p.v = pool->v, p.out = a->out, p.mask = a->mask;
+  p.B = a->batch, p.N = pool->num_kv_heads, p.S = a->q_len, p.L = 0, p.H = pool->head_dim;
+  p.scale = a->scale;
+  p.table = a->block_table, p.seq_lens = a->seq_lens, p.len_bias_dev = a->seq_len_bias_ptr, p.kv_start = a->kv_start;
+  p.k_bs = pool->k_block_stride, p.k_hs = pool->k_head_stride, p.v_bs = pool->v_block_stride, p.v_hs = pool->v_head_stride;
+  p.q_sb = a->q_stride_b, p.q_sh = a->q_stride_h, p.q_ss = a->q_stride_s;
+  p.o_sb = a->o_stride_b, p.o_sh = a->o_stride_h, p.o_ss = a->o_stride_s;
+  p.m_sb = a->mask_stride_b, p.m_ss = a->mask_stride_s;
+  p.table_stride = a->table_stride, p.len_bias = a->seq_len_bias, p.num_blocks = pool->num_blocks;
+  p.n_rep = a->num_q_heads / pool->num_kv_heads, p.causal = a->causal ? 1 : 0, p.mask_len = a->mask_len;
+  const int64_t rows = (int64_t)a->q_len * p.n_rep;
+  PACE_REQUIRE(rows < (1 << 27), "%s: too many query rows per KV head", who);
+  p.l_split = rows <= 16 ? 4 : (rows <= 32 ? 2 : 1);
+  const int rowgroups = (int)((rows + 15) / 16), per_wg = 4 / p.l_split;
+  const dim3 grid((rowgroups + per_wg - 1) / per_wg, pool->num_kv_heads, a->batch);
+  const int H = pool->head_dim;
+  const bool mf32 = a->mask_dtype == PACE_DTYPE_F32;
+#define PACE_PAGED_F32_GO(MT_, HP_) \
+  do { \
+    if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
+    else hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false>), grid, dim3(256), 0, stream, p); \
+  } while (0)
+#define PACE_PAGED_F32_HP(MT_) \
+  do { \
+    if (H <= 32) PACE_PAGED_F32_GO(MT_, 32); \
+    else if (H <= 64) PACE_PAGED_F32_GO(MT_, 64); \
+    else if (H <= 96) PACE_PAGED_F32_GO(MT_, 96); \
+    else if (H <= 128) PACE_PAGED_F32_GO(MT_, 128); \
+    else PACE_PAGED_F32_GO(MT_, 256); \
+  } while (0)
+  if (mf32) PACE_PAGED_F32_HP(float); else PACE_PAGED_F32_HP(uint16_t);
+#undef PACE_PAGED_F32_HP
+#undef PACE_PAGED_F32_GO
+  PACE_HIP_CHECK(hipGetLastError());
+  return PACE_KV_OK;
 }
 
 }  // namespace pace_kv
@@ -334,7 +434,7 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
     PACE_HIP_CHECK(hipGetLastError());
     return PACE_KV_OK;
   }
-  DenseParams p;
+  DenseParams p = {};
   p.q = q, p.k = k, p.v = v, p.out = out, p.mask = mask;
   p.B = B, p.N = N, p.S = S, p.L = L, p.H = H;
   p.mB = mB, p.mN = mN, p.mS = mS;

@@ -57,6 +57,44 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
                     vv);
 }
 
+// The same scatter into a pool of fp32 rows ([16 tokens][head_dim] floats per (block, head)): one thread moves
+// four dims (16 bytes) of one (token, head) row of K and of V, row to row.
+template <bool PAGED>
+__global__ __launch_bounds__(256) void kv_append_f32_kernel(pace_kv_pool_t pool, const float* __restrict__ k_new,
+                                                            const float* __restrict__ v_new, int64_t sb, int64_t sh,
+                                                            int64_t st, int32_t n_tokens, int32_t total_rows,
+                                                            const AppendDest dest) {
+  const int D = pool.head_dim, chunks = D / 4;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int chunk = (int)(gid % chunks);
+  const int64_t row = gid / chunks;  // (token i, head h), head fastest
+  if (row >= total_rows) return;
+  const int H = pool.num_kv_heads;
+  const int h = (int)(row % H);
+  const int64_t i = row / H;  // b * n_tokens + t
+  const int64_t b = i / n_tokens, t = i % n_tokens;
+  int64_t blk;
+  int off;
+  if (PAGED) {
+    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + t;
+    if (pos < 0 || pos / PACE_KV_BLOCK_TOKENS >= dest.table_stride) return;
+    blk = dest.table[b * dest.table_stride + pos / PACE_KV_BLOCK_TOKENS];
+    off = (int)(pos % PACE_KV_BLOCK_TOKENS);
+  } else {
+    const int64_t slot = dest.slots[i];
+    if (slot < 0) return;
+    blk = slot / PACE_KV_BLOCK_TOKENS;
+    off = (int)(slot % PACE_KV_BLOCK_TOKENS);
+  }
+  if (blk < 0 || blk >= pool.num_blocks) return;  // never write outside the pool
+  const int64_t src = b * sb + h * sh + t * st + chunk * 4;
+  const int64_t in_slab = (int64_t)off * D + chunk * 4;
+  const u32x4 kv = *reinterpret_cast<const u32x4*>(k_new + src);
+  const u32x4 vv = *reinterpret_cast<const u32x4*>(v_new + src);
+  *reinterpret_cast<u32x4*>(static_cast<float*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride + in_slab) = kv;
+  *reinterpret_cast<u32x4*>(static_cast<float*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride + in_slab) = vv;
+}
+
 // ---------------------------------------------------------------------------------
 // Block append (many tokens per sequence: prefill chunks).  One 256-thread workgroup
 // fills one destination block of one (sequence, head): the token rows that land in the
@@ -176,6 +214,26 @@ struct GatherOut {
   int32_t total_rows;         // packed: rows of the outputs
 };
 
+// Packed grid: which (sequence, head, logical block) workgroup `entry` stands for.
+// One grid entry per (logical block that can exist, KV head): sequence b owns the block entries
+// [cu[b] / 16 + b, cu[b+1] / 16 + b + 1) -- at least ceil(len_b / 16) of them, disjoint, in order -- so a
+// ragged batch launches (almost) no workgroup without rows.  Entries run sequence by sequence, head by
+// head, block by block (the order of the dense grid: with the heads of a block side by side instead the
+// launch measured 6 % slower).  The owner is found by bisection, uniform over the workgroup: scalar loads
+// from a table that stays in the scalar cache.
+__device__ __forceinline__ void packed_entry(const int32_t* __restrict__ cu, int batch, int H, unsigned entry, int& b, int& h, int& j) {
+  int lo = 0, hi = batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)(cu[mid] / PACE_KV_BLOCK_TOKENS + mid) * H <= (int64_t)entry) lo = mid; else hi = mid;
+  }
+  b = lo;
+  const int first = cu[b] / PACE_KV_BLOCK_TOKENS + b;
+  const int n = cu[b + 1] / PACE_KV_BLOCK_TOKENS + b + 1 - first;  // >= 1
+  const int r = (int)((int64_t)entry - (int64_t)first * H);
+  h = min(r / n, H - 1), j = r % n;
+}
+
 template <int D, bool PACKED>
 __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
                                                         int32_t table_stride, const int32_t* __restrict__ seq_lens,
@@ -184,25 +242,7 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
   constexpr int SLAB_CHUNKS = PACE_KV_BLOCK_TOKENS * CHUNKS;  // per (block, head)
   __shared__ uint16_t vt[D * PACE_KV_BLOCK_TOKENS + 8];
   int j = blockIdx.x, b = blockIdx.z, h = blockIdx.y;
-  if (PACKED) {
-    // One grid entry per (logical block that can exist, KV head): sequence b owns the block entries
-    // [cu[b] / 16 + b, cu[b+1] / 16 + b + 1) -- at least ceil(len_b / 16) of them, disjoint, in order -- so a
-    // ragged batch launches (almost) no workgroup without rows.  Entries run sequence by sequence, head by
-    // head, block by block (the order of the dense grid: with the heads of a block side by side instead the
-    // launch measured 6 % slower).  The owner is found by bisection, uniform over the workgroup: scalar loads
-    // from a table that stays in the scalar cache.
-    const int H = pool.num_kv_heads;
-    int lo = 0, hi = out.batch;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if ((int64_t)(out.cu_seqlens[mid] / PACE_KV_BLOCK_TOKENS + mid) * H <= (int64_t)blockIdx.x) lo = mid; else hi = mid;
-    }
-    b = lo;
-    const int first = out.cu_seqlens[b] / PACE_KV_BLOCK_TOKENS + b;
-    const int n = out.cu_seqlens[b + 1] / PACE_KV_BLOCK_TOKENS + b + 1 - first;  // >= 1
-    const int r = (int)((int64_t)blockIdx.x - (int64_t)first * H);
-    h = min(r / n, H - 1), j = r % n;
-  }
+  if (PACKED) packed_entry(out.cu_seqlens, out.batch, pool.num_kv_heads, blockIdx.x, b, h, j);
   // The length and the block id are fetched side by side (the table row exists whatever the length is; an
   // entry past the live blocks is clamped into the pool and never used): one round trip, not two, before
   // the slab loads can start.
@@ -255,6 +295,45 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
       const int64_t o = base + (int64_t)(h * n_rep + r) * out.stride_h + (int64_t)t * out.stride_t + chunk * 8;
       store16_stream(out.k + o, kreg[i]);
       store16_stream(out.v + o, vv);
+    }
+  }
+}
+
+// The gather out of a pool of fp32 rows: the same grid, rows copied as they are (16 bytes per lane access).
+template <bool PACKED>
+__global__ __launch_bounds__(256) void kv_gather_f32_kernel(pace_kv_pool_t pool, const int32_t* __restrict__ table,
+                                                            int32_t table_stride, const int32_t* __restrict__ seq_lens,
+                                                            int32_t len_bias, int32_t n_rep, const GatherOut out) {
+  int j = blockIdx.x, b = blockIdx.z, h = blockIdx.y;
+  if (PACKED) packed_entry(out.cu_seqlens, out.batch, pool.num_kv_heads, blockIdx.x, b, h, j);
+  const int len = seq_lens[b] + len_bias;
+  int64_t blk = table[(int64_t)b * table_stride + min(j, table_stride - 1)];
+  const int t0 = j * PACE_KV_BLOCK_TOKENS;
+  const bool live = t0 < len;  // uniform per workgroup
+  const int row_end = PACKED ? len : out.out_len;
+  if (!live && (PACKED || !out.zero_fill || t0 >= row_end)) return;  // nothing to write
+  blk = blk < 0 ? 0 : (blk >= pool.num_blocks ? pool.num_blocks - 1 : blk);  // never read outside the pool
+  const int D = pool.head_dim, chunks = D / 4;
+  const float* ksrc = static_cast<const float*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
+  const float* vsrc = static_cast<const float*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
+  float* ko = reinterpret_cast<float*>(out.k);
+  float* vo = reinterpret_cast<float*>(out.v);
+  const int64_t base = PACKED ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
+  for (int c = threadIdx.x; c < PACE_KV_BLOCK_TOKENS * chunks; c += 256) {
+    const int tok = c / chunks, chunk = c % chunks;
+    const int t = t0 + tok;
+    if (t >= row_end) continue;
+    if (PACKED && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
+    u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
+    if (t < len) {
+      kk = load16_stream(ksrc + c * 4), vv = load16_stream(vsrc + c * 4);
+    } else if (!out.zero_fill) {
+      continue;
+    }
+    for (int r = 0; r < n_rep; ++r) {
+      const int64_t o = base + (int64_t)(h * n_rep + r) * out.stride_h + (int64_t)t * out.stride_t + chunk * 4;
+      store16_stream(ko + o, kk);
+      store16_stream(vo + o, vv);
     }
   }
 }
@@ -333,14 +412,32 @@ int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void*
 static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
                       int64_t stride_b, int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
                       const AppendDest& dest, bool paged, void* stream) {
-  if (int rc = check_pool(pool, who)) return rc;
+  if (int rc = check_pool(pool, who, true)) return rc;
   PACE_REQUIRE(batch >= 0 && n_tokens >= 0, "%s: negative batch (%d) or n_tokens (%d)", who, batch, n_tokens);
   if (batch == 0 || n_tokens == 0) return PACE_KV_OK;
   PACE_REQUIRE(k_new && v_new, "%s: NULL input pointer", who);
   PACE_REQUIRE(aligned16(k_new) && aligned16(v_new), "%s: k_new / v_new must be 16-byte aligned", who);
-  PACE_REQUIRE(stride_b % 8 == 0 && stride_h % 8 == 0 && stride_t % 8 == 0,
-               "%s: input strides must be multiples of 8 elements", who);
+  const int per16 = pool_is_f32(pool) ? 4 : 8;
+  PACE_REQUIRE(stride_b % per16 == 0 && stride_h % per16 == 0 && stride_t % per16 == 0,
+               "%s: input strides must be multiples of %d elements", who, per16);
   hipStream_t s_early = static_cast<hipStream_t>(stream);
+  if (pool_is_f32(pool)) {
+    const int64_t rows = (int64_t)batch * n_tokens * pool->num_kv_heads;
+    PACE_REQUIRE(rows < (int64_t)1 << 31, "%s: too many rows (%lld)", who, (long long)rows);
+    const int64_t threads = rows * (pool->head_dim / 4);
+    PACE_REQUIRE((threads + 255) / 256 < (int64_t)1 << 31, "%s: grid too large", who);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    const float* k = static_cast<const float*>(k_new);
+    const float* v = static_cast<const float*>(v_new);
+    if (paged)
+      hipLaunchKernelGGL(kv_append_f32_kernel<true>, grid, dim3(256), 0, s_early, *pool, k, v, stride_b, stride_h, stride_t, n_tokens,
+                         (int32_t)rows, dest);
+    else
+      hipLaunchKernelGGL(kv_append_f32_kernel<false>, grid, dim3(256), 0, s_early, *pool, k, v, stride_b, stride_h, stride_t, n_tokens,
+                         (int32_t)rows, dest);
+    PACE_HIP_CHECK(hipGetLastError());
+    return PACE_KV_OK;
+  }
   if (paged && n_tokens >= 8)  // enough tokens per sequence to fill slabs: one workgroup per destination block
     return launch_block_append(who, pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest.table,
                                dest.table_stride, dest.seq_lens, dest.pos_offset, nullptr, s_early);
@@ -390,14 +487,15 @@ static int run_gather(const char* who, const pace_kv_pool_t* pool, const int32_t
                       const int32_t* seq_lens, int32_t seq_len_bias, int32_t batch, int32_t n_rep, int32_t rows,
                       const GatherOut& out_in, bool packed, void* stream) {
   const GatherOut& out = out_in;
-  if (int rc = check_pool(pool, who)) return rc;
+  if (int rc = check_pool(pool, who, true)) return rc;
   PACE_REQUIRE(batch >= 0 && rows >= 0 && n_rep >= 1, "%s: bad batch (%d), row count (%d) or n_rep (%d)", who, batch, rows, n_rep);
   if (batch == 0 || rows == 0) return PACE_KV_OK;
   PACE_REQUIRE(block_table && seq_lens && out.k && out.v, "%s: NULL pointer", who);
   PACE_REQUIRE(aligned16(out.k) && aligned16(out.v), "%s: outputs must be 16-byte aligned", who);
-  PACE_REQUIRE(out.stride_b % 8 == 0 && out.stride_h % 8 == 0 && out.stride_t % 8 == 0 && out.stride_t >= pool->head_dim &&
+  const int per16 = pool_is_f32(pool) ? 4 : 8;
+  PACE_REQUIRE(out.stride_b % per16 == 0 && out.stride_h % per16 == 0 && out.stride_t % per16 == 0 && out.stride_t >= pool->head_dim &&
                    out.stride_h >= pool->head_dim,
-               "%s: output strides must be multiples of 8 elements and hold a row of head_dim", who);
+               "%s: output strides must be multiples of %d elements and hold a row of head_dim", who, per16);
   const int n_blocks = (rows + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
   PACE_REQUIRE(table_stride >= 1, "%s: table_stride %d", who, table_stride);
   PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch/heads exceed grid limits", who);
@@ -408,6 +506,16 @@ static int run_gather(const char* who, const pace_kv_pool_t* pool, const int32_t
     grid = dim3((unsigned)entries, 1, 1);
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (pool_is_f32(pool)) {
+    if (packed)
+      hipLaunchKernelGGL(kv_gather_f32_kernel<true>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias, n_rep,
+                         out);
+    else
+      hipLaunchKernelGGL(kv_gather_f32_kernel<false>, grid, dim3(256), 0, s, *pool, block_table, table_stride, seq_lens, seq_len_bias, n_rep,
+                         out);
+    PACE_HIP_CHECK(hipGetLastError());
+    return PACE_KV_OK;
+  }
   for_head_dim(pool->head_dim, [&](auto d) {
     constexpr int DIM = decltype(d)::value;
     if (packed)
@@ -443,10 +551,24 @@ extern "C" int pace_kv_gather_packed(const pace_kv_pool_t* pool, const int32_t* 
                     out, true, stream);
 }
 
-extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src, const pace_kv_pool_t* dst, const int32_t* pairs,
+// A slab is copied verbatim, so a pool of fp32 rows is described to the copy kernels in their 2-byte units.
+static pace_kv_pool_t in_halfwords(const pace_kv_pool_t* p) {
+  pace_kv_pool_t q = *p;
+  if (pool_is_f32(p)) {
+    q.k_block_stride *= 2, q.k_head_stride *= 2, q.v_block_stride *= 2, q.v_head_stride *= 2, q.head_dim *= 2;
+    q.elem_bytes = 2;
+  }
+  return q;
+}
+
+extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src_in, const pace_kv_pool_t* dst_in, const int32_t* pairs,
                                    int32_t n_pairs, void* stream) {
-  if (int rc = check_pool(src, "pace_kv_copy_blocks(src)")) return rc;
-  if (int rc = check_pool(dst, "pace_kv_copy_blocks(dst)")) return rc;
+  if (int rc = check_pool(src_in, "pace_kv_copy_blocks(src)", true)) return rc;
+  if (int rc = check_pool(dst_in, "pace_kv_copy_blocks(dst)", true)) return rc;
+  PACE_REQUIRE(pool_is_f32(src_in) == pool_is_f32(dst_in), "pace_kv_copy_blocks: src and dst pools differ in element type");
+  const pace_kv_pool_t src_h = in_halfwords(src_in), dst_h = in_halfwords(dst_in);
+  const pace_kv_pool_t* src = &src_h;
+  const pace_kv_pool_t* dst = &dst_h;
   PACE_REQUIRE(src->head_dim == dst->head_dim && src->num_kv_heads == dst->num_kv_heads,
                "pace_kv_copy_blocks: src and dst pools differ in head_dim or num_kv_heads");
   PACE_REQUIRE(n_pairs >= 0, "pace_kv_copy_blocks: negative n_pairs");
@@ -490,7 +612,7 @@ extern "C" int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, in
     return PACE_KV_EINVAL;
   }
   for (int i = 0; i < n_pools; ++i) {
-    if (int rc = check_pool(pools[i], who)) return rc;
+    if (int rc = check_pool(pools[i], who, true)) return rc;
     if (pools[i]->num_blocks != pools[0]->num_blocks) {
       set_error("%s: pools of one table must have the same number of blocks", who);
       return PACE_KV_EINVAL;

@@ -1068,13 +1068,33 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     a_copy.workspace_bytes = kStaticScratchBytes;
   }
   const pace_paged_attn_args_t* a = &a_copy;
-  if (int rc = check_pool(pool, who)) return rc;
+  if (int rc = check_pool(pool, who, true)) return rc;
   PACE_REQUIRE(a->batch >= 0 && a->q_len >= 1 && a->num_q_heads >= 1, "%s: bad batch (%d), q_len (%d) or num_q_heads (%d)",
                who, a->batch, a->q_len, a->num_q_heads);
   if (a->batch == 0) return PACE_KV_OK;
   PACE_REQUIRE(a->q && a->out && a->block_table && a->seq_lens, "%s: NULL q / out / block_table / seq_lens", who);
   PACE_REQUIRE(a->num_q_heads % pool->num_kv_heads == 0, "%s: num_q_heads %d not a multiple of num_kv_heads %d", who,
                a->num_q_heads, pool->num_kv_heads);
+  if (pool_is_f32(pool)) {
+    // rows of fp32: the general kernel of the dense operator walks the block table (dense_attn.hip)
+    PACE_REQUIRE(!a->k_new && !a->v_new && !a->rope,
+                 "%s: an fp32 pool takes neither a fused append nor a rotary embedding inside the attention launch", who);
+    PACE_REQUIRE(aligned16(a->q) && aligned16(a->out) && (a->q_stride_b % 4) == 0 && (a->q_stride_h % 4) == 0 &&
+                     (a->q_stride_s % 4) == 0 && (a->o_stride_b % 4) == 0 && (a->o_stride_h % 4) == 0 && (a->o_stride_s % 4) == 0,
+                 "%s: q and out must be 16-byte aligned with strides that are multiples of 4 elements", who);
+    PACE_REQUIRE(a->max_seq_len >= 0 && a->table_stride >= 1 && (int64_t)a->table_stride * PACE_KV_BLOCK_TOKENS >= a->max_seq_len,
+                 "%s: block table row (%d blocks) cannot hold max_seq_len %d", who, a->table_stride, a->max_seq_len);
+    PACE_REQUIRE(a->scale > 0.f && a->scale < __builtin_inff(), "%s: softmax scale must be positive and finite (got %g)", who,
+                 (double)a->scale);
+    if (a->mask)
+      PACE_REQUIRE((a->mask_dtype == PACE_DTYPE_F32 || a->mask_dtype == PACE_DTYPE_BF16) && a->mask_len >= 0,
+                   "%s: bad mask dtype %d or mask_len %d", who, a->mask_dtype, a->mask_len);
+    if (g_name_out) {  // (pace_paged_attn_kernel_name: nothing is launched)
+      snprintf(g_name_out, g_name_cap, "pace_kv::attn_dense_kernel<float, ...> (paged rows)");
+      return PACE_KV_OK;
+    }
+    return launch_paged_f32(pool, a, who, static_cast<hipStream_t>(stream));
+  }
   PACE_REQUIRE(aligned16(a->q) && (a->q_stride_b % 8) == 0 && (a->q_stride_h % 8) == 0 && (a->q_stride_s % 8) == 0,
                "%s: q must be 16-byte aligned with strides that are multiples of 8 elements", who);
   PACE_REQUIRE((reinterpret_cast<uintptr_t>(a->out) & 7u) == 0 && (a->o_stride_b % 4) == 0 && (a->o_stride_h % 4) == 0 &&

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 11
+ABI_VERSION = 12
 STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
@@ -60,6 +60,8 @@ class PoolDesc(Structure):
         ("num_kv_heads", c_int32),
         ("head_dim", c_int32),
         ("block_size", c_int32),
+        ("elem_bytes", c_int32),  # 0 / 2: bf16 slabs, 4: fp32 rows
+        ("reserved", c_int32),
     ]
 
 

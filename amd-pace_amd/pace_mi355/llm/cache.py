@@ -153,6 +153,7 @@ class PagedKVCache(KVCacheBase):
         self._query_rope = None
         self._graph = None  # a DecodeGraph that has captured this cache's decode step
         self.cow_blocks_copied = 0  # blocks copied on write after forks (per layer pool)
+        self.f32 = False  # the pool holds fp32 rows (set by the first update)
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
     @property
@@ -170,8 +171,13 @@ class PagedKVCache(KVCacheBase):
             return
         if not key_states.is_cuda:
             raise RuntimeError("PagedKVCache stores its blocks in GPU memory; key/value states must be device tensors")
-        if key_states.dtype != torch.bfloat16:
-            raise RuntimeError(f"PagedKVCache stores bf16; got {key_states.dtype}")
+        if key_states.dtype not in (torch.bfloat16, torch.float32):
+            raise RuntimeError(f"PagedKVCache stores bf16 or fp32; got {key_states.dtype}")
+        # fp32 (the reference's caches keep the model's dtype, ``pace/llm/cache.py:255-266``): blocks of plain rows,
+        # read by the dense operator's fp32 kernel through the block table; nothing is folded into that launch
+        self.f32 = key_states.dtype == torch.float32
+        if self.f32:
+            self.fuse_append = False
         nat.load()
         B, h_in, _, D = key_states.shape
         if self._cfg_kv_heads is not None:
@@ -184,8 +190,8 @@ class PagedKVCache(KVCacheBase):
             raise RuntimeError(f"{h_in} input heads cannot be reduced to {hkv} KV heads")
         self.batch, self.num_kv_heads, self.model_dim = int(B), hkv, int(D)
         # e.g. 80 (OPT-2.7B) is kept in slabs of 96: zero dims change neither a score nor an output
-        self.head_dim = next((d for d in nat.HEAD_DIMS if d >= D), 0)
-        if not self.head_dim:
+        self.head_dim = (D + 3) // 4 * 4 if self.f32 else next((d for d in nat.HEAD_DIMS if d >= D), 0)
+        if not self.head_dim or self.head_dim > nat.HEAD_DIMS[-1]:
             raise RuntimeError(f"head_dim {D} unsupported (at most {nat.HEAD_DIMS[-1]})")
         D = self.head_dim
         self.n_rep = int(self._cfg_n_rep) if self._cfg_n_rep is not None else h_in // hkv
@@ -197,7 +203,7 @@ class PagedKVCache(KVCacheBase):
         nb = self.state.allocator.num_blocks
         # [block][head][K|V][16*D]: one block of one layer is contiguous (64 KiB at 8 heads x 128 dims)
         # and the K and V slabs a wavefront reads together are adjacent.
-        self.pool = torch.zeros((nb, hkv, 2, BLOCK * D), dtype=torch.bfloat16, device=key_states.device)
+        self.pool = torch.zeros((nb, hkv, 2, BLOCK * D), dtype=key_states.dtype, device=key_states.device)
         self.state.pools.append(self.pool)
         self._desc = self._describe(self.pool)
         self.lens = np.zeros(B, dtype=np.int64)
@@ -215,6 +221,7 @@ class PagedKVCache(KVCacheBase):
             num_kv_heads=hkv,
             head_dim=slab // BLOCK,
             block_size=BLOCK,
+            elem_bytes=pool.element_size(),
         )
 
     # -- reference interface ----------------------------------------------------
@@ -272,9 +279,19 @@ class PagedKVCache(KVCacheBase):
             if rope is not None:
                 raise NotImplementedError("rotary embedding with a zero-padded head size")
             k, v = (torch.nn.functional.pad(t, (0, self.head_dim - self.model_dim)) for t in (k, v))
+        if k.dtype != self.pool.dtype or v.dtype != self.pool.dtype:
+            raise RuntimeError(f"the cache holds {self.pool.dtype}; got {k.dtype} / {v.dtype}")
         ks = k.stride()
-        if ks[3] != 1 or ks != v.stride() or ks[0] % 8 or ks[1] % 8 or ks[2] % 8:
+        per16 = 4 if self.f32 else 8  # elements in 16 bytes
+        if ks[3] != 1 or ks != v.stride() or ks[0] % per16 or ks[1] % per16 or ks[2] % per16:
             k, v = k.contiguous(), v.contiguous()
+        if self.f32 and rope is not None:
+            # rotated in a launch of its own; the attention call that follows does the same with its queries
+            _, k = rope(None, k)
+            self._query_rope, rope = rope, None
+            keep_query_rope = True
+        else:
+            keep_query_rope = False
         head_step = h_in // self.num_kv_heads  # de-duplicate a repeat_kv-expanded input
         st = self.state
         lib = nat.load()
@@ -298,7 +315,8 @@ class PagedKVCache(KVCacheBase):
                 self._pending = (k, v, head_step, rope)
             else:
                 self._launch_append(k, v, head_step, new_lens, rope)
-            self._query_rope = rope  # the next attention call rotates its queries with it
+            if not keep_query_rope:
+                self._query_rope = rope  # the next attention call rotates its queries with it
         else:
             if (counts < 0).any() or (counts > T).any():
                 raise ValueError("counts must lie in [0, T]")
@@ -429,8 +447,8 @@ class PagedKVCache(KVCacheBase):
         L = int(self.lens.max(initial=0)) if pad_to is None else int(pad_to)
         shape = (self.batch, self.num_kv_heads * n_rep, L, self.head_dim)
         padded = self.head_dim != self.model_dim
-        k = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
-        v = torch.empty(shape, dtype=torch.bfloat16, device=self.pool.device)
+        k = torch.empty(shape, dtype=self.pool.dtype, device=self.pool.device)
+        v = torch.empty(shape, dtype=self.pool.dtype, device=self.pool.device)
         if L:
             st = self.state
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
@@ -458,8 +476,8 @@ class PagedKVCache(KVCacheBase):
         dev = self.pool.device
         cu_dev = torch.from_numpy(cu.astype(np.int32)).pin_memory().to(dev, non_blocking=True)
         shape = (total, self.num_kv_heads * n_rep, self.head_dim)
-        k = torch.empty(shape, dtype=torch.bfloat16, device=dev)
-        v = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+        k = torch.empty(shape, dtype=self.pool.dtype, device=dev)
+        v = torch.empty(shape, dtype=self.pool.dtype, device=dev)
         if total:
             st = self.state
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
@@ -481,15 +499,16 @@ class PagedKVCache(KVCacheBase):
         (the causal mask ``pace/llm/models/llama.py:292-299`` builds); with an additive
         mask ``[B|1, 1, S|1, Lm]`` the mask alone decides, as in the reference.
         """
-        if query.dim() != 4 or query.dtype != torch.bfloat16 or not query.is_cuda:
-            raise RuntimeError("paged attention expects a bf16 device tensor [B, Hq, S, D]")
+        if query.dim() != 4 or not query.is_cuda or self.pool is None or query.dtype != self.pool.dtype:
+            raise RuntimeError("paged attention expects a device tensor [B, Hq, S, D] of the cache's dtype (bf16 or fp32)")
         B, hq, S, D = query.shape
         if B != self.batch or D != self.model_dim or hq % self.num_kv_heads:
             raise RuntimeError(f"query {tuple(query.shape)} does not fit cache [B={self.batch}, Hkv={self.num_kv_heads}, D={self.model_dim}]")
         if self.head_dim != self.model_dim:
             query, D = torch.nn.functional.pad(query, (0, self.head_dim - self.model_dim)), self.head_dim
         qs = query.stride()
-        if qs[3] != 1 or qs[0] % 8 or qs[1] % 8 or qs[2] % 8 or query.data_ptr() % 16:
+        per16 = 4 if self.f32 else 8
+        if qs[3] != 1 or qs[0] % per16 or qs[1] % per16 or qs[2] % per16 or query.data_ptr() % 16:
             query = query.contiguous()
             qs = query.stride()
         rope, self._query_rope = self._query_rope, None
@@ -497,14 +516,17 @@ class PagedKVCache(KVCacheBase):
         if rope is not None:
             if tuple(rope.rows.shape) not in ((B, S), (1, S)):
                 raise RuntimeError(f"rope rows {tuple(rope.rows.shape)} do not match the query [B={B}, S={S}]")
-            rope_desc = rope.desc()
-            if attention_mask is not None or rope_desc.rotary_dim != D or D % 64:
+            rope_desc = None if self.f32 else rope.desc()
+            if self.f32:
+                query, _ = rope(query, None)  # (the keys were rotated before their append)
+                qs = query.stride()
+            elif attention_mask is not None or rope_desc.rotary_dim != D or D % 64:
                 # cases the attention launch does not fold in: rotate the queries (and a held-back append) first
                 self._flush()
                 query, _ = rope(query, None)
                 qs = query.stride()
                 rope_desc = None
-        out = torch.empty((B, hq, S, D), dtype=torch.bfloat16, device=query.device)
+        out = torch.empty((B, hq, S, D), dtype=query.dtype, device=query.device)
         st = self.state
         max_len = self.seq_len
         lib = nat.load()
@@ -515,7 +537,13 @@ class PagedKVCache(KVCacheBase):
         plan = lambda: st.plan_attention(self.lens, hq, self.num_kv_heads, self.head_dim, S, attention_mask is not None,
                                          self.partition_tokens)
         a = nat.PagedAttnArgs()
-        if graph is None:
+        if self.f32:
+            # rows of fp32: one launch of the dense operator's kernel over the block table, no work list, no workspace
+            items = parts = None
+            n_items = max_parts = ws_bytes = 0
+            table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
+            a.seq_len_bias = bias
+        elif graph is None:
             items, parts, n_items, max_parts, ws_bytes = plan()
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
             a.seq_len_bias = bias
@@ -549,8 +577,9 @@ class PagedKVCache(KVCacheBase):
             a.mask, a.causal = None, 1
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         a.max_seq_len, a.partition_tokens = max_len, 0
-        a.work_items, a.n_work_items = items.data_ptr(), n_items
-        a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
+        if items is not None:
+            a.work_items, a.n_work_items = items.data_ptr(), n_items
+            a.seq_parts, a.max_parts = parts.data_ptr(), max_parts
         a.scale = 1.0 / math.sqrt(self.model_dim)
         a.workspace = None if ws is None else ws.data_ptr()
         a.workspace_bytes = ws_bytes

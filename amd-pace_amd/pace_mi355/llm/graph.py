@@ -31,6 +31,8 @@ class DecodeGraph:
                  stream: Optional[torch.cuda.Stream] = None):
         if not caches or any(c.pool is None for c in caches):
             raise RuntimeError("the caches must hold their prompt before a decode step can be captured")
+        if any(c.f32 for c in caches):
+            raise RuntimeError("a decode graph rides on the append fused into the attention launch: bf16 pools only")
         st = caches[0].state
         if any(c.state is not st for c in caches):
             raise RuntimeError("the layers of one decode graph share one block table")

@@ -27,6 +27,17 @@
  * which covers both two separate K / V allocations and one interleaved
  * [block][2][head][16*head_dim] allocation.  Unwritten slots must hold finite
  * bit patterns (allocate the pool zero-filled).
+ *
+ * A pool may hold fp32 instead (elem_bytes = 4: the reference's caches keep
+ * whatever dtype the model runs in, pace/llm/cache.py:255-266, and its
+ * attention is registered for float32 and bfloat16, pace/ops/backends/jit.py:31-34).
+ * Its slabs are plain rows, [16 tokens][head_dim] floats, head_dim any multiple
+ * of 4 up to 256, strides in floats.  Append, append_paged, gather,
+ * gather_packed, copy_blocks, compact_blocks and the decode / verify attention
+ * take such a pool (new tokens, gathered rows, queries and outputs are then
+ * fp32 too, and the attention needs no workspace); what folds other steps into
+ * a launch (pace_rope_append_paged, args->rope, args->k_new) is bf16 only and
+ * says so when handed such a pool.
  */
 #ifndef PACE_KV_HIP_H
 #define PACE_KV_HIP_H
@@ -57,8 +68,10 @@ typedef struct pace_kv_pool {
   int64_t v_head_stride;
   int32_t num_blocks;
   int32_t num_kv_heads;
-  int32_t head_dim;       /* 64, 96, 128 or 256                              */
+  int32_t head_dim;       /* bf16: 64, 96, 128 or 256; fp32: 4 .. 256, % 4   */
   int32_t block_size;     /* must be PACE_KV_BLOCK_TOKENS                    */
+  int32_t elem_bytes;     /* 0 or 2: bf16 slabs; 4: fp32 rows (see above)    */
+  int32_t reserved;       /* 0                                               */
 } pace_kv_pool_t;
 
 /* Text of the last failure on the calling thread ("" if none). */

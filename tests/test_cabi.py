@@ -59,7 +59,7 @@ def test_struct_layouts_match_the_header():
     assert fields("pace_rope") == [f[0] for f in _native.RopeDesc._fields_]
     assert fields("pace_attn_plan") == [f[0] for f in _native.AttnPlan._fields_]
     assert int(re.search(r"#define PACE_ATTN_WORK_INTS (\d+)", text).group(1)) == _native.WORK_INTS
-    assert ctypes.sizeof(_native.PoolDesc) == 64
+    assert ctypes.sizeof(_native.PoolDesc) == 72
 
 
 def test_argument_errors_are_reported_without_a_gpu():
@@ -76,6 +76,21 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"head_dim 80 unsupported" in lib.pace_kv_last_error()
     with pytest.raises(_native.NativeError, match="head_dim 80"):
         _native.check(-1)
+    # a pool of fp32 rows: any multiple of 4 up to 256; entry points that fold other steps in refuse it
+    bad.elem_bytes = 4
+    assert lib.pace_kv_gather(ctypes.byref(bad), 0, 1, 0, 0, 1, 1, 16, 16, 8, 8, 16, 1, None) == -1
+    assert b"NULL pointer" in lib.pace_kv_last_error()  # (the pool itself passed)
+    bad.head_dim = 82
+    assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 0, 1, 1, 16, 16, 8, 8, 16, 1, None) == -1
+    assert b"head_dim 82 unsupported for an fp32 pool" in lib.pace_kv_last_error()
+    bad.head_dim = 80
+    assert lib.pace_rope_append_paged(ctypes.byref(bad), ctypes.byref(_native.RopeDesc()), None, None, 0, 0, 0, 0, 16, 16, 8, 8, 8, 1, 1,
+                                      16, 1, 16, 0, None) == -1
+    assert b"bf16 pools only" in lib.pace_kv_last_error()
+    bad.elem_bytes = 3
+    assert lib.pace_kv_gather(ctypes.byref(bad), 16, 1, 16, 0, 1, 1, 16, 16, 8, 8, 16, 1, None) == -1
+    assert b"elem_bytes 3" in lib.pace_kv_last_error()
+    bad.elem_bytes = 0
     assert lib.pace_attn_dense(16, 16, 16, 16, 1, 1, 1, 1, 1, 300, None, 0, 1, 1, 1, None) == -1
     assert b"head_dim 300 unsupported" in lib.pace_kv_last_error()
     assert lib.pace_paged_attn_workspace_bytes(0, 32, 1, 128, 4096, 0, 8) == 0
