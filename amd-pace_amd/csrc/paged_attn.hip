@@ -1090,7 +1090,9 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
       PACE_REQUIRE((a->mask_dtype == PACE_DTYPE_F32 || a->mask_dtype == PACE_DTYPE_BF16) && a->mask_len >= 0,
                    "%s: bad mask dtype %d or mask_len %d", who, a->mask_dtype, a->mask_len);
     if (g_name_out) {  // (pace_paged_attn_kernel_name: nothing is launched)
-      snprintf(g_name_out, g_name_cap, "pace_kv::attn_dense_kernel<float, ...> (paged rows)");
+      const int H = pool->head_dim, hp = H <= 32 ? 32 : (H <= 64 ? 64 : (H <= 96 ? 96 : (H <= 128 ? 128 : 256)));
+      snprintf(g_name_out, g_name_cap, "pace_kv::attn_paged_f32_kernel<%s, %d, %s>",
+               a->mask_dtype == PACE_DTYPE_F32 ? "float" : "unsigned short", hp, H == hp ? "true" : "false");
       return PACE_KV_OK;
     }
     return launch_paged_f32(pool, a, who, static_cast<hipStream_t>(stream));

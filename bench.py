@@ -19,6 +19,7 @@ Other workloads (same JSON shape, `config.workload` names them):
             op on 2048 x 2048 with the additive causal mask (roofline against the matrix-core peak)
   decode-gptj   the headline step at GPT-J-6B's attention shape (16 heads of 256, batch 64 x 2048)
   dense-f32     the dense op on fp32 tensors (the general kernel; roofline against the fp32 matrix-core peak)
+  decode-f32pool   the headline step over a pool of fp32 rows (an fp32 model on the paged cache)
   compact   Llama-3-70B-shape KV, batch 8, context 32768: evict 40% of the blocks, then time the
             compaction copy and the decode over the compacted cache
   gather / append    the block-table gather (dense and packed output) and the stand-alone append (1 / 8 / 512
@@ -109,7 +110,7 @@ def alloc_free_history(alloc, seed, lo_blocks, hi_blocks, occupancy=0.75, turnov
 
 
 def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor=None, headroom=64, permute=True,
-                history=False):
+                history=False, f32=False):
     """Paged cache holding lens[b] tokens per sequence, physical blocks in a seeded random order (a shuffle of
     the free list) or, with `history`, in the order a seeded admit / retire history of sequences leaves behind."""
     import numpy as np
@@ -126,6 +127,8 @@ def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor
         n = min(chunk, T - t0)
         k = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
         v = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
+        if f32:  # a pool of fp32 rows
+            k, v = k.float(), v.float()
         if t0 == 0:
             cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)  # creates the pool and the free list
             alloc = cache.state.allocator
@@ -161,7 +164,7 @@ class FixedStep:
         self.table = cache.state.device_table()
         self.lens_dev = torch.from_numpy(lens_after.astype(np.int32)).to(dev)
         self.lens_after = lens_after
-        self.out = torch.empty(B, hq, S, D, dtype=torch.bfloat16, device=dev)
+        self.out = torch.empty(B, hq, S, D, dtype=q.dtype, device=dev)
         max_len = int(lens_after.max())
         a = nat.PagedAttnArgs()
         a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
@@ -175,11 +178,14 @@ class FixedStep:
             a.mask_stride_b, a.mask_stride_s = mask.stride(0), mask.stride(2)
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         # the library's planner cuts the batch: descriptors of (sequence, partition) work items in scheduling order
-        self.items, self.parts, n_items, max_parts, ws_bytes = cache.state.plan_attention(
-            lens_after, hq, cache.num_kv_heads, cache.head_dim, S, mask is not None, partition)
         a.max_seq_len, a.partition_tokens, a.scale = max_len, 0, 1.0 / math.sqrt(D)
-        a.work_items, a.n_work_items = self.items.data_ptr(), n_items
-        a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
+        if cache.f32:  # rows of fp32: one launch over the block table, no work list, no workspace
+            n_items = max_parts = ws_bytes = 0
+        else:
+            self.items, self.parts, n_items, max_parts, ws_bytes = cache.state.plan_attention(
+                lens_after, hq, cache.num_kv_heads, cache.head_dim, S, mask is not None, partition)
+            a.work_items, a.n_work_items = self.items.data_ptr(), n_items
+            a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
         self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
         self.n_items, self.max_parts = n_items, max_parts
@@ -636,6 +642,22 @@ def wl_dense_f32(torch, dev, args):
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5)}, extra={"dtype": "f32"})
 
 
+def wl_decode_f32pool(torch, dev, args):
+    """The headline step for an fp32 model (the reference's caches keep the model's dtype,
+    pace/llm/cache.py:255-266): a pool of fp32 rows, a 1-token append and the decode attention in two launches."""
+    B, ctx, hq, hkv, D = args.batch or 64, args.context or 4096, 32, 8, 128
+    cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute, f32=True)
+    g = torch.Generator(device=dev).manual_seed(2)
+    k1, v1, q = (torch.randn(B, h, 1, D, generator=g, device=dev) for h in (hkv, hkv, hq))
+    fs = FixedStep(torch, cache, q, k1, v1, fused=False)
+    dt, attn_ms = run_timed(torch, fs, args.steps, args.warmup)
+    nbytes = 2 * decode_bytes(fs.lens_after.tolist(), hq, hkv, D) - 4 * B - 4 * B * math.ceil((ctx + 1) / 16)  # fp32 rows, the same table
+    return result_line(
+        args, f"decode over a pool of fp32 rows: batch {B}, context {ctx} (+1 appended), 32 Q / 8 KV heads, head_dim 128, KV block 16, "
+        "seeded random physical block permutation, 1-token append + GQA decode (two launches)",
+        nbytes + 2 * append_bytes(B, 1, hkv, D), B, dt, roofline(fs.kernel, nbytes, attn_ms), extra={"dtype": "f32"})
+
+
 def wl_compact(torch, dev, args):
     import numpy as np
 
@@ -760,7 +782,7 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, warmup=2, timed=5):
     }
 
 
-WORKLOADS = {"gather": wl_gather, "append": wl_append, "decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32,
+WORKLOADS = {"gather": wl_gather, "append": wl_append, "decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32, "decode-f32pool": wl_decode_f32pool,
              "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
 
