@@ -77,6 +77,10 @@ struct DenseParams {
   const int32_t* kv_start;
   int64_t k_bs, k_hs, v_bs, v_hs, q_sb, q_sh, q_ss, o_sb, o_sh, o_ss, m_sb, m_ss;
   int32_t table_stride, len_bias, num_blocks, n_rep, causal, mask_len;
+  // n_split > 1: the keys of a row group are cut over n_split workgroups (a batch that does not fill the GPU alone);
+  // each leaves (o unnormalised, m, l) per row in `part` ([row][n_split][H + 4] floats), attn_paged_f32_merge_kernel ends.
+  int32_t n_split;
+  float* part;
 };
 
 // HP: head size rounded up to the next size built (dims >= H read as zero).  VEC: H is a multiple
@@ -99,7 +103,9 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int split = p.l_split;
   const int head = blockIdx.y, b = blockIdx.z;  // PAGED: the KV head
-  const int rowgroup = blockIdx.x * (4 / split) + wave / split, ls = wave % split;
+  const int n_split = PAGED ? p.n_split : 1;
+  const int ks = PAGED ? blockIdx.x % n_split : 0, wg_x = PAGED ? blockIdx.x / n_split : blockIdx.x;
+  const int rowgroup = wg_x * (4 / split) + wave / split, ls = wave % split;
   const int row = rowgroup * 16 + n;
   // L: keys of this (batch, head); R: its query rows; [start, L) can be read, by this lane's row up to `limit`;
   // mcols: columns of a mask line.  Without PAGED these are the launch's constants.
@@ -166,8 +172,11 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     }
     tile_first = start / 16;
   }
-  const int tiles = max(tile_first, (key_end + 15) / 16), per = (tiles - tile_first + split - 1) / split;
-  const int tile_lo = min(tiles, tile_first + ls * per), tile_hi = min(tiles, tile_lo + per);
+  const int tiles = max(tile_first, (key_end + 15) / 16);
+  const int per_wg = (tiles - tile_first + n_split - 1) / n_split;  // (n_split 1: the whole range)
+  const int wg_lo = min(tiles, tile_first + ks * per_wg), wg_hi = min(tiles, wg_lo + per_wg);
+  const int per = (wg_hi - wg_lo + split - 1) / split;
+  const int tile_lo = min(wg_hi, wg_lo + ls * per), tile_hi = min(wg_hi, tile_lo + per);
   const bool has_rows = rowgroup * 16 < R;  // wave-uniform
   float kf[KS], vf[MTL][4], mv[4];
   auto fetch = [&](int tile, float (&kx)[KS], float (&vx)[MTL][4], float (&mx4)[4]) {
@@ -317,6 +326,26 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     __syncthreads();
   }
   if (ls != 0 || !valid) return;
+  if constexpr (PAGED) {
+    if (n_split > 1) {  // this workgroup's share of the row, left for the merge
+      const int64_t grow = ((int64_t)b * p.N * p.n_rep + qhead) * S + row_s;
+      float* slot = p.part + (grow * n_split + ks) * (H + 4);
+#pragma unroll
+      for (int jj = 0; jj < MTL; jj += VG) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int d = 16 * jj + VG * (4 * g + c);
+          if (VG == 4) {
+            if (d + 4 <= H) store4_out(slot + d, f32x4{o[jj][c], o[jj + (1 % VG)][c], o[jj + (2 % VG)][c], o[jj + (3 % VG)][c]});
+          } else {
+            if (d + 2 <= H) store2_out(slot + d, f32x2{o[jj][c], o[jj + (1 % VG)][c]});
+          }
+        }
+      }
+      if (g == 0) slot[H] = m_run, slot[H + 1] = l_run;
+      return;
+    }
+  }
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   T* orow = PAGED ? static_cast<T*>(p.out) + b * p.o_sb + qhead * p.o_sh + row_s * p.o_ss : static_cast<T*>(p.out) + (pair * S + row) * H;
   // o[j][c] of lane (row, g) is the output at dim v_dim(j, 4 g + c)
@@ -353,6 +382,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   attn_dense_body<float, MT, HP, true, false, EXACT, true>(p);
 }
 
+// Ends a launch whose sequences were cut over several workgroups: out = sum_i e^(m_i - M) o_i / sum_i e^(m_i - M) l_i
+// per query row; lane t owns dims 4t .. 4t + 3.
+__global__ __launch_bounds__(64) void attn_paged_f32_merge_kernel(const DenseParams p) {
+  const int64_t grow = blockIdx.x;  // (b, query head, token)
+  const int S = p.S, H = p.H, heads = p.N * p.n_rep;
+  const int s = (int)(grow % S), hq = (int)((grow / S) % heads), b = (int)(grow / ((int64_t)S * heads));
+  const float* slot = p.part + grow * p.n_split * (H + 4);
+  float M = kNegInf;
+  for (int i = 0; i < p.n_split; ++i) M = fmaxf(M, slot[i * (H + 4) + H]);
+  const float m_use = (M == kNegInf) ? 0.f : M;
+  const int d = 4 * threadIdx.x;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float L = 0.f;
+  for (int i = 0; i < p.n_split; ++i) {
+    const float* ps = slot + i * (H + 4);
+    const float w = exp_of(ps[H] - m_use);
+    L += w * ps[H + 1];
+    if (d < H) acc += load4_f32(ps + d) * w;
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  if (d < H) store4_out(static_cast<float*>(p.out) + b * p.o_sb + hq * p.o_sh + s * p.o_ss + d, acc * inv);
+}
+
 int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a, const char* who, hipStream_t stream) {
   PACE_REQUIRE(a->batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
   DenseParams p = {};
@@ -370,8 +422,23 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
   PACE_REQUIRE(rows < (1 << 27), "%s: too many query rows per KV head", who);
   p.l_split = rows <= 16 ? 4 : (rows <= 32 ? 2 : 1);
   const int rowgroups = (int)((rows + 15) / 16), per_wg = 4 / p.l_split;
-  const dim3 grid((rowgroups + per_wg - 1) / per_wg, pool->num_kv_heads, a->batch);
   const int H = pool->head_dim;
+  // A batch that leaves compute units idle: cut the keys of every row group over several workgroups, as many as fill the
+  // GPU twice, as leave a wave four tiles of the longest sequence, and as the caller's workspace has room for.
+  const int64_t wgs = (int64_t)((rowgroups + per_wg - 1) / per_wg) * pool->num_kv_heads * a->batch;
+  const int64_t rows_total = (int64_t)a->batch * a->num_q_heads * a->q_len;
+  p.n_split = 1, p.part = nullptr;
+  if (a->workspace && aligned16(a->workspace) && wgs < 2 * compute_units()) {
+    const int64_t tiles = (a->max_seq_len + 15) / 16;
+    int64_t n = (2 * compute_units() + wgs - 1) / wgs;
+    n = n < tiles / (4 * p.l_split) ? n : tiles / (4 * p.l_split);
+    const int64_t room = (int64_t)(a->workspace_bytes / ((size_t)rows_total * (H + 4) * sizeof(float)));
+    n = n < room ? n : room;
+    n = n < 64 ? n : 64;
+    if (n > 1) p.n_split = (int)n, p.part = static_cast<float*>(a->workspace);
+  }
+  PACE_REQUIRE(rows_total < ((int64_t)1 << 31), "%s: too many query rows", who);
+  const dim3 grid((unsigned)((rowgroups + per_wg - 1) / per_wg * p.n_split), pool->num_kv_heads, a->batch);
   const bool mf32 = a->mask_dtype == PACE_DTYPE_F32;
 #define PACE_PAGED_F32_GO(MT_, HP_) \
   do { \
@@ -390,6 +457,10 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
 #undef PACE_PAGED_F32_HP
 #undef PACE_PAGED_F32_GO
   PACE_HIP_CHECK(hipGetLastError());
+  if (p.n_split > 1) {
+    hipLaunchKernelGGL(attn_paged_f32_merge_kernel, dim3((unsigned)rows_total), dim3(64), 0, stream, p);
+    PACE_HIP_CHECK(hipGetLastError());
+  }
   return PACE_KV_OK;
 }
 

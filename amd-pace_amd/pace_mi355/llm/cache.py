@@ -541,6 +541,10 @@ class PagedKVCache(KVCacheBase):
             # rows of fp32: one launch of the dense operator's kernel over the block table, no work list, no workspace
             items = parts = None
             n_items = max_parts = ws_bytes = 0
+            rows = S * (hq // self.num_kv_heads)
+            if B * self.num_kv_heads * ((rows + 63) // 64 if rows > 32 else 1) < 512:
+                # a batch that does not fill the GPU: room for the library to cut every sequence over up to 64 workgroups
+                ws_bytes = min(B * hq * S * 64 * (D + 4) * 4, 64 << 20)
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
             a.seq_len_bias = bias
         elif graph is None:

@@ -35,7 +35,10 @@
  * of 4 up to 256, strides in floats.  Append, append_paged, gather,
  * gather_packed, copy_blocks, compact_blocks and the decode / verify attention
  * take such a pool (new tokens, gathered rows, queries and outputs are then
- * fp32 too, and the attention needs no workspace); what folds other steps into
+ * fp32 too; the attention needs no work list, and a workspace only helps it when
+ * the batch leaves compute units idle: with room for batch * num_q_heads * q_len
+ * * parts * (head_dim + 4) floats it cuts every sequence over up to parts <= 64
+ * workgroups); what folds other steps into
  * a launch (pace_rope_append_paged, args->rope, args->k_new) is bf16 only and
  * says so when handed such a pool.
  */

@@ -278,20 +278,60 @@ def test_decode_invariant_to_physical_block_permutation(device):
     assert_bits_equal(a.attend(q), b.attend(q), "permuted blocks")
 
 
+def _direct_args(cache, q, out, max_len):
+    from pace_mi355 import _native as nat
+
+    st = cache.state
+    table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
+    a = nat.PagedAttnArgs()
+    a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+    a.block_table, a.table_stride, a.seq_lens, a.seq_len_bias = table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias
+    a.batch, a.num_q_heads, a.q_len, a.causal = q.shape[0], q.shape[1], q.shape[2], 1
+    a.max_seq_len, a.scale = max_len, q.shape[3] ** -0.5
+    return a, (table, lens_dev)
+
+
+@pytest.mark.parametrize("S,n_rep,D,lens", [(1, 4, 128, [3000, 100]), (3, 4, 128, [3000, 100]), (1, 1, 64, [1029]), (9, 2, 256, [77, 2100, 0]),
+                                             (40, 1, 96, [40, 1500])])
+def test_sequences_cut_over_workgroups_when_a_workspace_is_given(device, S, n_rep, D, lens):
+    """A batch that leaves compute units idle: with a workspace the launch cuts every sequence over several workgroups
+    and merges; without one a workgroup walks its sequence alone.  Both match the oracle."""
+    from pace_mi355 import _native as nat
+
+    B, hkv = len(lens), 2
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=17 + S)
+    q = seeded_q(3, B, hkv * n_rep, S, D, dtype=F32)
+    ref = model.attention(q, n_rep)
+    for b, n in enumerate(lens):
+        if n == 0:
+            ref[b] = 0
+    qd = q.to(device)
+    lib, stream = nat.load(), nat.current_stream_ptr()
+    outs = []
+    for ws_bytes in (0, 8 << 20, 100_000):  # none; room for every cut; room for a few
+        out = torch.full_like(qd, float("nan"))
+        a, keep = _direct_args(cache, qd, out, max(lens))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
+        if ws_bytes:
+            a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
+        fn = lib.pace_paged_attn_decode if S == 1 else lib.pace_paged_attn_verify
+        nat.check(fn(ctypes.byref(cache._desc), ctypes.byref(a), stream))
+        _close(out, ref, f"workspace of {ws_bytes} bytes")
+        outs.append(out.cpu())
+    assert not torch.equal(outs[0], outs[1]), "the cut was expected to change the order of the sums"
+    assert_bits_equal(cache.attend(qd), outs[1], "PagedKVCache.attend passes a workspace for small batches")
+
+
 def test_entry_points_that_fold_steps_in_refuse_an_fp32_pool(device):
     from pace_mi355 import _native as nat
 
     cache, _ = _build(device, 2, 2, 2, 128, [20, 5], seed=1)
     lib = nat.load()
-    st = cache.state
-    table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
     q = seeded_q(3, 2, 4, 1, 128, dtype=F32).to(device)
     out = torch.empty_like(q)
-    a = nat.PagedAttnArgs()
-    a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
-    a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
-    a.block_table, a.table_stride, a.seq_lens, a.seq_len_bias = table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias
-    a.batch, a.num_q_heads, a.q_len, a.causal, a.max_seq_len, a.scale = 2, 4, 1, 1, 20, 128 ** -0.5
+    a, (table, lens_dev) = _direct_args(cache, q, out, 20)
+    bias = a.seq_len_bias
     stream = nat.current_stream_ptr()
     # the entry point that allocates nothing takes the pool too (this kernel has no scratch at all)
     nat.check(lib.pace_paged_attn_verify_static(ctypes.byref(cache._desc), ctypes.byref(a), stream))
@@ -353,3 +393,42 @@ def test_random_histories(device, seed):
         if min(model.seq_lens()) >= S:
             q = seeded_q(step, B, hkv * n_rep, S, D, dtype=F32)
             _close(cache.attend(q.to(device)), model.attention(q, n_rep), f"attention after step {step} ({op})")
+
+
+def test_manager_with_fp32_layers_and_beam_reorder(device):
+    """The manager's call order of a model step (update per layer, attention, rollback, beam gather:
+    ``pace/llm/cache.py:48-123``) with fp32 K/V; every layer shares the one block table."""
+    from pace_mi355.llm import KVCacheManager, KVCacheType
+    from pace_mi355.ops import MultiHeadAttention
+
+    class Cfg:
+        num_hidden_layers = 2
+        num_attention_heads = 8
+        num_key_value_heads = 2
+
+    B = 3
+    mgr = KVCacheManager(Cfg(), 96, KVCacheType.PAGED)
+    refs = [DynamicKVCacheRef(96) for _ in range(2)]
+    mha = MultiHeadAttention(dtype=F32)
+    for step, T in enumerate([30, 1, 1, 5]):
+        for layer in range(2):
+            k, v = seeded_kv(400 + 10 * step + layer, B, 2, T, 128, dtype=F32)
+            ke, ve = repeat_kv(k, 4), repeat_kv(v, 4)
+            rk, rv = refs[layer].update_cache(ke, ve, 2)
+            pk, pv = mgr[layer].update_cache(ke.to(device), ve.to(device), 2)
+            q = seeded_q(500 + step, B, 8, T, 128, dtype=F32)
+            L = refs[layer].seq_len
+            mask = causal_mask_4d(torch.ones(B, L, dtype=torch.long), T, L, F32)
+            out = mha(q.to(device), pk, pv, attention_mask=mask.to(device))
+            _close(out, sdpa_fp32(q, rk, rv, mask), f"step {step} layer {layer}")
+        assert len(mgr) == refs[0].seq_len
+    mgr.remove_cache(3)
+    beam = torch.tensor([2, 0, 0])
+    mgr.update_cache_with_beam_indices(beam.to(device))
+    for layer in range(2):
+        refs[layer].remove_cache(3)
+        refs[layer].update_cache_with_beam_indices(beam)
+        rk, rv = valid_prefix(refs[layer])
+        assert_bits_equal(mgr[layer].key.dense(), rk, f"layer {layer} K")
+        assert_bits_equal(mgr[layer].value.dense(), rv, f"layer {layer} V")
+    assert mgr[0].state is mgr[1].state and mgr[0].pool.dtype == F32
