@@ -89,8 +89,15 @@ struct DenseParams {
 // wave per SIMD at head size 128).  It pays where the launch is bound by memory (few query rows: +8 % on an fp32
 // decode step) and costs 10 % where it is bound by the matrix cores, so the launcher picks.
 // EXACT: H == HP (and VEC): no bound on a dim is checked anywhere, which is a third of the vector instructions of a tile.
-template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED>
+// COOP (row groups that do not share their keys with other waves, H == HP): the four waves of a workgroup walk the
+// same keys, so the workgroup fetches every tile once -- 16 bytes per thread and load, a tile ahead, in registers
+// over the tile's arithmetic -- and hands it round through LDS (two stages, one barrier per tile); rows keep their
+// order there with their 16-byte chunks rotated by the row number, which keeps the operand reads of sixteen rows
+// (the first product) and of sixteen chunks of a row (the second) off each other's banks.  Each wave fetching its
+// own operands from memory held the launch at 65 % of what the arithmetic alone takes.
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED, bool COOP = false>
 __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
+  static_assert(!COOP || (EXACT && !AHEAD && sizeof(T) == 4), "the cooperative walk: fp32 rows of a built head size");
   static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
   static_assert(!PAGED || (VEC && sizeof(T) == 4), "pools of rows hold fp32 with head sizes that are multiples of 4");
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
@@ -98,7 +105,10 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   constexpr int VG = MTL % 4 == 0 ? 4 : 2;  // output tiles whose dims of a lane are neighbours (see the V loads)
   static_assert(MTL % VG == 0, "head sizes built: multiples of 32");
   constexpr int ROW_F = HP + 2;
-  __shared__ float merge_buf[2 * 16 * ROW_F];
+  constexpr int CPR = HP / 4;            // 16-byte chunks of a row
+  constexpr int STAGE_F = 2 * 16 * HP;   // floats of one stage: the K tile, then the V tile
+  __shared__ __attribute__((aligned(16))) float lds_f[COOP ? 2 * STAGE_F : 2 * 16 * ROW_F];
+  float* const merge_buf = lds_f;
   const int H = EXACT ? HP : p.H, S = p.S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g = lane >> 4;
   const int split = p.l_split;
@@ -179,6 +189,30 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   const int tile_lo = min(wg_hi, wg_lo + ls * per), tile_hi = min(wg_hi, tile_lo + per);
   const bool has_rows = rowgroup * 16 < R;  // wave-uniform
   float kf[KS], vf[MTL][4], mv[4];
+  auto fetch_mask = [&](int tile, float (&mx4)[4]) {
+    // the lane's four mask values: one load where the four columns exist (mask lines start wherever L puts them;
+    // the hardware takes unaligned multi-dword loads), element by element at the end of a line
+    const int t = tile * 16 + 4 * g;
+    if (!mrow) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx4[i] = 0.f;
+    } else if (t + 4 <= mcols) {
+      if constexpr (sizeof(MT) == 4) {
+        u32x4 raw;
+        __builtin_memcpy(&raw, mrow + t, 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx4[i] = __uint_as_float(raw[i]);
+      } else {
+        u32x2 raw;
+        __builtin_memcpy(&raw, mrow + t, 8);
+        mx4[0] = __uint_as_float(raw[0] << 16), mx4[1] = __uint_as_float(raw[0] & 0xffff0000u);
+        mx4[2] = __uint_as_float(raw[1] << 16), mx4[3] = __uint_as_float(raw[1] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx4[i] = (t + i < mcols) ? load_f32<MT>(mrow + t + i) : 0.f;
+    }
+  };
   auto fetch = [&](int tile, float (&kx)[KS], float (&vx)[MTL][4], float (&mx4)[4]) {
     const int t0 = tile * 16;
     const T* kblock = kbase;
@@ -213,39 +247,10 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
         }
       }
     }
-    // the lane's four mask values: one load where the four columns exist (mask lines start wherever L puts them;
-    // the hardware takes unaligned multi-dword loads), element by element at the end of a line
-    const int t = t0 + 4 * g;
-    if (!mrow) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx4[i] = 0.f;
-    } else if (t + 4 <= mcols) {
-      if constexpr (sizeof(MT) == 4) {
-        u32x4 raw;
-        __builtin_memcpy(&raw, mrow + t, 16);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) mx4[i] = __uint_as_float(raw[i]);
-      } else {
-        u32x2 raw;
-        __builtin_memcpy(&raw, mrow + t, 8);
-        mx4[0] = __uint_as_float(raw[0] << 16), mx4[1] = __uint_as_float(raw[0] & 0xffff0000u);
-        mx4[2] = __uint_as_float(raw[1] << 16), mx4[3] = __uint_as_float(raw[1] & 0xffff0000u);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx4[i] = (t + i < mcols) ? load_f32<MT>(mrow + t + i) : 0.f;
-    }
+    fetch_mask(tile, mx4);
   };
-  if (AHEAD && has_rows && tile_lo < tile_hi) fetch(tile_lo, kf, vf, mv);
-  for (int tile = tile_lo; has_rows && tile < tile_hi; ++tile) {
-    const int t0 = tile * 16;
-    float kn[AHEAD ? KS : 1], vn[AHEAD ? MTL : 1][4], mn[4];
-    const bool more = AHEAD && tile + 1 < tile_hi;
-    if constexpr (AHEAD) {
-      if (more) fetch(tile + 1, kn, vn, mn);
-    } else {
-      fetch(tile, kf, vf, mv);
-    }
+  // One tile's arithmetic on the operands at hand.
+  auto tile_math = [&](int t0, const float (&kf)[KS], const float (&vf)[MTL][4], const float (&mv)[4]) {
     f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < KS; ++s) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], sc, 0, 0, 0);
@@ -281,16 +286,137 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < MTL; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j][i], pr[i], o[j], 0, 0, 0);
+  };
+  if constexpr (COOP) {
+    // Every wave of the workgroup passes every barrier: the walk covers the tiles any of its row groups reads, a wave
+    // computes on those of its own range.
+    int wg_end = L;
+    if constexpr (PAGED) {
+      if (p.causal) {  // the last token any row of the workgroup's four row groups reads (as key_end above, per group)
+        wg_end = 0;
+        for (int gi = wg_x * 4; gi < wg_x * 4 + 4 && gi * 16 < R; ++gi) {
+          const int s0 = (gi * 16) % S;
+          wg_end = max(wg_end, min(L, L - S + (s0 + 15 < S ? s0 + 15 : S - 1) + 1));
+        }
+      }
+    }
+    const int walk_lo = tile_first, walk_hi = max(tile_first, (wg_end + 15) / 16);
+    constexpr int TILE_CHUNKS = 16 * CPR, PER_T = (TILE_CHUNKS + 255) / 256;
+    auto rot = [](int x) { return (CPR & (CPR - 1)) == 0 ? (x & (CPR - 1)) : (x >= CPR ? x - CPR : x); };  // x < CPR + 16
+    // Offsets that do not change from tile to tile, formed once (the stage and the K / V half are constants of the
+    // instruction): where this thread's chunks of a tile come from and go to, where this lane's operands lie.
+    int src_row[PER_T], src_col[PER_T], dst_at[PER_T], k_at[KS / 4], v_at[4][MTL / VG];
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) {
+      const int id = min((int)threadIdx.x + 256 * i, TILE_CHUNKS - 1), r = id / CPR, c = id % CPR;
+      src_row[i] = r, src_col[i] = 4 * c, dst_at[i] = 4 * (r * CPR + rot(c + r));
+    }
+#pragma unroll
+    for (int k = 0; k < KS / 4; ++k) k_at[k] = 4 * (n * CPR + rot(d0 / 4 + k + n));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int jv = 0; jv < MTL / VG; ++jv) {
+        const int r = 4 * g + i, d = 16 * VG * jv + VG * n;
+        v_at[i][jv] = 4 * (r * CPR + rot(d / 4 + r)) + d % 4;
+      }
+    u32x4 sk[PER_T], sv[PER_T];
+    auto stage_load = [&](int tile) {
+      const int t0 = tile * 16;
+      const T* kblock = kbase + (int64_t)t0 * H;
+      const T* vblock = vbase + (int64_t)t0 * H;
+      if constexpr (PAGED) {
+        const int64_t blk = min(max(p.table[(int64_t)b * p.table_stride + min(tile, p.table_stride - 1)], 0), p.num_blocks - 1);
+        kblock = kbase + blk * p.k_bs, vblock = vbase + blk * p.v_bs;
+      }
+#pragma unroll
+      for (int i = 0; i < PER_T; ++i) {
+        if (TILE_CHUNKS % 256 == 0 || (int)threadIdx.x + 256 * i < TILE_CHUNKS) {
+          // rows past the end are masked in the arithmetic (PAGED: the block's 16 rows exist whatever the length is)
+          const int r = PAGED ? src_row[i] : min(L - 1 - t0, src_row[i]);
+          sk[i] = *reinterpret_cast<const u32x4*>(kblock + r * H + src_col[i]);
+          sv[i] = *reinterpret_cast<const u32x4*>(vblock + r * H + src_col[i]);
+        }
+      }
+    };
+    auto stage_store = [&](auto stage_c) {
+      constexpr int stage = decltype(stage_c)::value;
+#pragma unroll
+      for (int i = 0; i < PER_T; ++i) {
+        if (TILE_CHUNKS % 256 == 0 || (int)threadIdx.x + 256 * i < TILE_CHUNKS) {
+          *reinterpret_cast<u32x4*>(lds_f + stage * STAGE_F + dst_at[i]) = sk[i];
+          *reinterpret_cast<u32x4*>(lds_f + stage * STAGE_F + 16 * HP + dst_at[i]) = sv[i];
+        }
+      }
+    };
+    auto operands = [&](auto stage_c, float (&kx)[KS], float (&vx)[MTL][4]) {
+      constexpr int stage = decltype(stage_c)::value;
+#pragma unroll
+      for (int k = 0; k < KS / 4; ++k) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(lds_f + stage * STAGE_F + k_at[k]);
+        kx[4 * k] = t[0], kx[4 * k + 1] = t[1], kx[4 * k + 2] = t[2], kx[4 * k + 3] = t[3];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int jv = 0; jv < MTL / VG; ++jv) {
+          const float* at = lds_f + stage * STAGE_F + 16 * HP + v_at[i][jv];
+          if (VG == 4) {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(at);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vx[VG * jv + (e % VG)][i] = t[e];
+          } else {
+            const f32x2 t = *reinterpret_cast<const f32x2*>(at);
+            vx[VG * jv][i] = t[0], vx[VG * jv + (1 % VG)][i] = t[1];
+          }
+        }
+      }
+    };
+    auto walk = [&](int tile, auto stage_c) {
+      constexpr int stage = decltype(stage_c)::value;
+      const bool more = tile + 1 < walk_hi;
+      if (more) stage_load(tile + 1);  // in flight over this tile's arithmetic
+      if (has_rows && tile >= tile_lo && tile < tile_hi) {
+        fetch_mask(tile, mv);
+        operands(stage_c, kf, vf);
+        tile_math(tile * 16, kf, vf, mv);
+      }
+      // (the other stage was last read before the barrier that ended the tile before this one)
+      if (more) stage_store(std::integral_constant<int, stage ^ 1>{});
+      __syncthreads();
+    };
+    if (walk_lo < walk_hi) {
+      stage_load(walk_lo);
+      stage_store(std::integral_constant<int, 0>{});
+    }
+    __syncthreads();
+    for (int tile = walk_lo; tile < walk_hi; tile += 2) {
+      walk(tile, std::integral_constant<int, 0>{});
+      if (tile + 1 < walk_hi) walk(tile + 1, std::integral_constant<int, 1>{});
+    }
+  } else {
+    if (AHEAD && has_rows && tile_lo < tile_hi) fetch(tile_lo, kf, vf, mv);
+    for (int tile = tile_lo; has_rows && tile < tile_hi; ++tile) {
+      const int t0 = tile * 16;
+      float kn[AHEAD ? KS : 1], vn[AHEAD ? MTL : 1][4], mn[4];
+      const bool more = AHEAD && tile + 1 < tile_hi;
+      if constexpr (AHEAD) {
+        if (more) fetch(tile + 1, kn, vn, mn);
+      } else {
+        fetch(tile, kf, vf, mv);
+      }
+      tile_math(t0, kf, vf, mv);
     if constexpr (AHEAD) {
-      if (more) {
+        if (more) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) kf[s] = kn[s];
+          for (int s = 0; s < KS; ++s) kf[s] = kn[s];
 #pragma unroll
-        for (int j = 0; j < MTL; ++j)
+          for (int j = 0; j < MTL; ++j)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) vf[j][i] = vn[j][i];
+            for (int i = 0; i < 4; ++i) vf[j][i] = vn[j][i];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) mv[i] = mn[i];
+          for (int i = 0; i < 4; ++i) mv[i] = mn[i];
+        }
       }
     }
   }
@@ -373,6 +499,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   attn_dense_body<T, MT, HP, VEC, AHEAD, EXACT, false>(p);
 }
 
+// fp32 rows of a built head size, row groups with keys of their own (more than 32 query rows): the workgroup shares
+// its tiles through LDS (COOP above).  PAGED: over a pool of fp32 rows.
+template <typename MT, int HP, bool PAGED>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_coop_kernel(
+    const DenseParams p) {
+  attn_dense_body<float, MT, HP, true, false, true, PAGED, true>(p);
+}
+
 // The same walk over a pool of fp32 rows (pace_kv_pool_t with elem_bytes 4).  No fetch a tile ahead: here the second
 // wave per SIMD hides more than the second set of registers did (decode, batch 64 x 8 KV heads x 4096 tokens of 128
 // dims: 370 us against 460).
@@ -440,9 +574,11 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
   PACE_REQUIRE(rows_total < ((int64_t)1 << 31), "%s: too many query rows", who);
   const dim3 grid((unsigned)((rowgroups + per_wg - 1) / per_wg * p.n_split), pool->num_kv_heads, a->batch);
   const bool mf32 = a->mask_dtype == PACE_DTYPE_F32;
+  const bool coop = p.l_split == 1 && p.n_split == 1;
 #define PACE_PAGED_F32_GO(MT_, HP_) \
   do { \
-    if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
+    if (H == HP_ && coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
+    else if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
     else hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false>), grid, dim3(256), 0, stream, p); \
   } while (0)
 #define PACE_PAGED_F32_HP(MT_) \
@@ -523,6 +659,12 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
 #define PACE_DENSE_GO(T_, MT_, HP_) \
   do { \
     constexpr bool kAheadBuilt = HP_ <= 128; /* at 256 the second set of registers does not fit */ \
+    if constexpr (sizeof(T_) == 4) { \
+      if (vec && H == HP_ && p.l_split == 1) { \
+        hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false>), grid, dim3(256), 0, s, p); \
+        break; \
+      } \
+    } \
     if (ahead && kAheadBuilt) { \
       if (vec && H == HP_) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt, true>), grid, dim3(256), 0, s, p); \
       else if (vec) hipLaunchKernelGGL((attn_dense_kernel<T_, MT_, HP_, true, kAheadBuilt, false>), grid, dim3(256), 0, s, p); \
