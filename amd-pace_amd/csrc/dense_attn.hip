@@ -89,15 +89,16 @@ struct DenseParams {
 // wave per SIMD at head size 128).  It pays where the launch is bound by memory (few query rows: +8 % on an fp32
 // decode step) and costs 10 % where it is bound by the matrix cores, so the launcher picks.
 // EXACT: H == HP (and VEC): no bound on a dim is checked anywhere, which is a third of the vector instructions of a tile.
-// COOP (row groups that do not share their keys with other waves, H == HP): the four waves of a workgroup walk the
+// COOP (row groups that do not share their keys with other waves, fp32 rows): the four waves of a workgroup walk the
 // same keys, so the workgroup fetches every tile once -- 16 bytes per thread and load, a tile ahead, in registers
 // over the tile's arithmetic -- and hands it round through LDS (two stages, one barrier per tile); rows keep their
 // order there with their 16-byte chunks rotated by the row number, which keeps the operand reads of sixteen rows
-// (the first product) and of sixteen chunks of a row (the second) off each other's banks.  Each wave fetching its
+// (the first product) and of sixteen chunks of a row (the second) off each other's banks; a head size below the built
+// one is padded with zeros on the way in.  Each wave fetching its
 // own operands from memory held the launch at 65 % of what the arithmetic alone takes.
 template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED, bool COOP = false>
 __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
-  static_assert(!COOP || (EXACT && !AHEAD && sizeof(T) == 4), "the cooperative walk: fp32 rows of a built head size");
+  static_assert(!COOP || (VEC && !AHEAD && sizeof(T) == 4), "the cooperative walk: fp32 rows of a multiple of four dims");
   static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
   static_assert(!PAGED || (VEC && sizeof(T) == 4), "pools of rows hold fp32 with head sizes that are multiples of 4");
   constexpr int KS = HP / 4;   // contraction steps of the first product = dims per lane
@@ -254,32 +255,36 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < KS; ++s) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], sc, 0, 0, 0);
-    float val[4], mx = kNegInf;
+    // The softmax reference of a row moves lazily: only when a score lies more than kLazy above it (weights stay below
+    // e^kLazy = 245, far inside fp32), which in a row of a few hundred keys happens a handful of times instead of in
+    // most tiles -- and the accumulators are rescaled only then.  Whether any row of the wave moves is decided by
+    // comparing the lane's own scores with the threshold; the row maximum is formed only when one does.
+    constexpr float kLazy = 5.5f;
+    const float top = m_run + kLazy;  // (-inf while the row has seen nothing)
+    float val[4];
+    bool above = false;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int tk = t0 + 4 * g + i;
       val[i] = (tk < limit && (!PAGED || tk >= start)) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
-      mx = fmaxf(mx, val[i]);
+      above = above || val[i] > top;
     }
-    mx = row_max4(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = exp_of(m_run - m_use);
-    float pr[4], sum = 0.f;
+    if (__any(above)) {
+      const float mx = row_max4(fmaxf(fmaxf(val[0], val[1]), fmaxf(val[2], val[3])));
+      const float m_new = mx > top ? mx : m_run;  // (the same in the four lanes of a row)
+      const float alpha = exp_of(m_run - ((m_new == kNegInf) ? 0.f : m_new));  // 1 for a row that stays, 0 for a first score
+      l_run *= alpha;
+#pragma unroll
+      for (int j = 0; j < MTL; ++j) o[j] *= alpha;
+      m_run = m_new;
+    }
+    const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+    float pr[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       pr[i] = exp_of(val[i] - m_use);
-      sum += pr[i];
+      l_run += pr[i];
     }
-    // (no row of the wave has a new maximum: alpha is exactly 1 in every lane, and the products with it are skipped)
-    if (__any(m_new != m_run)) {
-      l_run = l_run * alpha + sum;
-#pragma unroll
-      for (int j = 0; j < MTL; ++j) o[j] *= alpha;
-    } else {
-      l_run += sum;
-    }
-    m_run = m_new;
     // token quarter by token quarter over all output tiles: neighbouring matrix instructions write different
     // accumulators (per tile the order of the four is unchanged)
 #pragma unroll
@@ -334,8 +339,11 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
         if (TILE_CHUNKS % 256 == 0 || (int)threadIdx.x + 256 * i < TILE_CHUNKS) {
           // rows past the end are masked in the arithmetic (PAGED: the block's 16 rows exist whatever the length is)
           const int r = PAGED ? src_row[i] : min(L - 1 - t0, src_row[i]);
-          sk[i] = *reinterpret_cast<const u32x4*>(kblock + r * H + src_col[i]);
-          sv[i] = *reinterpret_cast<const u32x4*>(vblock + r * H + src_col[i]);
+          sk[i] = sv[i] = u32x4{0u, 0u, 0u, 0u};
+          if (EXACT || src_col[i] < H) {  // (dims the rows do not have read as zero)
+            sk[i] = *reinterpret_cast<const u32x4*>(kblock + r * H + src_col[i]);
+            sv[i] = *reinterpret_cast<const u32x4*>(vblock + r * H + src_col[i]);
+          }
         }
       }
     };
@@ -499,12 +507,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
   attn_dense_body<T, MT, HP, VEC, AHEAD, EXACT, false>(p);
 }
 
-// fp32 rows of a built head size, row groups with keys of their own (more than 32 query rows): the workgroup shares
+// fp32 rows of a multiple of four dims, row groups with keys of their own (more than 32 query rows): the workgroup shares
 // its tiles through LDS (COOP above).  PAGED: over a pool of fp32 rows.
-template <typename MT, int HP, bool PAGED>
+template <typename MT, int HP, bool PAGED, bool EXACT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_coop_kernel(
     const DenseParams p) {
-  attn_dense_body<float, MT, HP, true, false, true, PAGED, true>(p);
+  attn_dense_body<float, MT, HP, true, false, EXACT, PAGED, true>(p);
 }
 
 // The same walk over a pool of fp32 rows (pace_kv_pool_t with elem_bytes 4).  No fetch a tile ahead: here the second
@@ -577,7 +585,8 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
   const bool coop = p.l_split == 1 && p.n_split == 1;
 #define PACE_PAGED_F32_GO(MT_, HP_) \
   do { \
-    if (H == HP_ && coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
+    if (H == HP_ && coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true, true>), grid, dim3(256), 0, stream, p); \
+    else if (coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true, false>), grid, dim3(256), 0, stream, p); \
     else if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
     else hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false>), grid, dim3(256), 0, stream, p); \
   } while (0)
@@ -660,8 +669,9 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
   do { \
     constexpr bool kAheadBuilt = HP_ <= 128; /* at 256 the second set of registers does not fit */ \
     if constexpr (sizeof(T_) == 4) { \
-      if (vec && H == HP_ && p.l_split == 1) { \
-        hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false>), grid, dim3(256), 0, s, p); \
+      if (vec && p.l_split == 1) { \
+        if (H == HP_) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false, true>), grid, dim3(256), 0, s, p); \
+        else hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false, false>), grid, dim3(256), 0, s, p); \
         break; \
       } \
     } \

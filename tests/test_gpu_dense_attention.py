@@ -22,6 +22,8 @@ CASES = [
     (2, 4, 1, 96, 700), (1, 3, 100, 96, 333), (2, 2, 1, 256, 900), (1, 2, 70, 256, 130), (1, 2, 9, 100, 50),
     # head sizes off every built one: not a multiple of 4 (element by element), 30 (the 32 build), 80 over several tiles
     (1, 2, 40, 50, 90), (1, 2, 20, 30, 45), (1, 2, 64, 80, 300),
+    # the smallest build on the walk that shares its tiles (half a tile of chunks per load), exact and padded
+    (1, 2, 48, 32, 100), (2, 1, 100, 28, 75),
 ]
 
 

@@ -183,7 +183,8 @@ def test_decode_matches_oracle(device, B, hkv, n_rep, D, lens):
 
 
 @pytest.mark.parametrize("S,lens,n_rep,D", [(2, [40, 41], 4, 128), (8, [100, 8, 515], 4, 128), (16, [16, 33, 700], 1, 64),
-                                             (20, [20, 333], 2, 128), (70, [70, 200], 4, 96), (130, [130, 400], 1, 256)])
+                                             (20, [20, 333], 2, 128), (70, [70, 200], 4, 96), (130, [130, 400], 1, 256),
+                                             (48, [48, 300], 2, 80), (33, [33, 100], 1, 100), (40, [77, 40, 1000], 4, 128)])
 def test_verify_causal_matches_oracle(device, S, lens, n_rep, D):
     """S new tokens already appended; row s reads tokens <= len - S + s (``llama.py:292-299``)."""
     B, hkv = len(lens), 2
