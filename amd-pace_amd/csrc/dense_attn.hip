@@ -14,8 +14,10 @@
 //       supplies V[token 4g+i][dim 16j+n] and its own probability of token 4g+i,
 // so probabilities never leave their lane and the state of query row n lives in lanes (n, 0..3).
 // The four waves of a workgroup take four row groups, or split the keys of fewer row groups among
-// themselves (few query rows: decode) and merge through LDS.  Operands come straight from global
-// memory: at 32 cycles per matrix instruction their traffic is far from any limit.
+// themselves (few query rows: decode) and merge through LDS.  Four row groups of fp32 rows share
+// the tiles they walk: the workgroup fetches each once and hands it round through LDS (COOP below);
+// elsewhere every wave takes its operands straight from global memory.  The same body walks a pool of
+// fp32 rows through its block table (PAGED).
 #include "attn_core.h"
 
 namespace pace_kv {
