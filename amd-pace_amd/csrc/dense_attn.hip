@@ -512,7 +512,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 // fp32 rows of a multiple of four dims, row groups with keys of their own (more than 32 query rows): the workgroup shares
 // its tiles through LDS (COOP above).  PAGED: over a pool of fp32 rows.
 template <typename MT, int HP, bool PAGED, bool EXACT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_dense_coop_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_f32_coop_kernel(
     const DenseParams p) {
   attn_dense_body<float, MT, HP, true, false, EXACT, PAGED, true>(p);
 }
@@ -587,8 +587,8 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
   const bool coop = p.l_split == 1 && p.n_split == 1;
 #define PACE_PAGED_F32_GO(MT_, HP_) \
   do { \
-    if (H == HP_ && coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true, true>), grid, dim3(256), 0, stream, p); \
-    else if (coop) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, true, false>), grid, dim3(256), 0, stream, p); \
+    if (H == HP_ && coop) hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, true, true>), grid, dim3(256), 0, stream, p); \
+    else if (coop) hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, true, false>), grid, dim3(256), 0, stream, p); \
     else if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
     else hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false>), grid, dim3(256), 0, stream, p); \
   } while (0)
@@ -672,8 +672,8 @@ extern "C" int pace_attn_dense_ws(const void* q, const void* k, const void* v, v
     constexpr bool kAheadBuilt = HP_ <= 128; /* at 256 the second set of registers does not fit */ \
     if constexpr (sizeof(T_) == 4) { \
       if (vec && p.l_split == 1) { \
-        if (H == HP_) hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false, true>), grid, dim3(256), 0, s, p); \
-        else hipLaunchKernelGGL((attn_dense_coop_kernel<MT_, HP_, false, false>), grid, dim3(256), 0, s, p); \
+        if (H == HP_) hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, false, true>), grid, dim3(256), 0, s, p); \
+        else hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, false, false>), grid, dim3(256), 0, s, p); \
         break; \
       } \
     } \

@@ -637,7 +637,7 @@ def wl_dense_f32(torch, dev, args):
     return result_line(
         args, "dense op on fp32 tensors: batch 8, 32 heads, 512 queries x 512 keys, head_dim 128, additive mask [B,1,1,L]; "
         "step = one torch.ops.pace.attention call (output allocation included)", once, B * S, dt,
-        {"bound": "mfma", "kernel": "attn_dense_coop_kernel<float,128,false,true>", "achieved": round(tflops, 1),
+        {"bound": "mfma", "kernel": "attn_f32_coop_kernel<float,128,false,true>", "achieved": round(tflops, 1),
          "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops / MFMA_F32_PEAK_TFLOPS, 4), "traffic": None,
          "flops_per_launch": flops, "avg_launch_ms": round(attn_ms, 5)}, extra={"dtype": "f32"})
 
