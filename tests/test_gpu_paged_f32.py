@@ -197,6 +197,34 @@ def test_verify_causal_matches_oracle(device, S, lens, n_rep, D):
     assert_bits_equal(cache.attend(qt), out, "strided queries")
 
 
+@pytest.mark.parametrize("S,n_rep,D", [(40, 2, 128), (70, 1, 80), (5, 4, 64)])
+def test_kv_start_and_mask_tensors_with_many_query_rows(device, S, n_rep, D):
+    """The launches whose workgroups share their tiles (more than 32 query rows per KV head), and a small one beside
+    them: a first readable token per sequence, then an explicit mask tensor of each dtype with fewer columns than
+    the longest sequence has tokens."""
+    from oracle.attention_ref import lengths_mask_4d
+
+    lens, hkv = [S + 3, 300, S + 130], 2
+    B = len(lens)
+    cache, model = _build(device, B, hkv, n_rep, D, lens, seed=S)
+    q = seeded_q(4, B, hkv * n_rep, S, D, dtype=F32)
+    K, V = model.dense(n_rep)
+    start = torch.tensor([2, 37, 100], dtype=torch.int32)
+    out = cache.attend(q.to(device), kv_start=start.to(device))
+    _close(out, sdpa_fp32(q, K, V, lengths_mask_4d(lens, S, K.shape[2], F32, kv_start=start)), "kv_start")
+    g = torch.Generator().manual_seed(S)
+    for mdt in (torch.float32, torch.bfloat16):
+        cols = 290
+        m = torch.randn(B, 1, S, cols, generator=g).to(mdt)
+        m[:, :, :, 17:40] = torch.finfo(mdt).min
+        out = cache.attend(q.to(device), m.to(device))
+        # the mask alone decides; a sequence's own length and the mask's width bound the columns
+        full = torch.full((B, 1, S, K.shape[2]), float("-inf"))
+        for b, n in enumerate(lens):
+            full[b, :, :, : min(n, cols)] = m[b, :, :, : min(n, cols)].float()
+        _close(out, sdpa_fp32(q, K, V, full), f"mask tensor {mdt}")
+
+
 @pytest.mark.parametrize("mdt", [torch.float32, torch.bfloat16])
 def test_additive_mask_path_matches_reference_semantics(device, mdt):
     """A left-padded batch the way the reference runs it (shared length, 4-D additive mask,
