@@ -149,6 +149,12 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   }
   // causal: query token s reads keys <= L - S + s
   const int limit = (PAGED && p.causal) ? min(L, L - S + row_s + 1) : L;
+  int limit_lo = limit;  // the smallest limit of the wave's rows (wave-uniform)
+  if constexpr (PAGED) {
+#pragma unroll
+    for (int o = 1; o < 64; o *= 2) limit_lo = min(limit_lo, __shfl_xor(limit_lo, o, 64));
+    limit_lo = __builtin_amdgcn_readfirstlane(limit_lo);
+  }
   // This lane's dims of a row for the first product: d0 .. d0 + KS - 1.
   const int d0 = g * KS;
   auto load_run = [&](const T* r, float (&x)[KS]) {
@@ -265,11 +271,19 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     const float top = m_run + kLazy;  // (-inf while the row has seen nothing)
     float val[4];
     bool above = false;
+    if (t0 + 16 <= limit_lo && (!PAGED || t0 >= start)) {  // every row of the wave reads the whole tile: no bound to check
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int tk = t0 + 4 * g + i;
-      val[i] = (tk < limit && (!PAGED || tk >= start)) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
-      above = above || val[i] > top;
+      for (int i = 0; i < 4; ++i) {
+        val[i] = fmaf(sc[i], p.scale, mv[i]);
+        above = above || val[i] > top;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tk = t0 + 4 * g + i;
+        val[i] = (tk < limit && (!PAGED || tk >= start)) ? fmaf(sc[i], p.scale, mv[i]) : kNegInf;
+        above = above || val[i] > top;
+      }
     }
     if (__any(above)) {
       const float mx = row_max4(fmaxf(fmaxf(val[0], val[1]), fmaxf(val[2], val[3])));
@@ -313,10 +327,12 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     // Offsets that do not change from tile to tile, formed once (the stage and the K / V half are constants of the
     // instruction): where this thread's chunks of a tile come from and go to, where this lane's operands lie.
     int src_row[PER_T], src_col[PER_T], dst_at[PER_T], k_at[KS / 4], v_at[4][MTL / VG];
+    uint32_t src_at[PER_T];
 #pragma unroll
     for (int i = 0; i < PER_T; ++i) {
       const int id = min((int)threadIdx.x + 256 * i, TILE_CHUNKS - 1), r = id / CPR, c = id % CPR;
       src_row[i] = r, src_col[i] = 4 * c, dst_at[i] = 4 * (r * CPR + rot(c + r));
+      src_at[i] = (uint32_t)(r * H + 4 * c) * (uint32_t)sizeof(T);
     }
 #pragma unroll
     for (int k = 0; k < KS / 4; ++k) k_at[k] = 4 * (n * CPR + rot(d0 / 4 + k + n));
@@ -336,15 +352,17 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
         const int64_t blk = min(max(p.table[(int64_t)b * p.table_stride + min(tile, p.table_stride - 1)], 0), p.num_blocks - 1);
         kblock = kbase + blk * p.k_bs, vblock = vbase + blk * p.v_bs;
       }
+      // Rows past the end of a dense tensor are not read (zeros take their place; the arithmetic masks them.  PAGED:
+      // a block's 16 rows exist whatever the length is).  The offsets were formed before the walk -- unsigned 32-bit
+      // byte offsets from a pointer the whole wave shares, which is the load's own addressing: no vector arithmetic
+      // per tile.
 #pragma unroll
       for (int i = 0; i < PER_T; ++i) {
         if (TILE_CHUNKS % 256 == 0 || (int)threadIdx.x + 256 * i < TILE_CHUNKS) {
-          // rows past the end are masked in the arithmetic (PAGED: the block's 16 rows exist whatever the length is)
-          const int r = PAGED ? src_row[i] : min(L - 1 - t0, src_row[i]);
           sk[i] = sv[i] = u32x4{0u, 0u, 0u, 0u};
-          if (EXACT || src_col[i] < H) {  // (dims the rows do not have read as zero)
-            sk[i] = *reinterpret_cast<const u32x4*>(kblock + r * H + src_col[i]);
-            sv[i] = *reinterpret_cast<const u32x4*>(vblock + r * H + src_col[i]);
+          if ((EXACT || src_col[i] < H) && (PAGED || src_row[i] < L - t0)) {  // (dims the rows do not have read as zero)
+            sk[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(kblock) + src_at[i]);
+            sv[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(vblock) + src_at[i]);
           }
         }
       }
