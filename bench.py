@@ -179,8 +179,9 @@ class FixedStep:
         a.batch, a.num_q_heads, a.q_len = B, hq, S
         # the library's planner cuts the batch: descriptors of (sequence, partition) work items in scheduling order
         a.max_seq_len, a.partition_tokens, a.scale = max_len, 0, 1.0 / math.sqrt(D)
-        if cache.f32:  # rows of fp32: one launch over the block table, no work list, no workspace
-            n_items = max_parts = ws_bytes = 0
+        if cache.f32:  # rows of fp32: one launch over the block table, no work list; the workspace lets a small batch be cut
+            n_items = max_parts = 0
+            ws_bytes = min(B * hq * S * 64 * (D + 4) * 4, 64 << 20)
         else:
             self.items, self.parts, n_items, max_parts, ws_bytes = cache.state.plan_attention(
                 lens_after, hq, cache.num_kv_heads, cache.head_dim, S, mask is not None, partition)
