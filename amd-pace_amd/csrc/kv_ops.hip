@@ -19,6 +19,7 @@ struct AppendDest {
   const int32_t* seq_lens;
   int32_t table_stride;
   int32_t pos_offset;
+  const int32_t* offset_dev;  // optional: one more offset, read on the device (a counter a captured graph advances)
 };
 
 template <int D, bool PAGED>
@@ -38,7 +39,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(pace_kv_pool_t pool, con
   int64_t blk;
   int off;
   if (PAGED) {
-    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + t;
+    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + (dest.offset_dev ? *dest.offset_dev : 0) + t;
     if (pos < 0 || pos / PACE_KV_BLOCK_TOKENS >= dest.table_stride) return;
     blk = dest.table[b * dest.table_stride + pos / PACE_KV_BLOCK_TOKENS];
     off = (int)(pos % PACE_KV_BLOCK_TOKENS);
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(256) void kv_append_f32_kernel(pace_kv_pool_t pool,
   int64_t blk;
   int off;
   if (PAGED) {
-    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + t;
+    const int64_t pos = (int64_t)dest.seq_lens[b] + dest.pos_offset + (dest.offset_dev ? *dest.offset_dev : 0) + t;
     if (pos < 0 || pos / PACE_KV_BLOCK_TOKENS >= dest.table_stride) return;
     blk = dest.table[b * dest.table_stride + pos / PACE_KV_BLOCK_TOKENS];
     off = (int)(pos % PACE_KV_BLOCK_TOKENS);
@@ -390,7 +391,7 @@ int launch_block_append(const char* who, const pace_kv_pool_t* pool, const void*
                         int32_t table_stride, const int32_t* seq_lens, int32_t pos_offset, const RopeDev* rope,
                         hipStream_t stream) {
   PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch / heads exceed grid limits", who);
-  const AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset};
+  const AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset, nullptr};
   const unsigned blocks_x = (unsigned)((n_tokens + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS + 1);
   dim3 grid(blocks_x, pool->num_kv_heads, batch);
   const uint16_t* kq = static_cast<const uint16_t*>(k_new);
@@ -438,7 +439,7 @@ static int run_append(const char* who, const pace_kv_pool_t* pool, const void* k
     PACE_HIP_CHECK(hipGetLastError());
     return PACE_KV_OK;
   }
-  if (paged && n_tokens >= 8)  // enough tokens per sequence to fill slabs: one workgroup per destination block
+  if (paged && n_tokens >= 8 && !dest.offset_dev)  // enough tokens per sequence to fill slabs: one workgroup per destination block
     return launch_block_append(who, pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest.table,
                                dest.table_stride, dest.seq_lens, dest.pos_offset, nullptr, s_early);
   const int64_t rows = (int64_t)batch * n_tokens * pool->num_kv_heads;
@@ -466,7 +467,7 @@ extern "C" int pace_kv_append(const pace_kv_pool_t* pool, const void* k_new, con
                               int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
                               const int64_t* slot_mapping, void* stream) {
   if (batch > 0 && n_tokens > 0) PACE_REQUIRE(slot_mapping != nullptr, "pace_kv_append: slot_mapping is NULL");
-  AppendDest dest = {slot_mapping, nullptr, nullptr, 0, 0};
+  AppendDest dest = {slot_mapping, nullptr, nullptr, 0, 0, nullptr};
   return run_append("pace_kv_append", pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest, false,
                     stream);
 }
@@ -478,8 +479,20 @@ extern "C" int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_ne
   if (batch > 0 && n_tokens > 0)
     PACE_REQUIRE(block_table != nullptr && seq_lens != nullptr && table_stride >= 1,
                  "pace_kv_append_paged: NULL block_table / seq_lens or bad table_stride");
-  AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset};
+  AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset, nullptr};
   return run_append("pace_kv_append_paged", pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest, true,
+                    stream);
+}
+
+extern "C" int pace_kv_append_paged_at(const pace_kv_pool_t* pool, const void* k_new, const void* v_new, int64_t stride_b,
+                                       int64_t stride_h, int64_t stride_t, int32_t batch, int32_t n_tokens,
+                                       const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens,
+                                       int32_t pos_offset, const int32_t* pos_offset_dev, void* stream) {
+  if (batch > 0 && n_tokens > 0)
+    PACE_REQUIRE(block_table != nullptr && seq_lens != nullptr && table_stride >= 1,
+                 "pace_kv_append_paged_at: NULL block_table / seq_lens or bad table_stride");
+  AppendDest dest = {nullptr, block_table, seq_lens, table_stride, pos_offset, pos_offset_dev};
+  return run_append("pace_kv_append_paged_at", pool, k_new, v_new, stride_b, stride_h, stride_t, batch, n_tokens, dest, true,
                     stream);
 }
 

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 12
+ABI_VERSION = 13
 STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
@@ -23,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "pace_kv_abi_version",
     "pace_kv_append",
     "pace_kv_append_paged",
+    "pace_kv_append_paged_at",
     "pace_kv_gather",
     "pace_kv_gather_packed",
     "pace_kv_copy_blocks",
@@ -174,6 +175,11 @@ def load() -> ctypes.CDLL:
     lib.pace_kv_append_paged.argtypes = [
         P, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
         c_void_p, c_int32, c_void_p, c_int32, c_void_p,
+    ]
+    lib.pace_kv_append_paged_at.restype = ctypes.c_int
+    lib.pace_kv_append_paged_at.argtypes = [
+        P, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
+        c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p,
     ]
     lib.pace_kv_gather.restype = ctypes.c_int
     lib.pace_kv_gather.argtypes = [

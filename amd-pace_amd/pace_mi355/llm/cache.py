@@ -154,6 +154,7 @@ class PagedKVCache(KVCacheBase):
         self._graph = None  # a DecodeGraph that has captured this cache's decode step
         self.cow_blocks_copied = 0  # blocks copied on write after forks (per layer pool)
         self.f32 = False  # the pool holds fp32 rows (set by the first update)
+        self._graph_appended = False  # fp32, inside a captured step: this step's append has been launched
         PACE_LLM_DEBUG(f"PagedKVCache initialized with max sequence length: {max_seq_length}")
 
     @property
@@ -295,12 +296,27 @@ class PagedKVCache(KVCacheBase):
         head_step = h_in // self.num_kv_heads  # de-duplicate a repeat_kv-expanded input
         st = self.state
         lib = nat.load()
-        if self._graph is not None and counts is None and self.fuse_append and T <= 32 and self._pending is None:
-            # a step of a decode graph: blocks and table were prepared for every step; the append rides in the
-            # attention launch, and the lengths advance on the device
-            self._graph.reserve(T)
-            self._pending = (k, v, head_step, rope)
-            self._query_rope = rope
+        if (self._graph is not None and counts is None and (self.fuse_append or self.f32) and T <= 32
+                and self._pending is None and not self._graph_appended):
+            # a step of a decode graph: blocks and table were prepared for every step, and the lengths advance on the
+            # device.  bf16: the append rides in the attention launch.  fp32: a launch of its own, its positions
+            # taken from the graph's frozen lengths plus the device counter.
+            graph = self._graph
+            graph.reserve(T)
+            if self.f32:
+                nat.check(
+                    lib.pace_kv_append_paged_at(
+                        ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
+                        B, T, graph.table.data_ptr(), graph.table.stride(0), graph.lens_dev.data_ptr(), 0,
+                        graph.counter.data_ptr(), nat.current_stream_ptr(),
+                    )
+                )
+                self._graph_appended = True
+                if not keep_query_rope:
+                    self._query_rope = None
+            else:
+                self._pending = (k, v, head_step, rope)
+                self._query_rope = rope
             self.lens = self.lens + T
             self.seq_len += T
             return
@@ -360,6 +376,7 @@ class PagedKVCache(KVCacheBase):
         comes through here first, which ends a decode graph (its frozen plan and lengths no longer hold)."""
         if self._graph is not None:
             self._graph.close()
+        self._graph_appended = False
         if self._pending is not None:
             k, v, head_step, rope = self._pending
             self._pending = None
@@ -531,9 +548,10 @@ class PagedKVCache(KVCacheBase):
         max_len = self.seq_len
         lib = nat.load()
         graph = self._graph
-        if graph is not None and self._pending is None:
+        if graph is not None and self._pending is None and not self._graph_appended:
             graph.close()  # attention without the step's append is not the captured step
             graph = None
+        self._graph_appended = False
         plan = lambda: st.plan_attention(self.lens, hq, self.num_kv_heads, self.head_dim, S, attention_mask is not None,
                                          self.partition_tokens)
         a = nat.PagedAttnArgs()
@@ -545,8 +563,13 @@ class PagedKVCache(KVCacheBase):
             if B * self.num_kv_heads * ((rows + 63) // 64 if rows > 32 else 1) < 512:
                 # a batch that does not fill the GPU: room for the library to cut every sequence over up to 64 workgroups
                 ws_bytes = min(B * hq * S * 64 * (D + 4) * 4, 64 << 20)
-            table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
-            a.seq_len_bias = bias
+            if graph is None:
+                table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
+                a.seq_len_bias = bias
+            else:  # captured step: frozen table and lengths, the device counter counts the tokens of the steps before
+                table, lens_dev = graph.table, graph.lens_dev
+                a.seq_len_bias, a.seq_len_bias_ptr = graph.new_tokens, graph.counter.data_ptr()
+                max_len = int(graph.base.max()) + graph.new_tokens * graph.max_steps
         elif graph is None:
             items, parts, n_items, max_parts, ws_bytes = plan()
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)

@@ -3,7 +3,8 @@
 The reference's generator runs one Python step per token (``pace/llm/generator.py:741-801``); at small batch
 the GPU work of a layer (tens of microseconds) is shorter than the interpreter's work to enqueue it.  Nothing
 in the library allocates, clears memory or synchronises, so the launches of a whole step -- every layer's
-fused append + attention -- can be captured once and replayed with one call.  What changes from step to step
+fused append + attention (fp32 pools: an append launch and an attention launch) -- can be captured once and
+replayed with one call.  What changes from step to step
 lives on the device: the caller's static q / k / v buffers, and a length counter that the graph itself advances
 (``seq_len_bias_ptr`` of the attention arguments).  Everything the host would otherwise upload per step is
 prepared before the capture: blocks for every future position, the block table, the work list.
@@ -31,8 +32,6 @@ class DecodeGraph:
                  stream: Optional[torch.cuda.Stream] = None):
         if not caches or any(c.pool is None for c in caches):
             raise RuntimeError("the caches must hold their prompt before a decode step can be captured")
-        if any(c.f32 for c in caches):
-            raise RuntimeError("a decode graph rides on the append fused into the attention launch: bf16 pools only")
         st = caches[0].state
         if any(c.state is not st for c in caches):
             raise RuntimeError("the layers of one decode graph share one block table")
@@ -79,7 +78,7 @@ class DecodeGraph:
 
     def _restore(self) -> None:
         for c, (lens, seq_len) in zip(self.caches, self._host):
-            c.lens, c.seq_len, c._pending = lens.copy(), seq_len, None
+            c.lens, c.seq_len, c._pending, c._graph_appended = lens.copy(), seq_len, None, False
 
     def reserve(self, new_tokens: int) -> None:
         """Called by the first ``update_cache`` of the eager run: blocks and table for every future position."""

@@ -113,6 +113,20 @@ int pace_kv_append_paged(const pace_kv_pool_t* pool, const void* k_new, const vo
                          const int32_t* seq_lens, int32_t pos_offset, void* stream);
 
 /*
+ * pace_kv_append_paged with one more offset that is read on the device: token (b,t) goes to position
+ * seq_lens[b] + pos_offset + *pos_offset_dev + t.  For a decode step captured in a HIP graph, whose
+ * lengths advance in a device counter (seq_len_bias_ptr of the attention arguments) while seq_lens and
+ * the block table stay as they were captured; the fused append of the attention launch (k_new) does
+ * the same for bf16 pools in one launch.  pos_offset_dev == NULL: pace_kv_append_paged.
+ */
+int pace_kv_append_paged_at(const pace_kv_pool_t* pool, const void* k_new, const void* v_new,
+                            int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                            int32_t batch, int32_t n_tokens,
+                            const int32_t* block_table, int32_t table_stride,
+                            const int32_t* seq_lens, int32_t pos_offset,
+                            const int32_t* pos_offset_dev, void* stream);
+
+/*
  * Gather: block-table walk back into the reference's dense layout.
  * Produces what the reference cache holds (pace/llm/cache.py:391-399 after
  * repeat_kv, pace/llm/models/llama.py:151-158): k_out / v_out are bf16

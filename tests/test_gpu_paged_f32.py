@@ -373,10 +373,6 @@ def test_entry_points_that_fold_steps_in_refuse_an_fp32_pool(device):
                                     k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), 2, 1, table.data_ptr(), table.stride(0),
                                     lens_dev.data_ptr(), bias, stream)
     assert rc != 0 and "bf16 pools only" in lib.pace_kv_last_error().decode()
-    with pytest.raises(RuntimeError, match="bf16 pools only"):
-        from pace_mi355.llm.graph import DecodeGraph
-
-        DecodeGraph([cache], lambda: None, 4)
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -461,3 +457,74 @@ def test_manager_with_fp32_layers_and_beam_reorder(device):
         assert_bits_equal(mgr[layer].key.dense(), rk, f"layer {layer} K")
         assert_bits_equal(mgr[layer].value.dense(), rv, f"layer {layer} V")
     assert mgr[0].state is mgr[1].state and mgr[0].pool.dtype == F32
+
+
+def test_decode_step_captured_into_a_graph(device):
+    """``KVCacheManager.capture_decode`` with fp32 layers: per layer an append launch (positions from the graph's
+    frozen lengths plus its device counter) and an attention launch, captured once, replayed per token."""
+    from pace_mi355.llm import KVCacheManager, KVCacheType
+    from pace_mi355.ops import MultiHeadAttention
+
+    class Cfg:
+        num_hidden_layers = 2
+        num_attention_heads = 8
+        num_key_value_heads = 2
+
+    B, hkv, n_rep, D, steps = 3, 2, 4, 128, 40
+    lens0 = [300, 17, 1200]
+    mgr = KVCacheManager(Cfg(), 2048, KVCacheType.PAGED)
+    models = [RaggedCacheModel(B, hkv, D, dtype=F32) for _ in range(2)]
+    for layer in range(2):
+        k, v = seeded_kv(10 + layer, B, hkv, max(lens0), D, dtype=F32)
+        mgr[layer].append_ragged(k.to(device), v.to(device), lens0)
+        models[layer].append(k, v, lens0)
+    mha = MultiHeadAttention(dtype=F32)
+    qs = [torch.zeros(B, hkv * n_rep, 1, D, device=device) for _ in range(2)]
+    ks = [torch.zeros(B, hkv, 1, D, device=device) for _ in range(2)]
+    vs = [torch.zeros(B, hkv, 1, D, device=device) for _ in range(2)]
+
+    def step():
+        outs = []
+        for layer in range(2):
+            pk, pv = mgr[layer].update_cache(ks[layer], vs[layer], 2)
+            outs.append(mha(qs[layer], pk, pv))
+        return outs
+
+    graph = mgr.capture_decode(step, max_steps=steps)
+    assert len(mgr) == max(lens0), "capturing leaves the cache as it was"
+    for i in range(steps):
+        new = []
+        for layer in range(2):
+            kn, vn = seeded_kv(1000 + 2 * i + layer, B, hkv, 1, D, dtype=F32)
+            qn = seeded_q(2000 + 2 * i + layer, B, hkv * n_rep, 1, D, dtype=F32)
+            ks[layer].copy_(kn), vs[layer].copy_(vn), qs[layer].copy_(qn)
+            models[layer].append(kn, vn)
+            new.append(qn)
+        outs = graph.replay()
+        assert len(mgr) == max(lens0) + i + 1
+        if i % 7 == 0 or i == steps - 1:
+            for layer in range(2):
+                _close(outs[layer], models[layer].attention(new[layer], n_rep), f"replay {i} layer {layer}")
+    with pytest.raises(RuntimeError, match="reserved blocks for"):
+        graph.replay()
+    for layer in range(2):
+        K, V = models[layer].dense(1)
+        gk, gv = mgr[layer].gather(n_rep=1)
+        assert_bits_equal(gk, K, f"pool K of layer {layer}")
+        assert_bits_equal(gv, V, f"pool V of layer {layer}")
+    # a second graph, ended early by a rollback; step-by-step operation carries on from there
+    graph = mgr.capture_decode(step, max_steps=8)
+    for layer in range(2):
+        kn, vn = seeded_kv(5000 + layer, B, hkv, 1, D, dtype=F32)
+        ks[layer].copy_(kn), vs[layer].copy_(vn)
+        models[layer].append(kn, vn)
+    graph.replay()
+    mgr.remove_cache(1)
+    for m in models:
+        m.truncate([1] * B)
+    with pytest.raises(RuntimeError, match="spent"):
+        graph.replay()
+    outs = step()
+    for layer in range(2):
+        models[layer].append(ks[layer].cpu(), vs[layer].cpu())
+        _close(outs[layer], models[layer].attention(qs[layer].cpu(), n_rep), f"eager step after the graph, layer {layer}")
