@@ -44,6 +44,16 @@ __device__ __forceinline__ f32x4 load4_f32(const uint16_t* p) {
   return f32x4{bf16_bits_to_f32(w[0] & 0xffffu), __uint_as_float(w[0] & 0xffff0000u), bf16_bits_to_f32(w[1] & 0xffffu),
                __uint_as_float(w[1] & 0xffff0000u)};
 }
+// Four elements of a K / V row.  ONCE: the row is read by one row group and nobody after it (few query rows: decode);
+// fetched non-temporally, which lifts a stream on this GPU from 6.0 - 6.25 to 7.0 - 7.25 TB/s -- provided every
+// cache line is consumed by few instructions (past the L1 each instruction fetches its lines again; see ONCE below).
+template <bool ONCE>
+__device__ __forceinline__ f32x4 load4_kv(const float* p) {
+  if constexpr (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+  else return load4_f32(p);
+}
+template <bool ONCE>
+__device__ __forceinline__ f32x4 load4_kv(const uint16_t* p) { return load4_f32(p); }
 // Two consecutive elements (p 8- resp. 4-byte aligned).
 __device__ __forceinline__ f32x2 load2_f32(const float* p) { return *reinterpret_cast<const f32x2*>(p); }
 __device__ __forceinline__ f32x2 load2_f32(const uint16_t* p) {
@@ -157,13 +167,21 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   }
   // This lane's dims of a row for the first product: d0 .. d0 + KS - 1.
   const int d0 = g * KS;
-  auto load_run = [&](const T* r, float (&x)[KS]) {
+  // Launches whose K / V are read by one row group (the dense kernel's key-splitting variants, the pool's small-row
+  // launches): non-temporal loads, and the first product's dims dealt out so that the four lanes of a row read 64
+  // contiguous bytes per load -- a 128-byte line is then consumed by two instructions instead of eight (fetched
+  // non-temporally with a lane's dims as one run, the fp32 pool's decode launch took 638 us instead of 370; with both
+  // changes 357, the dense op's fp32 decode 1.29 ms instead of 1.39).  Any assignment of dims to steps gives the same
+  // sum as long as Q and K share it.
+  constexpr bool ONCE = AHEAD || (PAGED && !COOP);
+  auto load_run = [&](const T* r, float (&x)[KS], auto once_c) {
+    constexpr bool kOnce = decltype(once_c)::value;
 #pragma unroll
     for (int s4 = 0; s4 < KS; s4 += 4) {
-      const int d = d0 + s4;
+      const int d = ONCE ? 4 * s4 + 4 * g : d0 + s4;
       if (VEC) {  // H is a multiple of 4: the four dims exist together or not at all
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
-        if (d + 4 <= H) t = load4_f32(r + d);
+        if (d + 4 <= H) t = load4_kv<kOnce>(r + d);
         x[s4] = t[0], x[s4 + 1] = t[1], x[s4 + 2] = t[2], x[s4 + 3] = t[3];
       } else {
 #pragma unroll
@@ -172,7 +190,7 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
     }
   };
   float qf[KS];
-  load_run(qrow, qf);
+  load_run(qrow, qf, std::false_type{});
   if (!valid) {
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = 0.f;
@@ -231,7 +249,7 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
       kblock = kbase + blk * p.k_bs - (int64_t)t0 * H, vblock = vbase + blk * p.v_bs - (int64_t)t0 * H;
     }
     // rows past the end are masked below (PAGED: the block's 16 rows exist whatever the length is)
-    load_run(kblock + (int64_t)(PAGED ? t0 + n : min(L - 1, t0 + n)) * H, kx);
+    load_run(kblock + (int64_t)(PAGED ? t0 + n : min(L - 1, t0 + n)) * H, kx, std::integral_constant<bool, ONCE>{});
     // V: output tile j of lane n stands for dim v_dim(j, n) = 16 VG (j / VG) + VG n + j % VG, so that the VG values a
     // lane needs of one token for VG neighbouring tiles are one contiguous run: a quarter of the load instructions
     // that one value per load takes, and every load of a wave covers whole 256-byte stretches of four rows.
@@ -243,7 +261,7 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
         const int d = 16 * jj + VG * n;
         if (VEC && VG == 4) {
           f32x4 t = {0.f, 0.f, 0.f, 0.f};
-          if (d + 4 <= H) t = load4_f32(vr + d);
+          if (d + 4 <= H) t = load4_kv<ONCE>(vr + d);
 #pragma unroll
           for (int e = 0; e < 4; ++e) vx[jj + (e % VG)][i] = t[e];
         } else if (VEC && VG == 2) {
