@@ -511,8 +511,9 @@ static int run_gather(const char* who, const pace_kv_pool_t* pool, const int32_t
                "%s: output strides must be multiples of %d elements and hold a row of head_dim", who, per16);
   const int n_blocks = (rows + PACE_KV_BLOCK_TOKENS - 1) / PACE_KV_BLOCK_TOKENS;
   PACE_REQUIRE(table_stride >= 1, "%s: table_stride %d", who, table_stride);
-  PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch/heads exceed grid limits", who);
-  dim3 grid(n_blocks, pool->num_kv_heads, batch);
+  // the dense form puts heads and sequences on the grid's y and z axes; the packed form's grid is one-dimensional
+  if (!packed) PACE_REQUIRE(batch <= 65535 && pool->num_kv_heads <= 65535, "%s: batch/heads exceed grid limits", who);
+  dim3 grid(n_blocks, packed ? 1 : pool->num_kv_heads, packed ? 1 : batch);
   if (packed) {
     const int64_t entries = ((int64_t)out.total_rows / PACE_KV_BLOCK_TOKENS + batch) * pool->num_kv_heads;
     PACE_REQUIRE(entries < ((int64_t)1 << 31), "%s: grid too large", who);

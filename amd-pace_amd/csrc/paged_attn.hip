@@ -1046,12 +1046,16 @@ static int static_scratch(const char* who, void** out) {
   int dev = 0;
   PACE_HIP_CHECK(hipGetDevice(&dev));
   PACE_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device ordinal %d out of range", who, dev);
+  if (void* known = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE)) {  // every call after the first
+    *out = known;
+    return PACE_KV_OK;
+  }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
     void* ptr = nullptr;
     PACE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     PACE_REQUIRE(ptr != nullptr, "%s: the scratch array has no device address", who);
-    g_scratch_ptr[dev] = ptr;
+    __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
   }
   *out = g_scratch_ptr[dev];
   return PACE_KV_OK;
@@ -1061,10 +1065,13 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
                           bool use_static_scratch = false) {
   PACE_REQUIRE(a_in != nullptr, "%s: args is NULL", who);
   pace_paged_attn_args_t a_copy = *a_in;
+  // The array's address is looked up on the first attention call of any entry point on a device, not on the first
+  // call of the entry point that uses it: a caller that captures pace_paged_attn_verify_static into a graph has run
+  // a step eagerly before (any entry point will do), so the look-up never falls inside a capture.
   if (use_static_scratch) {
-    void* ptr = nullptr;
-    if (int rc = static_scratch(who, &ptr)) return rc;
-    a_copy.workspace = ptr;
+    void* static_ptr = nullptr;
+    if (int rc = static_scratch(who, &static_ptr)) return rc;
+    a_copy.workspace = static_ptr;
     a_copy.workspace_bytes = kStaticScratchBytes;
   }
   const pace_paged_attn_args_t* a = &a_copy;
@@ -1130,6 +1137,10 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     PACE_REQUIRE(a->mask == nullptr, "%s: rope in the attention launch cannot be combined with an explicit mask", who);
     PACE_REQUIRE(!a->k_new || a->n_new == a->q_len, "%s: with rope, the fused append takes n_new == q_len (got %d, %d)", who,
                  a->n_new, a->q_len);
+  }
+  if (!g_name_out && !use_static_scratch) {  // (the arguments are in order: this call will launch)
+    void* unused = nullptr;
+    (void)static_scratch(who, &unused);  // a failure here only matters to the entry point that uses the array
   }
   const int n_rep = a->num_q_heads / pool->num_kv_heads;
   const int rows = a->q_len * n_rep;

@@ -375,6 +375,11 @@ class PagedKVCache(KVCacheBase):
         """Store a held-back append into the pool now.  Every operation other than a captured decode step
         comes through here first, which ends a decode graph (its frozen plan and lengths no longer hold)."""
         if self._graph is not None:
+            if self._graph._capturing:
+                # anything that comes through here uploads host data or allocates blocks: recorded into a graph it
+                # would replay stale values
+                raise RuntimeError("the captured step differs from its eager run: a cache operation other than the "
+                                   "step's one update_cache + attention per layer ran during the capture")
             self._graph.close()
         self._graph_appended = False
         if self._pending is not None:
@@ -549,6 +554,8 @@ class PagedKVCache(KVCacheBase):
         lib = nat.load()
         graph = self._graph
         if graph is not None and self._pending is None and not self._graph_appended:
+            if graph._capturing:
+                raise RuntimeError("the captured step differs from its eager run: attention without the step's append")
             graph.close()  # attention without the step's append is not the captured step
             graph = None
         self._graph_appended = False

@@ -59,6 +59,9 @@ class DecodeGraph:
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 step_fn()                      # eager run: loads kernels, makes the plans, sizes the workspace
+                if self.closed or not self._reserved:
+                    raise RuntimeError("this step cannot be captured: it must be, for every layer, one update_cache of 1..32 "
+                                       "tokens followed by the attention call, and nothing else on the caches")
                 self._restore()
                 self.counter.zero_()
                 side.synchronize()
@@ -71,7 +74,10 @@ class DecodeGraph:
                 self._restore()
             torch.cuda.current_stream().wait_stream(side)
         except Exception:
+            # a refused capture leaves the caches as they were: whatever the failed step appended is forgotten
+            self._capturing = False
             self.close()
+            self._restore()
             raise
 
     _capturing = False

@@ -85,153 +85,7 @@ def append_bytes(batch, new_tokens, kv_heads, head_dim):
     return 2 * batch * new_tokens * kv_token_bytes(kv_heads, head_dim) + 4 * batch * new_tokens
 
 
-def _randn_bf16(torch, shape, gen, dev):
-    return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
-
-
-def alloc_free_history(alloc, seed, lo_blocks, hi_blocks, occupancy=0.75, turnover=4.0):
-    """Leave the free list in the order a serving history leaves it in: sequences of lo..hi blocks (log-uniform)
-    are admitted while the pool is below `occupancy` and retired at random, until `turnover` times the pool has
-    been handed out; then the survivors retire in random order.  Seeded."""
-    import numpy as np
-
-    rng = np.random.default_rng(seed)
-    live, handed = [], 0
-    while handed < turnover * alloc.num_blocks:
-        used = alloc.num_blocks - alloc.num_free
-        n = int(round(math.exp(rng.uniform(math.log(lo_blocks), math.log(hi_blocks)))))
-        if used + n <= occupancy * alloc.num_blocks and (not live or rng.random() < 0.7):
-            live.append(alloc.allocate(n))
-            handed += n
-        elif live:
-            alloc.free(live.pop(int(rng.integers(len(live)))))
-    for i in rng.permutation(len(live))[::-1]:
-        alloc.free(live[i])
-
-
-def build_cache(torch, dev, lens, q_heads, kv_heads, head_dim, seed, pool_factor=None, headroom=64, permute=True,
-                history=False, f32=False):
-    """Paged cache holding lens[b] tokens per sequence, physical blocks in a seeded random order (a shuffle of
-    the free list) or, with `history`, in the order a seeded admit / retire history of sequences leaves behind."""
-    import numpy as np
-    from pace_mi355.llm import PagedKVCache
-
-    B, T = len(lens), max(lens)
-    live = sum((n + headroom + 15) // 16 for n in lens)
-    num_blocks = int(pool_factor * live) if pool_factor else live
-    cache = PagedKVCache(T + headroom, num_kv_heads=kv_heads, n_rep=q_heads // kv_heads, num_blocks=num_blocks)
-    g = torch.Generator(device=dev).manual_seed(seed)
-    lens_np = np.asarray(lens)
-    chunk = 1024
-    for t0 in range(0, T, chunk):
-        n = min(chunk, T - t0)
-        k = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
-        v = _randn_bf16(torch, (B, kv_heads, n, head_dim), g, dev)
-        if f32:  # a pool of fp32 rows
-            k, v = k.float(), v.float()
-        if t0 == 0:
-            cache.append_ragged(k[:, :, :1], v[:, :, :1], [0] * B)  # creates the pool and the free list
-            alloc = cache.state.allocator
-            if history:
-                alloc_free_history(alloc, seed, 8, 1024)
-                cache.append_ragged(k, v, np.clip(lens_np - t0, 0, n))
-                continue
-            ids = alloc.allocate(alloc.num_free)
-            if permute:
-                np.random.default_rng(seed).shuffle(ids)  # consecutive logical blocks end up far apart in HBM
-            else:
-                ids = ids[::-1]
-            alloc.free(ids)
-        cache.append_ragged(k, v, np.clip(lens_np - t0, 0, n))
-    return cache
-
-
-class FixedStep:
-    """Direct C-ABI calls with metadata frozen at "T new tokens on top of the prefilled cache":
-    the new tokens land on the same positions every step, so each step moves the same bytes."""
-
-    def __init__(self, torch, cache, q, k_new, v_new, partition=0, fused=True, rope=None, mask=None):
-        import numpy as np
-        from pace_mi355 import _native as nat
-
-        self.nat, self.lib = nat, nat.load()
-        dev = q.device
-        B, hq, S, D = q.shape
-        T = k_new.shape[2]
-        self.cache, self.k, self.v, self.T, self.B = cache, k_new, v_new, T, B
-        lens_after = cache.lens + T
-        cache.state.ensure_capacity(lens_after)
-        self.table = cache.state.device_table()
-        self.lens_dev = torch.from_numpy(lens_after.astype(np.int32)).to(dev)
-        self.lens_after = lens_after
-        self.out = torch.empty(B, hq, S, D, dtype=q.dtype, device=dev)
-        max_len = int(lens_after.max())
-        a = nat.PagedAttnArgs()
-        a.q, a.q_stride_b, a.q_stride_h, a.q_stride_s = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
-        a.out, a.o_stride_b, a.o_stride_h, a.o_stride_s = (self.out.data_ptr(), self.out.stride(0), self.out.stride(1),
-                                                           self.out.stride(2))
-        a.block_table, a.table_stride, a.seq_lens = self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr()
-        a.kv_start, a.mask, a.causal = None, None, 1
-        if mask is not None:  # additive bf16 [B,1,S,L]: the mask alone decides what a row reads
-            self.mask = mask
-            a.mask, a.mask_dtype, a.mask_len, a.causal = mask.data_ptr(), nat.DTYPE_BF16, mask.shape[3], 0
-            a.mask_stride_b, a.mask_stride_s = mask.stride(0), mask.stride(2)
-        a.batch, a.num_q_heads, a.q_len = B, hq, S
-        # the library's planner cuts the batch: descriptors of (sequence, partition) work items in scheduling order
-        a.max_seq_len, a.partition_tokens, a.scale = max_len, 0, 1.0 / math.sqrt(D)
-        if cache.f32:  # rows of fp32: one launch over the block table, no work list; the workspace lets a small batch be cut
-            n_items = max_parts = 0
-            ws_bytes = min(B * hq * S * 64 * (D + 4) * 4, 64 << 20)
-        else:
-            self.items, self.parts, n_items, max_parts, ws_bytes = cache.state.plan_attention(
-                lens_after, hq, cache.num_kv_heads, cache.head_dim, S, mask is not None, partition)
-            a.work_items, a.n_work_items = self.items.data_ptr(), n_items
-            a.seq_parts, a.max_parts = self.parts.data_ptr(), max_parts
-        self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-        a.workspace, a.workspace_bytes = self.ws.data_ptr(), ws_bytes
-        self.n_items, self.max_parts = n_items, max_parts
-        self.fused = fused
-        if fused:  # the attention launch reads the new tokens from k_new / v_new and stores them into the pool
-            a.k_new, a.v_new, a.n_new = k_new.data_ptr(), v_new.data_ptr(), T
-            a.new_stride_b, a.new_stride_h, a.new_stride_t = k_new.stride(0), k_new.stride(1), k_new.stride(2)
-        # rope (a pace_rope_t with positions == NULL: rows follow the sequence positions): folded into the
-        # attention launch when the append is, else into the append launch, which then also rotates q
-        self.rope, self.q_rot = rope, None
-        if rope is not None and fused:
-            a.rope = ctypes.pointer(rope)
-        elif rope is not None:
-            self.q_rot = torch.empty_like(q)
-            a.q = self.q_rot.data_ptr()
-        self.args, self.q = a, q
-        self.attn = self.lib.pace_paged_attn_decode if S == 1 else self.lib.pace_paged_attn_verify
-        self.stream = nat.current_stream_ptr()
-        self.kernel = nat.kernel_name(cache._desc, a)  # the instantiation these arguments launch
-
-    def append(self):
-        k, v = self.k, self.v
-        if self.rope is not None:
-            q, qo = self.q, self.q_rot
-            self.nat.check(self.lib.pace_rope_append_paged(
-                ctypes.byref(self.cache._desc), ctypes.byref(self.rope), q.data_ptr(), qo.data_ptr(), q.stride(0), q.stride(1),
-                q.stride(2), q.shape[1], k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2), self.B, self.T,
-                self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr(), -self.T, self.stream))
-            return
-        self.nat.check(self.lib.pace_kv_append_paged(
-            ctypes.byref(self.cache._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2), self.B, self.T,
-            self.table.data_ptr(), self.table.stride(0), self.lens_dev.data_ptr(), -self.T, self.stream))
-
-    def attend(self):
-        self.nat.check(self.attn(ctypes.byref(self.cache._desc), ctypes.byref(self.args), self.stream))
-        return self.out
-
-    def __call__(self, ev=None):
-        if not self.fused:
-            self.append()
-        if ev:
-            ev[0].record()
-        self.attend()
-        if ev:
-            ev[1].record()
+from pace_mi355.utils.fixed_step import FixedStep, build_cache, randn_bf16 as _randn_bf16  # noqa: E402
 
 
 EVENT_EVERY = 8  # an event record costs several microseconds of GPU timeline; bracket one launch in eight
@@ -301,6 +155,55 @@ def result_line(args, workload, step_bytes, tokens_per_step, dt, roof, extra_cfg
     if extra:
         line.update(extra)
     return line
+
+
+CHECK_NOTE = ("last timed step vs the fp32 CPU oracle (caps 2e-2 max abs / 1e-2 relative per sequence); slots of the new "
+              "tokens bit-exact for every sequence")
+
+
+def check_attention(torch, q, out, gk, gv, lens, rows):
+    """Output rows of the sampled sequences `rows` against the fp32 oracle (the restated reference attention on the
+    CPU) over the dense K / V `gk`, `gv` [B, Hkv, L, D] gathered back from the pool.  Caps: max abs error 2e-2,
+    relative error (per sequence, Euclidean norm) 1e-2."""
+    from oracle.attention_ref import lengths_mask_4d, sdpa_fp32
+    from oracle.cache_ref import repeat_kv
+
+    S, n_rep = q.shape[2], q.shape[1] // gk.shape[1]
+    idx = torch.tensor(rows, device=gk.device)
+    ls = [int(lens[r]) for r in rows]
+    L = max(ls)
+    got = out[idx].float().cpu()
+    ref = sdpa_fp32(q[idx].cpu(), repeat_kv(gk[idx][:, :, :L].cpu(), n_rep), repeat_kv(gv[idx][:, :, :L].cpu(), n_rep),
+                    lengths_mask_4d(ls, S, L, torch.float32))
+    err = (got - ref).abs()
+    rel = float((err.flatten(1).norm(dim=1) / ref.flatten(1).norm(dim=1)).max())
+    max_abs = float(err.max())
+    ok = bool(max_abs <= 2e-2 and rel <= 1e-2 and not torch.isnan(got).any())
+    return {"checked": ok, "max_abs_err": round(max_abs, 6), "max_rel_err": round(rel, 6), "checked_sequences": [int(r) for r in rows]}
+
+
+def self_check(torch, step, rows):
+    """After the timed region: the last step's output for the sampled sequences against the oracle, and the slots
+    the step's new tokens were stored in against the tokens themselves, bit for bit, for every sequence."""
+    torch.cuda.synchronize()
+    gk, gv = step.gathered()
+    T = step.T
+    slots_ok = True
+    for b, n in enumerate(step.lens_after.tolist()):
+        slots_ok = slots_ok and torch.equal(gk[b, :, n - T:n], step.k[b]) and torch.equal(gv[b, :, n - T:n], step.v[b])
+    res = check_attention(torch, step.q, step.out, gk, gv, step.lens_after, rows)
+    res["appended_slots_bit_exact"] = bool(slots_ok)
+    res["checked"] = bool(res["checked"] and slots_ok)
+    res["check"] = CHECK_NOTE
+    return res
+
+
+def spread_rows(lens):
+    """Sequences to sample: the shortest, the median, the longest and the last of the batch."""
+    import numpy as np
+
+    order = np.argsort(np.asarray(lens), kind="stable")
+    return sorted({int(order[0]), int(order[len(order) // 2]), int(order[-1]), len(lens) - 1})
 
 
 # ---- workloads ---------------------------------------------------------------------------------
@@ -408,12 +311,15 @@ def _wl_decode(torch, dev, args, shape, label, has_traffic_profile, with_cpu):
     launch_bytes = dec + (append_bytes(B, 1, hkv, D) if fused else 0)
     kernel = fixed[0].kernel if args.path == "direct" else "pace_kv::paged_attn_kernel (through PagedKVCache / MultiHeadAttention)"
     traffic = measured_traffic(kernel) if has_traffic_profile else None
+    check = None
+    if args.path == "direct" and not args.rope and not args.no_check:
+        check = self_check(torch, fixed[(turn[0] - 1) % n_layers], spread_rows([ctx] * B))
     line = result_line(
         args, label, dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline(kernel + (" (decode, append fused in)" if fused else " (decode)"), launch_bytes, attn_ms, {"traffic": traffic}),
         {"path": args.path, "append_fused": fused, "rope": bool(args.rope and args.path == "direct"),
          "mask": bool(args.mask and args.path == "api"), "layers": n_layers,
-         "distinct_pool_bytes": int(n_layers * B * ctx * kv_token_bytes(hkv, D))})
+         "distinct_pool_bytes": int(n_layers * B * ctx * kv_token_bytes(hkv, D))}, extra=check)
     if with_cpu and not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, B, ctx, hq, hkv, D)
     return line
@@ -441,12 +347,13 @@ def wl_ragged(torch, dev, args):
         fn = gather_call(torch, cache, form)
         forms[form] = roofline(f"kv_gather_kernel<128,{'true' if form == 'packed' else 'false'}> ({form.replace('_', ' ')})", gather_b,
                                time_call(torch, fn, reps=5, warmup=1))
+    check = {} if args.no_check else self_check(torch, step, spread_rows(lens1))
     return result_line(
         args, f"ragged serving mix: batch 256, contexts log-uniform [128,16384] (seed 2, {sum(lens)} live tokens), pool 1.3x "
         "with the free list left by a seeded admit / retire history (seed 3), "
         "1-token append + GQA decode", dec + append_bytes(B, 1, hkv, D), B, dt,
         roofline(step.kernel + " (decode, ragged) + merge", dec, attn_ms, {"work_items": step.n_items, "max_parts": step.max_parts}),
-        extra={"gather": forms})
+        extra=dict(check, gather=forms))
 
 
 def gather_call(torch, cache, form):
@@ -535,11 +442,13 @@ def wl_verify(torch, dev, args):
     lens_v = [n + S for n in lens]
     dec = decode_bytes(lens_v, hq, hkv, D, q_len=S)
     flops = 4.0 * sum(lens_v) * hq * S * D
+    check = {} if args.no_check else self_check(torch, step, spread_rows(lens_v))
     return result_line(
         args, "PARD speculative verify: batch 32, contexts U[1024,8192] (seed 4), 8 draft tokens appended + causal "
         "8-query attention", dec + append_bytes(B, S, hkv, D), B * S, dt,
         roofline(step.kernel + " (verify) + merge", dec, attn_ms,
-                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2), "work_items": step.n_items, "max_parts": step.max_parts}))
+                 {"mfma_tflops": round(flops / (attn_ms * 1e-3) / 1e12, 2), "work_items": step.n_items, "max_parts": step.max_parts}),
+        extra=check)
 
 
 def wl_prefill(torch, dev, args):
@@ -699,13 +608,22 @@ def wl_compact(torch, dev, args):
     lens = cache.lens.tolist()
     dec = decode_bytes(lens, hq, hkv, D)
     attn_ms = time_call(torch, lambda: cache.attend(q), reps=args.steps, warmup=args.warmup)
+    check = {}
+    if not args.no_check:  # decode over the compacted cache against the oracle over the surviving tokens, gathered back
+        gk, gv = cache.gather(n_rep=1)
+        check = check_attention(torch, q, cache.attend(q), gk, gv, lens, [0, B - 1])
+        used = np.concatenate([cache.state.table[b, : cache.state.n_blocks[b]] for b in range(B)])
+        check["blocks_contiguous"] = bool(sorted(used.tolist()) == list(range(len(used))))
+        check["checked"] = bool(check["checked"] and check["blocks_contiguous"])
+        check["check"] = "decode after compaction vs the fp32 CPU oracle over the surviving tokens; live blocks occupy ids 0..n-1"
     return result_line(
         args, f"long-context compaction: 70B-shape KV (64 Q / 8 KV heads), batch 8, context 32768, 40% of blocks evicted "
         f"(seed 6), {moved} blocks moved, then decode over {lens[0]} tokens/seq", dec, B, attn_ms * 1e-3,
         roofline("paged_attn_kernel<128,1,...> (decode after compaction) + merge", dec, attn_ms),
         extra={"compaction": roofline("kv_copy_blocks_kernel", 2 * moved * block_bytes, compact_ms,
                                       {"blocks_moved": moved, "end_to_end_ms": round(host_ms, 3),
-                                       "end_to_end_note": "plan + upload + copy + table rewrite, wall clock between two synchronizes"})})
+                                       "end_to_end_note": "plan + upload + copy + table rewrite, wall clock between two synchronizes"}),
+               **check})
 
 
 def wl_copy_calibration(torch, dev, args):
@@ -783,6 +701,31 @@ def cpu_baseline(torch, batch, ctx, hq, hkv, D, warmup=2, timed=5):
     }
 
 
+def other_configs(torch, dev, args):
+    """Short legs over the other benchmark configurations (the ragged serving mix, the speculative verify step, the
+    long-context compaction), at most 20 timed steps each, so that one default run carries every configuration's
+    roofline figure.  `value` of the line stays the headline workload's."""
+    import copy
+    import gc
+
+    out = {}
+    for name in ("ragged", "verify", "compact"):
+        a = copy.copy(args)
+        a.steps, a.warmup, a.workload = min(args.steps, 20), min(args.warmup, 5), name
+        gc.collect()
+        torch.cuda.empty_cache()
+        res = WORKLOADS[name](torch, dev, a)
+        keep = {k: res[k] for k in ("value", "unit", "pct_of_hbm_peak", "tokens_per_s", "steps", "warmup", "ms_per_step", "roofline",
+                                    "checked", "max_abs_err", "max_rel_err", "appended_slots_bit_exact", "checked_sequences",
+                                    "gather", "compaction", "blocks_contiguous") if k in res}
+        keep["workload"] = res["config"]["workload"]
+        keep["bytes_per_step"] = res["config"]["bytes_per_step"]
+        out[name] = keep
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
 WORKLOADS = {"gather": wl_gather, "append": wl_append, "decode-8b": wl_decode_8b, "decode-gptj": wl_decode_gptj, "ragged": wl_ragged, "verify": wl_verify, "prefill": wl_prefill, "dense-f32": wl_dense_f32, "decode-f32pool": wl_decode_f32pool,
              "dense-prefill": wl_dense_prefill, "compact": wl_compact, "copy-calibration": wl_copy_calibration}
 
@@ -806,6 +749,10 @@ def main() -> int:
                          "4 x 1.07 GB is 16 times the last-level cache, 1 re-reads one pool every step")
     ap.add_argument("--partition", type=int, default=0, help="context split size in tokens (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true", dest="no_check",
+                    help="skip the comparison of the last step's results with the CPU oracle after the timed region")
+    ap.add_argument("--no-others", action="store_true", dest="no_others",
+                    help="default workload only: skip the short legs over the other configurations (ragged, verify, compact)")
     ap.add_argument("--mask", action="store_true",
                     help="decode-8b, api path: pass repeat_kv-expanded K/V and the step's additive mask, as the reference's "
                          "models call the cache and the attention operator; prefill: pass the causal mask as a tensor")
@@ -827,7 +774,12 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    print(json.dumps(WORKLOADS[args.workload](torch, dev, args)))
+    line = WORKLOADS[args.workload](torch, dev, args)
+    plain_default = (args.workload == "decode-8b" and args.path == "direct" and not (args.batch or args.context or args.rope or args.mask
+                                                                                    or args.no_fuse or args.no_permute or args.partition))
+    if plain_default and not args.no_others:
+        line["others"] = other_configs(torch, dev, args)
+    print(json.dumps(line))
     return 0
 
 

@@ -409,6 +409,9 @@ int pace_paged_attn_verify(const pace_kv_pool_t* pool, const pace_paged_attn_arg
  * allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that may overlap there
  * (different streams, different threads) race; order them on one stream.  Nothing in the array needs
  * clearing between calls: every partial a launch reads, it has written.
+ * Under graph capture: the array's address is looked up once per device, on the first attention call of any
+ * entry point there (pace_paged_attn_decode / _verify / _verify_static).  Run one attention step eagerly on the
+ * device before capturing -- the warm-up step every capture needs anyway -- so that the look-up is not recorded.
  */
 #define PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES (32u << 20)
 int pace_paged_attn_verify_static(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* args, void* stream);

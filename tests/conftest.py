@@ -35,3 +35,22 @@ def _announce(request):
         sys.stdout.write(f"\n[gpu-case] {request.node.nodeid}\n")
         sys.stdout.flush()
     yield
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The observed attention errors of this run, worst comparison per test (the caps are in helpers.py)."""
+    try:
+        import helpers
+    except ImportError:
+        return
+    if not helpers.OBSERVED:
+        return
+    worst = {}
+    for test, what, max_abs, rel, numel in helpers.OBSERVED:
+        w = worst.setdefault(test, [0.0, 0.0, 0])
+        w[0], w[1], w[2] = max(w[0], max_abs), max(w[1], rel), w[2] + 1
+    tr = terminalreporter
+    tr.write_sep("-", f"observed attention error vs the fp32 oracle (caps: max abs {helpers.ATTN_MAX_ABS}, relative {helpers.ATTN_MAX_REL})")
+    for test, (a, r, n) in sorted(worst.items()):
+        tr.write_line(f"{a:.3e}  {r:.3e}  {n:4d} comparisons  {test}")
+    tr.write_line(f"overall: max abs {max(w[0] for w in worst.values()):.3e}, relative {max(w[1] for w in worst.values()):.3e}")

@@ -24,7 +24,7 @@ def _scramble(cache, k1, v1, seed, history=False):
     cache.append_ragged(k1, v1, [0] * k1.shape[0])
     alloc = cache.state.allocator
     if history:
-        from bench import alloc_free_history
+        from pace_mi355.utils.history import alloc_free_history
 
         alloc_free_history(alloc, seed, 8, 1024)
         return
@@ -235,3 +235,80 @@ def test_cfg5_evict_compact_decode_70b_shape(device):
     assert torch.equal(before, after)
     rows = [0, 7]
     assert_attention_close(after[rows], _oracle_rows(q, Ks, Vs, cache.lens.tolist(), rows, 8), "cfg5 decode")
+
+
+def _oracle_all_rows(q, K, V, lens, n_rep, out, what, chunk=8):
+    """Every sequence of the batch against the fp32 oracle, `chunk` sequences at a time."""
+    for b0 in range(0, q.shape[0], chunk):
+        rows = list(range(b0, min(b0 + chunk, q.shape[0])))
+        assert_attention_close(out[rows], _oracle_rows(q, K, V, lens, rows, n_rep), f"{what}, sequences {rows[0]}..{rows[-1]}")
+
+
+def test_cfg2_headline_launch_as_benchmarked(device):
+    """The launch the headline figure is timed on, as bench.py issues it: the fused append + decode kernel started
+    through the C ABI with frozen metadata and a work list, batch 64 x 4096 (+1), permuted pool.  All 64 sequences
+    are compared with the fp32 oracle, and the slot the launch writes (position 4096) bit for bit."""
+    from pace_mi355.llm import PagedKVCache
+    from pace_mi355.utils.fixed_step import FixedStep
+
+    B, Hq, Hkv, D, ctx = 64, 32, 8, 128, 4096
+    gen = torch.Generator(device=device).manual_seed(1)
+    cache = PagedKVCache(ctx + 64, num_kv_heads=Hkv, n_rep=4, num_blocks=B * 260)
+    K, V = _fill(cache, [ctx] * B, gen, device, Hkv, D, seed=1)
+    k1, v1 = _randn_bf16((B, Hkv, 1, D), gen, device), _randn_bf16((B, Hkv, 1, D), gen, device)
+    q = _randn_bf16((B, Hq, 1, D), gen, device)
+    step = FixedStep(torch, cache, q, k1, v1, fused=True)
+    assert step.kernel == "pace_kv::paged_attn_kernel<128, 1, false, 4, 2, 8, true, false, true>", step.kernel
+    assert step.n_items >= B and step.args.work_items, "the benchmarked launch runs from a work list"
+    pool_before = cache.pool.clone()
+    step()  # one fused launch: stores token 4096 of every sequence and attends over 4097 tokens
+    torch.cuda.synchronize()
+    out = step.out.clone()
+    K1, V1 = torch.cat([K, k1], 2), torch.cat([V, v1], 2)
+    _oracle_all_rows(q, K1, V1, [ctx + 1] * B, 4, out, "cfg2 fused launch")
+    # what the launch stored: the new token's slot holds k1 / v1 bit for bit, nothing else in the pool changed
+    cache.lens = cache.lens + 1  # (the direct call does not move the host-side lengths)
+    cache.seq_len += 1
+    gk, gv = cache.gather(n_rep=1)
+    assert torch.equal(gk[:, :, ctx], k1[:, :, 0]) and torch.equal(gv[:, :, ctx], v1[:, :, 0]), "slot 4096 must hold the new token"
+    assert torch.equal(gk, K1) and torch.equal(gv, V1)
+    changed = (cache.pool != pool_before).flatten(1).any(1).sum().item()
+    assert changed <= B, f"the launch rewrote {changed} blocks; it may touch one per sequence"
+    # a second launch on the same state (what the timed loop does) gives the same bits
+    step()
+    torch.cuda.synchronize()
+    assert torch.equal(step.out, out)
+
+
+def test_cfg4_fused_verify_launch_as_benchmarked(device):
+    """The cfg4 launch of bench.py --workload verify: 8 draft tokens per sequence appended by the attention launch
+    itself (fused), causal 8-query attention, batch 32 with contexts U[1024, 8192]; every sequence against the
+    oracle, the eight new slots of every sequence bit for bit."""
+    from pace_mi355.llm import PagedKVCache
+    from pace_mi355.utils.fixed_step import FixedStep
+
+    B, Hq, Hkv, D, S = 32, 32, 8, 128, 8
+    lens = np.random.default_rng(4).integers(1024, 8193, B).tolist()
+    cache = PagedKVCache(max(lens) + 64, num_kv_heads=Hkv, n_rep=4, num_blocks=B * ((max(lens) + 64) // 16 + 1))
+    gen = torch.Generator(device=device).manual_seed(4)
+    K, V = _fill(cache, lens, gen, device, Hkv, D, chunk=2048, seed=4)
+    kd, vd = _randn_bf16((B, Hkv, S, D), gen, device), _randn_bf16((B, Hkv, S, D), gen, device)
+    q = _randn_bf16((B, Hq, S, D), gen, device)
+    step = FixedStep(torch, cache, q, kd, vd, fused=True)
+    assert "paged_attn_kernel<128, 2, false" in step.kernel and ", true, false, true>" in step.kernel, step.kernel
+    step()
+    torch.cuda.synchronize()
+    out = step.out.clone()
+    K1 = torch.cat([K, torch.zeros_like(kd)], 2)
+    V1 = torch.cat([V, torch.zeros_like(vd)], 2)
+    for b, n in enumerate(lens):
+        K1[b, :, n : n + S], V1[b, :, n : n + S] = kd[b], vd[b]
+    lens_v = [n + S for n in lens]
+    _oracle_all_rows(q, K1, V1, lens_v, 4, out, "cfg4 fused verify launch")
+    cache.lens = cache.lens + S
+    cache.seq_len = int(cache.lens.max())
+    gk, gv = cache.gather(n_rep=1)
+    assert torch.equal(gk, K1) and torch.equal(gv, V1), "the eight new slots of every sequence hold the drafts bit for bit"
+    step()
+    torch.cuda.synchronize()
+    assert torch.equal(step.out, out)

@@ -227,3 +227,54 @@ def test_manager_decode_step_captured_once_and_replayed_per_token(device):
         models[layer].append(ks[layer].cpu(), vs[layer].cpu())
         from helpers import assert_attention_close
         assert_attention_close(outs[layer], models[layer].attention(qs[layer].cpu(), n_rep), f"eager step after the graph, layer {layer}")
+
+
+def test_a_step_that_is_not_the_captured_kind_is_refused(device):
+    """A step that does more on a cache than one update_cache + attention per layer would make the capture record
+    uploads of host data (stale on replay): the eager run shows it and the capture is refused; a step that only
+    departs from its eager run while it is being captured raises inside the capture.  The cache works on
+    step by step afterwards."""
+    from oracle.paged_ref import RaggedCacheModel
+    from pace_mi355.llm import PagedKVCache
+    from pace_mi355.llm.graph import DecodeGraph
+
+    B, hkv, n_rep, D = 2, 2, 4, 128
+    cache = PagedKVCache(512, num_kv_heads=hkv, n_rep=n_rep)
+    model = RaggedCacheModel(B, hkv, D)
+    k, v = seeded_kv(1, B, hkv, 100, D)
+    cache.append_ragged(k.to(device), v.to(device), [100, 40])
+    model.append(k, v, [100, 40])
+    k1, v1 = (t.to(device) for t in seeded_kv(2, B, hkv, 1, D))
+    q = seeded_q(3, B, hkv * n_rep, 1, D).to(device)
+
+    def two_updates():  # the second update of the layer flushes the first: not a captured step
+        cache.update_cache(k1, v1, 2)
+        cache.update_cache(k1, v1, 2)
+        return cache.attend(q)
+
+    with pytest.raises(RuntimeError, match="cannot be captured"):
+        DecodeGraph([cache], two_updates, 4)
+    assert cache._graph is None and cache.lens.tolist() == [100, 40], "a refused capture leaves the cache as it was"
+
+    calls = [0]
+
+    def changes_its_mind():  # eager run: a proper step; under capture: a gather in the middle
+        calls[0] += 1
+        cache.update_cache(k1, v1, 2)
+        if calls[0] == 2:
+            cache.gather()
+        return cache.attend(q)
+
+    with pytest.raises(RuntimeError, match="differs from its eager run"):
+        DecodeGraph([cache], changes_its_mind, 4)
+    torch.cuda.synchronize()
+    assert cache._graph is None and cache.lens.tolist() == [100, 40] and cache._pending is None
+    # step by step from here, as if nothing had happened
+    cache.update_cache(k1, v1, 2)
+    model.append(k1.cpu(), v1.cpu())
+    from helpers import assert_attention_close
+    assert_attention_close(cache.attend(q), model.attention(q.cpu(), n_rep), "eager step after the refused captures")
+    K, V = model.dense(1)
+    gk, gv = cache.gather(n_rep=1)
+    assert_bits_equal(gk, K, "pool K")
+    assert_bits_equal(gv, V, "pool V")

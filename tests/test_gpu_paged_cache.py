@@ -293,4 +293,24 @@ def test_random_histories_with_real_data(device, seed):
         gk, gv = cache.gather(n_rep=1)
         assert_bits_equal(gk, K, f"K after step {step} ({op})")
         assert_bits_equal(gv, V, f"V after step {step} ({op})")
-    assert cache.cow_blocks_copied > 0
+    # Copy-on-write by construction, whatever the history above happened to do: every sequence is brought to a
+    # partly filled last block, sequences 1 and 3 become copies of 0 and 2, and a uniform append follows.  The first
+    # writer of each shared tail block must get a private copy of it (one block per pair), the second then owns the
+    # original alone; the dense view and the attention over it must still match the oracle.
+    counts = [(5 - n) % 16 for n in model.seq_lens()]
+    k, v = seeded_kv(9000 + seed, B, H, 16, D)
+    cache.append_ragged(k.to(device), v.to(device), counts)
+    model.append(k, v, counts)
+    cache.reorder([0, 0, 2, 2])
+    model.reorder([0, 0, 2, 2])
+    copied_before = cache.cow_blocks_copied
+    k, v = seeded_kv(9100 + seed, B, H, 1, D)
+    cache.update_cache(k.to(device), v.to(device), 2)
+    model.append(k, v)
+    q = seeded_q(9200 + seed, B, H * n_rep, 1, D)
+    assert_attention_close(cache.attend(q.to(device)), model.attention(q, n_rep), "attention after the forced copy-on-write")
+    assert cache.cow_blocks_copied == copied_before + 2
+    K, V = model.dense()
+    gk, gv = cache.gather(n_rep=1)
+    assert_bits_equal(gk, K, "K after the forced copy-on-write")
+    assert_bits_equal(gv, V, "V after the forced copy-on-write")
