@@ -59,4 +59,4 @@ int check_pool(const pace_kv_pool_t* pool, const char* who, bool f32_ok) {
 
 extern "C" const char* pace_kv_last_error(void) { return pace_kv::g_error; }
 
-extern "C" int32_t pace_kv_abi_version(void) { return 13; }
+extern "C" int32_t pace_kv_abi_version(void) { return 14; }

@@ -618,8 +618,8 @@ extern "C" int pace_kv_copy_blocks(const pace_kv_pool_t* src_in, const pace_kv_p
 }
 
 extern "C" int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, int32_t n_pools, const int32_t* block_table,
-                                          int32_t table_stride, const int64_t* n_blocks, int32_t batch, int32_t* moves_host,
-                                          int32_t capacity, int32_t* moves_dev, void* stream) {
+                                          int32_t table_stride, const int64_t* n_blocks, int32_t batch, const uint8_t* is_free,
+                                          int32_t* moves_host, int32_t capacity, int32_t* moves_dev, void* stream) {
   const char* who = "pace_kv_compact_blocks";
   if (!pools || n_pools < 1 || !moves_host || !moves_dev) {
     set_error("%s: NULL pools / moves_host / moves_dev or no pool", who);
@@ -633,8 +633,10 @@ extern "C" int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, in
     }
   }
   // the plan reads the table only (apply = 0): the caller rewrites it with pace_kv_apply_moves while the copies run
-  const int32_t n = pace_kv_plan_compaction(const_cast<int32_t*>(block_table), table_stride, n_blocks, batch, pools[0]->num_blocks,
-                                            moves_host, capacity, 0, nullptr);
+  // (from the allocator's free flags when the caller has them: a pass over one byte per block instead of the table)
+  const int32_t n = is_free ? pace_kv_plan_compaction_flags(is_free, pools[0]->num_blocks, moves_host, capacity)
+                            : pace_kv_plan_compaction(const_cast<int32_t*>(block_table), table_stride, n_blocks, batch,
+                                                      pools[0]->num_blocks, moves_host, capacity, 0, nullptr);
   if (n <= 0) return n;
   if (hipMemcpyAsync(moves_dev, moves_host, (size_t)n * 2 * sizeof(int32_t), hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)) !=
       hipSuccess) {

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 
 BLOCK_TOKENS = 16
 DTYPE_F32, DTYPE_BF16 = 0, 1
-ABI_VERSION = 13
+ABI_VERSION = 14
 STATIC_SCRATCH_BYTES = 32 << 20  # PACE_PAGED_ATTN_STATIC_SCRATCH_BYTES
 HEAD_DIMS = (64, 96, 128, 256)  # head sizes the pool kernels are built for
 
@@ -35,6 +35,8 @@ EXPORTED_SYMBOLS = (
     "pace_paged_attn_kernel_name",
     "pace_kv_plan_compaction",
     "pace_kv_apply_moves",
+    "pace_kv_apply_moves_tracked",
+    "pace_kv_plan_compaction_flags",
     "pace_paged_attn_workspace_bytes",
     "pace_paged_attn_workspace_bytes_for_parts",
     "pace_paged_attn_decode",
@@ -229,7 +231,13 @@ def load() -> ctypes.CDLL:
         c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
     ]
     lib.pace_kv_compact_blocks.restype = c_int32
-    lib.pace_kv_compact_blocks.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
+    lib.pace_kv_compact_blocks.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_void_p,
+                                           c_void_p]
+    lib.pace_kv_plan_compaction_flags.restype = c_int32
+    lib.pace_kv_plan_compaction_flags.argtypes = [c_void_p, c_int32, c_void_p, c_int32]
+    lib.pace_kv_apply_moves_tracked.restype = ctypes.c_int
+    lib.pace_kv_apply_moves_tracked.argtypes = [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p,
+                                                c_void_p]
     lib.pace_attn_dense_ws.restype = ctypes.c_int
     lib.pace_attn_dense_ws.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,

@@ -207,6 +207,7 @@ class PagedKVCache(KVCacheBase):
         self.pool = torch.zeros((nb, hkv, 2, BLOCK * D), dtype=key_states.dtype, device=key_states.device)
         self.state.pools.append(self.pool)
         self._desc = self._describe(self.pool)
+        self.state.pool_descs.append(self._desc)
         self.lens = np.zeros(B, dtype=np.int64)
 
     def _describe(self, pool: torch.Tensor) -> nat.PoolDesc:
@@ -424,7 +425,7 @@ class PagedKVCache(KVCacheBase):
             if p.pool is not None:
                 p._flush()
         # one library call plans the moves, uploads them and starts the copies of every layer's pool
-        moves = self.state.compact_blocks([self._describe(pool) for pool in self.state.pools])
+        moves = self.state.compact_blocks(self.state.pool_descs)
         if len(moves):
             self.state.apply_moves(moves)  # the table rewrite runs on the host while the GPU copies
         return len(moves)

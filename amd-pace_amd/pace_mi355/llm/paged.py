@@ -135,6 +135,11 @@ class BlockAllocator:
     def free_ids(self) -> np.ndarray:
         return np.nonzero(self._is_free)[0]
 
+    def free_flags_ptr(self) -> int:
+        """Address of the free flags, one byte per block id (1 = free), for the native planner."""
+        assert self._is_free.dtype == np.bool_ and self._is_free.flags.c_contiguous
+        return self._is_free.ctypes.data
+
 
 def _ragged_cells(first: np.ndarray, count: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
     """Row and column indices of cells ``first[b] .. first[b] + count[b] - 1`` of every row ``b``, row by row."""
@@ -165,6 +170,7 @@ class PagedState:
         self.table = np.zeros((self.batch, self.max_blocks_per_seq), dtype=np.int32)
         self.n_blocks = np.zeros(self.batch, dtype=np.int64)  # table entries in use per sequence
         self.pools: List["torch.Tensor"] = []  # one [num_blocks][Hkv][2][16*D] tensor per layer
+        self.pool_descs: list = []  # the library's descriptor of each pool, in the same order
         self._table_dev: Optional[torch.Tensor] = None
         self._table_dirty = True
         self._lens_dev: Optional[torch.Tensor] = None
@@ -394,7 +400,7 @@ class PagedState:
         ptrs = (ctypes.c_void_p * len(descs))(*[ctypes.addressof(d) for d in descs])
         n = int(nat.load().pace_kv_compact_blocks(
             ptrs, len(descs), self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch,
-            self._pairs_host.data_ptr(), cap, self._pairs_dev.data_ptr(), nat.current_stream_ptr()))
+            self.allocator.free_flags_ptr(), self._pairs_host.data_ptr(), cap, self._pairs_dev.data_ptr(), nat.current_stream_ptr()))
         if n < 0:
             nat.check(n)
         if n:
@@ -460,9 +466,8 @@ class PagedState:
         id below it.  Returns ``[n_moves, 2]`` int32 ``(src, dst)``; the two id
         sets are disjoint.  (The passes over the table run in the library.)"""
         moves = np.empty((self.allocator.num_blocks, 2), dtype=np.int32)
-        n = int(nat.load().pace_kv_plan_compaction(
-            self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch, self.allocator.num_blocks,
-            moves.ctypes.data, moves.shape[0], 0, None))
+        n = int(nat.load().pace_kv_plan_compaction_flags(self.allocator.free_flags_ptr(), self.allocator.num_blocks, moves.ctypes.data,
+                                                         moves.shape[0]))
         if n < 0:
             nat.check(n)
         return moves[:n]
@@ -473,11 +478,13 @@ class PagedState:
         if not len(moves):
             return
         moves = np.ascontiguousarray(moves, dtype=np.int32)
-        refs = np.empty(self.allocator.num_blocks, dtype=np.int32)
-        nat.check(nat.load().pace_kv_apply_moves(
-            self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch, self.allocator.num_blocks,
-            moves.ctypes.data, len(moves), refs.ctypes.data))
-        self.allocator.reset_free(refs == 0, refs)
+        alloc = self.allocator
+        n_free = ctypes.c_int32(0)
+        # the table, the owners per block, the free flags and the free list in one pass of native code
+        nat.check(nat.load().pace_kv_apply_moves_tracked(
+            self.table.ctypes.data, self.table.shape[1], self.n_blocks.ctypes.data, self.batch, alloc.num_blocks,
+            moves.ctypes.data, len(moves), alloc.refs.ctypes.data, alloc.free_flags_ptr(), alloc._stack.ctypes.data, ctypes.byref(n_free)))
+        alloc._n_free = int(n_free.value)
         self._table_dirty = True
         self.table_version += 1
 

@@ -185,7 +185,8 @@ int pace_kv_apply_moves(int32_t* block_table, int32_t table_stride, const int64_
                         int32_t num_blocks, const int32_t* moves, int32_t n_moves, int32_t* refs);
 
 /*
- * Compaction in one call: pace_kv_plan_compaction (apply = 0) into moves_host [capacity][2], the upload of the
+ * Compaction in one call: pace_kv_plan_compaction (apply = 0; with is_free != NULL: pace_kv_plan_compaction_flags,
+ * below) into moves_host [capacity][2], the upload of the
  * moves to moves_dev (device memory for as many pairs) and pace_kv_copy_blocks for each of the n_pools pools that
  * share the table (the layers of a model), all on `stream`.  Returns the number of moves or a negative code.
  * Afterwards the caller rewrites its table with pace_kv_apply_moves(moves_host, returned count) -- on the host,
@@ -194,8 +195,26 @@ int pace_kv_apply_moves(int32_t* block_table, int32_t table_stride, const int64_
  * caches are dense tensors (pace/llm/cache.py:161-167 is its only copy between cache rows).
  */
 int32_t pace_kv_compact_blocks(const pace_kv_pool_t* const* pools, int32_t n_pools, const int32_t* block_table,
-                               int32_t table_stride, const int64_t* n_blocks, int32_t batch, int32_t* moves_host,
-                               int32_t capacity, int32_t* moves_dev, void* stream);
+                               int32_t table_stride, const int64_t* n_blocks, int32_t batch, const uint8_t* is_free,
+                               int32_t* moves_host, int32_t capacity, int32_t* moves_dev, void* stream);
+
+/*
+ * The plan of pace_kv_plan_compaction from the allocator's own record of the pool instead of the table: is_free
+ * [num_blocks], one byte per block id, non-zero = free (every id the table names must be marked used).  The same
+ * moves in the same order; a pass over num_blocks bytes instead of a walk over every table entry.
+ */
+int32_t pace_kv_plan_compaction_flags(const uint8_t* is_free, int32_t num_blocks, int32_t* moves, int32_t capacity);
+
+/*
+ * pace_kv_apply_moves with the allocator's bookkeeping moved along instead of recounted: refs [num_blocks] (owners
+ * per block) and is_free [num_blocks] (1 = free, 0 = used) are updated in place -- a moved block takes its owners
+ * with it, its old id becomes free -- and the free list is written afresh into free_stack [num_blocks]: *n_free ids,
+ * the lowest id last (the stack's top).  Every move must take a used id to a free one and no id may occur twice
+ * (else PACE_KV_EINVAL and nothing is changed).
+ */
+int pace_kv_apply_moves_tracked(int32_t* block_table, int32_t table_stride, const int64_t* n_blocks, int32_t batch,
+                                int32_t num_blocks, const int32_t* moves, int32_t n_moves, int32_t* refs,
+                                uint8_t* is_free, int32_t* free_stack, int32_t* n_free);
 
 /*
  * Rotary position embedding, the step the models run on q and k right before the

@@ -334,6 +334,54 @@ def test_fork_shares_blocks_and_copy_on_write_touches_only_shared_tails():
         st2.fork([0, 5])
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_compaction_plan_from_free_flags_and_tracked_apply_agree_with_the_table_walk(seed):
+    """The planner that reads the allocator's free flags gives the moves of the planner that walks the table, and the
+    apply that moves the bookkeeping along leaves what a recount leaves: the same table, owners per block, free
+    flags, and a free list that hands out the lowest ids first.  Forked sequences (blocks with several owners)
+    included; a move that does not take a used block to a free one is refused and nothing changes."""
+    from pace_mi355 import _native as nat
+
+    lib = nat.load()
+    rng = np.random.default_rng(seed)
+    B, N = 5, 157
+    st = _state(batch=B, max_len=16 * 40, blocks=N)
+    lens = rng.integers(1, 16 * 30, B)
+    st.ensure_capacity(lens)
+    for b in range(B):
+        n = int(st.n_blocks[b])
+        if n > 2:
+            lens = st.evict(b, sorted(rng.choice(n, size=n // 3, replace=False).tolist()), lens)
+    st.fork([0, 0, 2, 3, 3])  # shared blocks: owners per block above one
+    lens = lens[[0, 0, 2, 3, 3]]
+    alloc = st.allocator
+    # the two planners
+    by_table = np.empty((N, 2), np.int32)
+    n1 = lib.pace_kv_plan_compaction(st.table.ctypes.data, st.table.shape[1], st.n_blocks.ctypes.data, B, N, by_table.ctypes.data, N, 0, None)
+    by_flags = st.plan_compaction()
+    assert n1 == len(by_flags) > 0 and np.array_equal(by_table[:n1], by_flags)
+    # reference result: the recounting apply on copies
+    table0, refs0 = st.table.copy(), alloc.refs.copy()
+    want_table, want_refs = st.table.copy(), np.empty(N, np.int32)
+    nat.check(lib.pace_kv_apply_moves(want_table.ctypes.data, want_table.shape[1], st.n_blocks.ctypes.data, B, N, by_flags.ctypes.data, n1,
+                                      want_refs.ctypes.data))
+    # a bad move first: destination in use -> refused, nothing touched
+    bad = by_flags.copy()
+    bad[-1, 1] = by_flags[0, 0]
+    flags0, stack0, nfree0 = alloc._is_free.copy(), alloc._stack.copy(), alloc.num_free
+    with pytest.raises(Exception, match="does not take a live block to a free one"):
+        st.apply_moves(bad)
+    assert np.array_equal(st.table, table0) and np.array_equal(alloc.refs, refs0) and np.array_equal(alloc._is_free, flags0)
+    assert np.array_equal(alloc._stack, stack0) and alloc.num_free == nfree0
+    st.apply_moves(by_flags)
+    assert np.array_equal(st.table, want_table) and np.array_equal(alloc.refs, want_refs)
+    assert np.array_equal(alloc._is_free, want_refs == 0) and alloc.num_free == int((want_refs == 0).sum())
+    live = st.live_block_count()
+    assert sorted(alloc.free_ids().tolist()) == list(range(live, N))
+    assert alloc.allocate(3) == [live, live + 1, live + 2], "the lowest free ids are handed out first"
+    assert len(st.plan_compaction()) == 0
+
+
 def test_compaction_moves_a_shared_block_once():
     st = _state(batch=3, max_len=160, blocks=30)
     st.ensure_capacity(np.array([48, 48, 48]))
