@@ -93,6 +93,13 @@ struct DenseParams {
   // each leaves (o unnormalised, m, l) per row in `part` ([row][n_split][H + 4] floats), attn_paged_f32_merge_kernel ends.
   int32_t n_split;
   float* part;
+  // PAGED with a fused append (FUSED): the last n_new tokens of every sequence are read from k_new / v_new
+  // ([batch][KV heads][n_new][H] floats, element strides n_sb / n_sh / n_st) instead of from the pool, and the first
+  // workgroup of every (sequence, KV head) stores them into their pool rows.
+  const float* k_new;
+  const float* v_new;
+  int64_t n_sb, n_sh, n_st;
+  int32_t n_new;
 };
 
 // HP: head size rounded up to the next size built (dims >= H read as zero).  VEC: H is a multiple
@@ -108,8 +115,9 @@ struct DenseParams {
 // (the first product) and of sixteen chunks of a row (the second) off each other's banks; a head size below the built
 // one is padded with zeros on the way in.  Each wave fetching its
 // own operands from memory held the launch at 65 % of what the arithmetic alone takes.
-template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED, bool COOP = false>
+template <typename T, typename MT, int HP, bool VEC, bool AHEAD, bool EXACT, bool PAGED, bool COOP = false, bool FUSED = false>
 __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
+  static_assert(!FUSED || (PAGED && !COOP), "the fused append belongs to the pool's launches of few query rows");
   static_assert(!COOP || (VEC && !AHEAD && sizeof(T) == 4), "the cooperative walk: fp32 rows of a multiple of four dims");
   static_assert(!EXACT || VEC, "a head size that is one of the built ones is a multiple of 4");
   static_assert(!PAGED || (VEC && sizeof(T) == 4), "pools of rows hold fp32 with head sizes that are multiples of 4");
@@ -133,8 +141,10 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   // L: keys of this (batch, head); R: its query rows; [start, L) can be read, by this lane's row up to `limit`;
   // mcols: columns of a mask line.  Without PAGED these are the launch's constants.
   int L = p.L, R = S, start = 0, mcols = p.L;
+  int pool_end = 0x7fffffff, n_new = 0;  // FUSED: tokens [pool_end, pool_end + n_new) are this step's new ones
   if constexpr (PAGED) {
     L = max(0, p.seq_lens[b] + p.len_bias + (p.len_bias_dev ? *p.len_bias_dev : 0));
+    if constexpr (FUSED) n_new = min(p.n_new, L), pool_end = L - n_new;
     if (p.mask) L = min(L, p.mask_len);  // columns the mask does not have are masked
     start = p.kv_start ? min(max(p.kv_start[b], 0), L) : 0;
     R = S * p.n_rep, mcols = p.mask_len;
@@ -215,6 +225,25 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
   const int per = (wg_hi - wg_lo + split - 1) / split;
   const int tile_lo = min(wg_hi, wg_lo + ls * per), tile_hi = min(wg_hi, tile_lo + per);
   const bool has_rows = rowgroup * 16 < R;  // wave-uniform
+  if constexpr (FUSED) {
+    // The first workgroup of this (sequence, KV head) stores the step's new rows into the pool; no workgroup of the
+    // launch reads those pool rows (they all take them from the caller's buffers).
+    if (blockIdx.x == 0 && n_new > 0) {
+      const int chunks = H / 4;  // (H is a multiple of 4)
+      for (int item = threadIdx.x; item < n_new * chunks; item += 256) {
+        const int idx = item / chunks, c = item % chunks, pos = pool_end + idx, jb = pos / PACE_KV_BLOCK_TOKENS;
+        if (jb >= p.table_stride) continue;
+        const int64_t blk = p.table[(int64_t)b * p.table_stride + jb];
+        if (blk < 0 || blk >= p.num_blocks) continue;  // never write outside the pool
+        const int64_t src = b * p.n_sb + head * p.n_sh + (int64_t)idx * p.n_st + 4 * c;
+        const int64_t dst = (int64_t)(pos % PACE_KV_BLOCK_TOKENS) * H + 4 * c;
+        float* kdst = const_cast<float*>(static_cast<const float*>(p.k)) + blk * p.k_bs + head * p.k_hs + dst;
+        float* vdst = const_cast<float*>(static_cast<const float*>(p.v)) + blk * p.v_bs + head * p.v_hs + dst;
+        *reinterpret_cast<u32x4*>(kdst) = *reinterpret_cast<const u32x4*>(p.k_new + src);
+        *reinterpret_cast<u32x4*>(vdst) = *reinterpret_cast<const u32x4*>(p.v_new + src);
+      }
+    }
+  }
   float kf[KS], vf[MTL][4], mv[4];
   auto fetch_mask = [&](int tile, float (&mx4)[4]) {
     // the lane's four mask values: one load where the four columns exist (mask lines start wherever L puts them;
@@ -248,14 +277,28 @@ __device__ __forceinline__ void attn_dense_body(const DenseParams& p) {
       const int64_t blk = min(max(p.table[(int64_t)b * p.table_stride + min(tile, p.table_stride - 1)], 0), p.num_blocks - 1);
       kblock = kbase + blk * p.k_bs - (int64_t)t0 * H, vblock = vbase + blk * p.v_bs - (int64_t)t0 * H;
     }
+    // FUSED, a tile that holds new tokens: their rows are read from the caller's buffers (index held inside them:
+    // rows past the end are masked below), the others from the pool as ever.  Wave-uniform.
+    const bool with_new = FUSED && n_new > 0 && t0 + 16 > pool_end;
+    const T* new_k = nullptr;
+    const T* new_v = nullptr;
+    if constexpr (FUSED) {
+      new_k = reinterpret_cast<const T*>(p.k_new) + b * p.n_sb + head * p.n_sh;
+      new_v = reinterpret_cast<const T*>(p.v_new) + b * p.n_sb + head * p.n_sh;
+    }
+    auto row_of = [&](const T* pool_rows, const T* new_rows, int pos) -> const T* {
+      if (with_new && pos >= pool_end) return new_rows + (int64_t)min(pos - pool_end, n_new - 1) * p.n_st;
+      return pool_rows + (int64_t)pos * H;
+    };
     // rows past the end are masked below (PAGED: the block's 16 rows exist whatever the length is)
-    load_run(kblock + (int64_t)(PAGED ? t0 + n : min(L - 1, t0 + n)) * H, kx, std::integral_constant<bool, ONCE>{});
+    if (FUSED) load_run(row_of(kblock, new_k, t0 + n), kx, std::integral_constant<bool, ONCE>{});
+    else load_run(kblock + (int64_t)(PAGED ? t0 + n : min(L - 1, t0 + n)) * H, kx, std::integral_constant<bool, ONCE>{});
     // V: output tile j of lane n stands for dim v_dim(j, n) = 16 VG (j / VG) + VG n + j % VG, so that the VG values a
     // lane needs of one token for VG neighbouring tiles are one contiguous run: a quarter of the load instructions
     // that one value per load takes, and every load of a wave covers whole 256-byte stretches of four rows.
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const T* vr = vblock + (int64_t)(PAGED ? t0 + 4 * g + i : min(L - 1, t0 + 4 * g + i)) * H;
+      const T* vr = FUSED ? row_of(vblock, new_v, t0 + 4 * g + i) : vblock + (int64_t)(PAGED ? t0 + 4 * g + i : min(L - 1, t0 + 4 * g + i)) * H;
 #pragma unroll
       for (int jj = 0; jj < MTL; jj += VG) {
         const int d = 16 * jj + VG * n;
@@ -556,10 +599,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128
 // The same walk over a pool of fp32 rows (pace_kv_pool_t with elem_bytes 4).  No fetch a tile ahead: here the second
 // wave per SIMD hides more than the second set of registers did (decode, batch 64 x 8 KV heads x 4096 tokens of 128
 // dims: 370 us against 460).
-template <typename MT, int HP, bool EXACT>
+template <typename MT, int HP, bool EXACT, bool FUSED = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, HP > 128 ? 1 : 2))) void attn_paged_f32_kernel(
     const DenseParams p) {
-  attn_dense_body<float, MT, HP, true, false, EXACT, true>(p);
+  attn_dense_body<float, MT, HP, true, false, EXACT, true, false, FUSED>(p);
 }
 
 // Ends a launch whose sequences were cut over several workgroups: out = sum_i e^(m_i - M) o_i / sum_i e^(m_i - M) l_i
@@ -621,10 +664,19 @@ int launch_paged_f32(const pace_kv_pool_t* pool, const pace_paged_attn_args_t* a
   const dim3 grid((unsigned)((rowgroups + per_wg - 1) / per_wg * p.n_split), pool->num_kv_heads, a->batch);
   const bool mf32 = a->mask_dtype == PACE_DTYPE_F32;
   const bool coop = p.l_split == 1 && p.n_split == 1;
+  const bool fused = a->k_new != nullptr;
+  if (fused) {
+    PACE_REQUIRE(rows <= 32, "%s: over an fp32 pool the append rides in launches of up to 32 query rows per KV head (got %lld)", who,
+                 (long long)rows);
+    p.k_new = static_cast<const float*>(a->k_new), p.v_new = static_cast<const float*>(a->v_new);
+    p.n_sb = a->new_stride_b, p.n_sh = a->new_stride_h, p.n_st = a->new_stride_t, p.n_new = a->n_new;
+  }
 #define PACE_PAGED_F32_GO(MT_, HP_) \
   do { \
     if (H == HP_ && coop) hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, true, true>), grid, dim3(256), 0, stream, p); \
     else if (coop) hipLaunchKernelGGL((attn_f32_coop_kernel<MT_, HP_, true, false>), grid, dim3(256), 0, stream, p); \
+    else if (H == HP_ && fused) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true, true>), grid, dim3(256), 0, stream, p); \
+    else if (fused) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false, true>), grid, dim3(256), 0, stream, p); \
     else if (H == HP_) hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, true>), grid, dim3(256), 0, stream, p); \
     else hipLaunchKernelGGL((attn_paged_f32_kernel<MT_, HP_, false>), grid, dim3(256), 0, stream, p); \
   } while (0)

@@ -1084,8 +1084,14 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
                a->num_q_heads, pool->num_kv_heads);
   if (pool_is_f32(pool)) {
     // rows of fp32: the general kernel of the dense operator walks the block table (dense_attn.hip)
-    PACE_REQUIRE(!a->k_new && !a->v_new && !a->rope,
-                 "%s: an fp32 pool takes neither a fused append nor a rotary embedding inside the attention launch", who);
+    PACE_REQUIRE(!a->rope, "%s: an fp32 pool takes no rotary embedding inside the attention launch", who);
+    if (a->k_new || a->v_new) {
+      PACE_REQUIRE(a->k_new && a->v_new, "%s: k_new and v_new must be given together", who);
+      PACE_REQUIRE(a->n_new >= 1 && a->n_new <= 32, "%s: fused append takes 1..32 new tokens (got %d)", who, a->n_new);
+      PACE_REQUIRE(aligned16(a->k_new) && aligned16(a->v_new) && (a->new_stride_b % 4) == 0 && (a->new_stride_h % 4) == 0 &&
+                       (a->new_stride_t % 4) == 0,
+                   "%s: k_new / v_new must be 16-byte aligned with strides that are multiples of 4 elements", who);
+    }
     PACE_REQUIRE(aligned16(a->q) && aligned16(a->out) && (a->q_stride_b % 4) == 0 && (a->q_stride_h % 4) == 0 &&
                      (a->q_stride_s % 4) == 0 && (a->o_stride_b % 4) == 0 && (a->o_stride_h % 4) == 0 && (a->o_stride_s % 4) == 0,
                  "%s: q and out must be 16-byte aligned with strides that are multiples of 4 elements", who);
@@ -1098,8 +1104,8 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
                    "%s: bad mask dtype %d or mask_len %d", who, a->mask_dtype, a->mask_len);
     if (g_name_out) {  // (pace_paged_attn_kernel_name: nothing is launched)
       const int H = pool->head_dim, hp = H <= 32 ? 32 : (H <= 64 ? 64 : (H <= 96 ? 96 : (H <= 128 ? 128 : 256)));
-      snprintf(g_name_out, g_name_cap, "pace_kv::attn_paged_f32_kernel<%s, %d, %s>",
-               a->mask_dtype == PACE_DTYPE_F32 ? "float" : "unsigned short", hp, H == hp ? "true" : "false");
+      snprintf(g_name_out, g_name_cap, "pace_kv::attn_paged_f32_kernel<%s, %d, %s, %s>",
+               a->mask_dtype == PACE_DTYPE_F32 ? "float" : "unsigned short", hp, H == hp ? "true" : "false", a->k_new ? "true" : "false");
       return PACE_KV_OK;
     }
     return launch_paged_f32(pool, a, who, static_cast<hipStream_t>(stream));

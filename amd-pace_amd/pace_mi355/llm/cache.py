@@ -175,10 +175,9 @@ class PagedKVCache(KVCacheBase):
         if key_states.dtype not in (torch.bfloat16, torch.float32):
             raise RuntimeError(f"PagedKVCache stores bf16 or fp32; got {key_states.dtype}")
         # fp32 (the reference's caches keep the model's dtype, ``pace/llm/cache.py:255-266``): blocks of plain rows,
-        # read by the dense operator's fp32 kernel through the block table; nothing is folded into that launch
+        # read by the dense operator's fp32 kernel through the block table; the append rides in that launch when it
+        # has up to 32 query rows per KV head (decode, short verify steps), the rotary embedding never does
         self.f32 = key_states.dtype == torch.float32
-        if self.f32:
-            self.fuse_append = False
         nat.load()
         B, h_in, _, D = key_states.shape
         if self._cfg_kv_heads is not None:
@@ -300,11 +299,12 @@ class PagedKVCache(KVCacheBase):
         if (self._graph is not None and counts is None and (self.fuse_append or self.f32) and T <= 32
                 and self._pending is None and not self._graph_appended):
             # a step of a decode graph: blocks and table were prepared for every step, and the lengths advance on the
-            # device.  bf16: the append rides in the attention launch.  fp32: a launch of its own, its positions
-            # taken from the graph's frozen lengths plus the device counter.
+            # device.  The append rides in the attention launch; over an fp32 pool only with up to 32 query rows per KV
+            # head (else, or with fuse_append off: a launch of its own, its positions taken from the graph's frozen
+            # lengths plus the device counter).
             graph = self._graph
             graph.reserve(T)
-            if self.f32:
+            if self.f32 and (not self.fuse_append or T * self.n_rep > 32):
                 nat.check(
                     lib.pace_kv_append_paged_at(
                         ctypes.byref(self._desc), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * head_step, k.stride(2),
@@ -534,6 +534,8 @@ class PagedKVCache(KVCacheBase):
         if qs[3] != 1 or qs[0] % per16 or qs[1] % per16 or qs[2] % per16 or query.data_ptr() % 16:
             query = query.contiguous()
             qs = query.stride()
+        if self.f32 and self._pending is not None and self._graph is None and S * (hq // self.num_kv_heads) > 32:
+            self._flush()  # over an fp32 pool the append rides in launches of up to 32 query rows per KV head
         rope, self._query_rope = self._query_rope, None
         rope_desc = None
         if rope is not None:

@@ -554,18 +554,36 @@ def wl_dense_f32(torch, dev, args):
 
 def wl_decode_f32pool(torch, dev, args):
     """The headline step for an fp32 model (the reference's caches keep the model's dtype,
-    pace/llm/cache.py:255-266): a pool of fp32 rows, a 1-token append and the decode attention in two launches."""
+    pace/llm/cache.py:255-266): a pool of fp32 rows, the 1-token append and the decode attention in one launch
+    (--no-fuse: the append as a launch of its own)."""
     B, ctx, hq, hkv, D = args.batch or 64, args.context or 4096, 32, 8, 128
     cache = build_cache(torch, dev, [ctx] * B, hq, hkv, D, seed=1, permute=not args.no_permute, f32=True)
     g = torch.Generator(device=dev).manual_seed(2)
     k1, v1, q = (torch.randn(B, h, 1, D, generator=g, device=dev) for h in (hkv, hkv, hq))
-    fs = FixedStep(torch, cache, q, k1, v1, fused=False)
+    fused = not args.no_fuse
+    fs = FixedStep(torch, cache, q, k1, v1, fused=fused)
     dt, attn_ms = run_timed(torch, fs, args.steps, args.warmup)
     nbytes = 2 * decode_bytes(fs.lens_after.tolist(), hq, hkv, D) - 4 * B - 4 * B * math.ceil((ctx + 1) / 16)  # fp32 rows, the same table
+    app = 2 * append_bytes(B, 1, hkv, D)
+    check = {}
+    if not args.no_check:  # the step's output against the fp32 oracle (1e-5), the appended rows bit for bit
+        from oracle.attention_ref import lengths_mask_4d, sdpa_fp32
+        from oracle.cache_ref import repeat_kv
+
+        torch.cuda.synchronize()
+        gk, gv = fs.gathered()
+        rows = [0, B // 2, B - 1]
+        idx = torch.tensor(rows, device=dev)
+        ref = sdpa_fp32(q[idx].cpu(), repeat_kv(gk[idx].cpu(), hq // hkv), repeat_kv(gv[idx].cpu(), hq // hkv),
+                        lengths_mask_4d([ctx + 1] * len(rows), 1, ctx + 1, torch.float32))
+        err = float((fs.out[idx].cpu() - ref).abs().max())
+        slots = bool(torch.equal(gk[:, :, ctx], k1[:, :, 0]) and torch.equal(gv[:, :, ctx], v1[:, :, 0]))
+        check = {"checked": bool(err <= 1e-5 and slots), "max_abs_err": err, "appended_slots_bit_exact": slots, "checked_sequences": rows,
+                 "check": "last timed step vs the fp32 CPU oracle (cap 1e-5); slots of the new tokens bit-exact for every sequence"}
     return result_line(
         args, f"decode over a pool of fp32 rows: batch {B}, context {ctx} (+1 appended), 32 Q / 8 KV heads, head_dim 128, KV block 16, "
-        "seeded random physical block permutation, 1-token append + GQA decode (two launches)",
-        nbytes + 2 * append_bytes(B, 1, hkv, D), B, dt, roofline(fs.kernel, nbytes, attn_ms), extra={"dtype": "f32"})
+        f"seeded random physical block permutation, 1-token append + GQA decode ({'one launch' if fused else 'two launches'})",
+        nbytes + app, B, dt, roofline(fs.kernel, nbytes + (app if fused else 0), attn_ms), extra=dict(check, dtype="f32"))
 
 
 def wl_compact(torch, dev, args):

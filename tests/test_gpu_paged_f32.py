@@ -365,14 +365,84 @@ def test_entry_points_that_fold_steps_in_refuse_an_fp32_pool(device):
     # the entry point that allocates nothing takes the pool too (this kernel has no scratch at all)
     nat.check(lib.pace_paged_attn_verify_static(ctypes.byref(cache._desc), ctypes.byref(a), stream))
     assert_bits_equal(out, cache.attend(q), "static entry point")
-    a.k_new, a.v_new, a.n_new = q.data_ptr(), q.data_ptr(), 1
+    # a rotary embedding never rides in the launch over an fp32 pool; a fused append only with up to 32 query rows per KV head
+    rope = nat.RopeDesc()
+    a.rope = ctypes.pointer(rope)
     assert lib.pace_paged_attn_decode(ctypes.byref(cache._desc), ctypes.byref(a), stream) != 0
     assert "fp32 pool" in lib.pace_kv_last_error().decode()
+    a.rope = None
+    S = 20  # 40 query rows per KV head
+    q2 = seeded_q(4, 2, 4, S, 128, dtype=F32).to(device)
+    out2 = torch.empty_like(q2)
+    a2, keep = _direct_args(cache, q2, out2, 20)
+    kn = torch.zeros(2, 2, S, 128, device=device)
+    a2.k_new, a2.v_new, a2.n_new = kn.data_ptr(), kn.data_ptr(), S
+    a2.new_stride_b, a2.new_stride_h, a2.new_stride_t = kn.stride(0), kn.stride(1), kn.stride(2)
+    assert lib.pace_paged_attn_verify(ctypes.byref(cache._desc), ctypes.byref(a2), stream) != 0
+    assert "up to 32 query rows" in lib.pace_kv_last_error().decode()
     k = torch.zeros(2, 2, 1, 128, dtype=torch.bfloat16, device=device)
     rc = lib.pace_rope_append_paged(ctypes.byref(cache._desc), ctypes.byref(nat.RopeDesc()), None, None, 0, 0, 0, 0, k.data_ptr(),
                                     k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), 2, 1, table.data_ptr(), table.stride(0),
                                     lens_dev.data_ptr(), bias, stream)
     assert rc != 0 and "bf16 pools only" in lib.pace_kv_last_error().decode()
+
+
+@pytest.mark.parametrize("T,n_rep,D,lens", [
+    (1, 4, 128, [4096, 33, 1500, 15]),      # decode; a token that opens a block (15 -> 16) and ones that do not
+    (1, 1, 64, [16, 31, 700]),              # no GQA; lengths on and next to block boundaries
+    (4, 4, 128, [300, 14, 2000, 61, 5]),    # 16 query rows; new tokens straddling a block boundary (14 + 4, 61 + 4)
+    (8, 4, 100, [1000, 9]),                 # 32 query rows, a head size that is none of the built ones
+    (3, 8, 128, [40]),                      # one short sequence (cut over several workgroups through the workspace)
+    (2, 2, 256, [500, 3000]),
+])
+def test_fused_append_equals_append_then_attend(device, T, n_rep, D, lens):
+    """update_cache holds the new tokens back and the attention launch both reads them from the caller's tensors and
+    stores them into the pool (launches of up to 32 query rows per KV head): the same attention result as
+    append-then-attend, within 1e-5 of the oracle, and bit-identical pool contents; the step after reads the stored
+    rows from the pool."""
+    B, hkv = len(lens), 2
+    k_new, v_new = seeded_kv(900 + T, B, hkv, T, D, dtype=F32)
+    q = seeded_q(901, B, hkv * n_rep, T, D, dtype=F32)
+    outs, caches = [], []
+    for fuse in (True, False):
+        cache, model = _build(device, B, hkv, n_rep, D, lens, seed=sum(lens) + T)
+        cache.fuse_append = fuse
+        cache.update_cache(repeat_kv(k_new, n_rep).to(device), repeat_kv(v_new, n_rep).to(device), 2)
+        assert (cache._pending is not None) == fuse
+        outs.append(cache.attend(q.to(device)))
+        assert cache._pending is None
+        caches.append(cache)
+    model.append(k_new, v_new)
+    ref = model.attention(q, n_rep)
+    _close(outs[0], ref, "fused")
+    _close(outs[1], ref, "unfused")
+    K, V = model.dense(1)
+    for c in caches:
+        gk, gv = c.gather(n_rep=1)
+        assert_bits_equal(gk, K, "pool K")
+        assert_bits_equal(gv, V, "pool V")
+    q1 = seeded_q(902, B, hkv * n_rep, 1, D, dtype=F32)
+    k1, v1 = seeded_kv(903, B, hkv, 1, D, dtype=F32)
+    caches[0].update_cache(k1.to(device), v1.to(device), 2)
+    model.append(k1, v1)
+    _close(caches[0].attend(q1.to(device)), model.attention(q1, n_rep), "step after the fused one")
+
+
+def test_held_back_append_is_stored_first_when_the_launch_has_too_many_rows(device):
+    """More than 32 query rows per KV head over an fp32 pool: the held-back append goes out as a launch of its own."""
+    B, hkv, n_rep, D, T = 2, 2, 4, 128, 12   # 48 rows
+    cache, model = _build(device, B, hkv, n_rep, D, [200, 70], seed=5)
+    k_new, v_new = seeded_kv(7, B, hkv, T, D, dtype=F32)
+    q = seeded_q(8, B, hkv * n_rep, T, D, dtype=F32)
+    cache.update_cache(k_new.to(device), v_new.to(device), 2)
+    assert cache._pending is not None
+    out = cache.attend(q.to(device))
+    model.append(k_new, v_new)
+    _close(out, model.attention(q, n_rep), "48 rows")
+    K, V = model.dense(1)
+    gk, gv = cache.gather(n_rep=1)
+    assert_bits_equal(gk, K, "pool K")
+    assert_bits_equal(gv, V, "pool V")
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -460,8 +530,8 @@ def test_manager_with_fp32_layers_and_beam_reorder(device):
 
 
 def test_decode_step_captured_into_a_graph(device):
-    """``KVCacheManager.capture_decode`` with fp32 layers: per layer an append launch (positions from the graph's
-    frozen lengths plus its device counter) and an attention launch, captured once, replayed per token."""
+    """``KVCacheManager.capture_decode`` with fp32 layers: per layer one launch (the append rides in the attention
+    launch), captured once, replayed per token."""
     from pace_mi355.llm import KVCacheManager, KVCacheType
     from pace_mi355.ops import MultiHeadAttention
 
