@@ -66,7 +66,7 @@ __device__ __forceinline__ void load_new_unit(UnitRegs<D>& r, const PagedAttnPar
   const u32x4 zero = {0u, 0u, 0u, 0u};
   // Every load is issued unconditionally from a clamped (valid) token row and masked afterwards:
   // without branches around them the loads all go out before the first wait.
-  u32x4 tab[ROPE ? 2 : 1][D / 32];
+  u32x4 tab[ROPE ? 2 : 1][kRopeTabRegs<D>];
   bool live[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -255,7 +255,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
 
   // Query rows of this wave (B operand of the first product) and per-row limits.
   u32x4 qreg[NQT][KK];
-  u32x4 qtab[ROPE ? NQT : 1][KK];  // cos / sin of the rows: fetched here, applied once the first unit is on its way
+  u32x4 qtab[ROPE ? NQT : 1][kRopeTabRegs<D>];  // cos / sin of the rows: fetched here, applied once the first unit is on its way
   RowState<D, NQT> st;
   int row_s[NQT], row_h[NQT];
   int min_limit = 0x7fffffff;
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(OCC, OC
         rope_fetch_row<D>(p.rope, tab_row[qt], g, qtab[qt]);
       } else {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
+        for (int kk = 0; kk < kRopeTabRegs<D>; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
   const int tile0 = (rg * NW + wave) * NQT;  // first query tile of this wave
 
   u32x4 qreg[NQT][KK];
-  u32x4 qtab[ROPE ? NQT : 1][KK];
+  u32x4 qtab[ROPE ? NQT : 1][kRopeTabRegs<D>];
   RowState<D, NQT> st;
   int row_s[NQT], row_h[NQT];
   int min_limit = 0x7fffffff;
@@ -521,7 +521,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         rope_fetch_row<D>(p.rope, tab_row[qt], g, qtab[qt]);
       } else {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
+        for (int kk = 0; kk < kRopeTabRegs<D>; ++kk) qtab[qt][kk] = u32x4{0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
@@ -861,10 +861,7 @@ static void launch(const PagedAttnParams& p, bool has_mask, hipStream_t s) {
     }                                                                                    \
   } while (0)
   if (p.rope.cos) {  // never together with an explicit mask (checked by the caller)
-    // (head sizes whose halves fall inside a 32-dim operand step have no in-register rotation: refused by the caller)
-    if constexpr (D % 64 == 0) {
-      if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
-    }
+    if (fused) PACE_GO(false, true, true); else PACE_GO(false, false, true);
   } else if (has_mask) {
     if constexpr (NQT <= 2) {  // shape_for() never asks for more tiles with a mask
       if (fused) PACE_GO(true, true, false); else PACE_GO(true, false, false);
@@ -1138,8 +1135,6 @@ static int run_paged_attn(const pace_kv_pool_t* pool, const pace_paged_attn_args
     if (int rc = make_rope_dev(a->rope, pool->head_dim, false, who, &rope_dev)) return rc;
     PACE_REQUIRE(rope_dev.rot == pool->head_dim, "%s: rotary_dim %d must equal head_dim %d when rope rides in the attention launch",
                  who, rope_dev.rot, pool->head_dim);
-    PACE_REQUIRE(pool->head_dim % 64 == 0, "%s: rope cannot ride in the attention launch with head_dim %d (rotate with pace_rope_* first)",
-                 who, pool->head_dim);
     PACE_REQUIRE(a->mask == nullptr, "%s: rope in the attention launch cannot be combined with an explicit mask", who);
     PACE_REQUIRE(!a->k_new || a->n_new == a->q_len, "%s: with rope, the fused append takes n_new == q_len (got %d, %d)", who,
                  a->n_new, a->q_len);

@@ -123,10 +123,39 @@ __device__ __forceinline__ void rope_rotate_chunks(const RopeDev& r, int row, in
 // quarter g).  Both members of every rotation pair sit in the same lane: dim d pairs with
 // d + D/2 (register kk + KK/2) or, interleaved, with its neighbour inside the 16 bytes.
 // Split in two so that the table loads can be issued early and consumed late.
+// A head size that is no multiple of 64 (96) paired by halves: the partner of dim d, d + D/2, falls into another
+// lane quarter -- dims 8g .. of quarter g pair with dims 32 + 8 (g + 2) .. of quarter g + 2, and so on round the
+// three registers -- so the quarters g and g ^ 2 (the lanes 32 apart, which hold the same row) exchange their
+// registers; every lane then rotates the three chunks it owns.  The table registers number 2 KK there (a cos and a
+// sin chunk per register of the row).
 template <int D>
-__device__ __forceinline__ void rope_fetch_row(const RopeDev& rope, int row, int g, u32x4 (&tab)[D / 32]) {
+constexpr int kRopeTabRegs = (D % 64 == 0) ? D / 32 : 2 * (D / 32);
+
+// Odd KK: the table column of register k of the row, and whether the register holds the lower member of its pairs.
+template <int D>
+__device__ __forceinline__ void rope_odd_chunk(int k, int g, int& col, bool& is_lo) {
+  const int dim = 32 * k + 8 * g;
+  is_lo = dim < D / 2;
+  col = is_lo ? dim : dim - D / 2;
+}
+
+template <int D>
+__device__ __forceinline__ void rope_fetch_row(const RopeDev& rope, int row, int g, u32x4 (&tab)[kRopeTabRegs<D>]) {
   constexpr int KK = D / 32;
   const int64_t base = (int64_t)row * (D / 2);
+  if constexpr (KK % 2 != 0) {
+    if (!rope.interleaved) {
+#pragma unroll
+      for (int k = 0; k < KK; ++k) {
+        int col;
+        bool is_lo;
+        rope_odd_chunk<D>(k, g, col, is_lo);
+        tab[2 * k] = rope_load8(rope.cos, rope.is_f32, base + col);
+        tab[2 * k + 1] = rope_load8(rope.sin, rope.is_f32, base + col);
+      }
+      return;
+    }
+  }
   if (!rope.interleaved) {
 #pragma unroll
     for (int kk = 0; kk < KK / 2; ++kk) {
@@ -145,8 +174,39 @@ __device__ __forceinline__ void rope_fetch_row(const RopeDev& rope, int row, int
 }
 
 template <int D>
-__device__ __forceinline__ void rope_apply_row(const RopeDev& rope, const u32x4 (&tab)[D / 32], u32x4 (&x)[D / 32]) {
+__device__ __forceinline__ void rope_apply_row(const RopeDev& rope, const u32x4 (&tab)[kRopeTabRegs<D>], u32x4 (&x)[D / 32]) {
   constexpr int KK = D / 32;
+  if constexpr (KK % 2 != 0) {
+    // every lane of the wave comes through here together (the exchange below reads the lane 32 away)
+    static_assert(KK == 3, "head size 96");
+    const int g = (threadIdx.x & 63) >> 4;
+    u32x4 y[KK];  // the registers of the lane 32 away: the same row, quarter g ^ 2
+#pragma unroll
+    for (int k = 0; k < KK; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[k][e] = (uint32_t)__shfl_xor((int)x[k][e], 32, 64);
+    if (!rope.interleaved) {
+      // partner of register k: k + 1 (mod 3) in the lower quarters, k + 2 (mod 3) in the upper ones
+      const bool upper = g >= 2;
+#pragma unroll
+      for (int k = 0; k < KK; ++k) {
+        int col;
+        bool is_lo;
+        rope_odd_chunk<D>(k, g, col, is_lo);
+        u32x4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t other = upper ? y[(k + 2) % KK][e] : y[(k + 1) % KK][e];
+          const uint32_t lo = is_lo ? x[k][e] : other, hi = is_lo ? other : x[k][e];
+          uint32_t a, b;
+          rope_pair2(lo, hi, tab[2 * k][e], tab[2 * k + 1][e], a, b);
+          out[e] = is_lo ? a : b;
+        }
+        x[k] = out;  // (the partners were read from y: nothing rotated is read again)
+      }
+      return;
+    }
+  }
   if (!rope.interleaved) {
 #pragma unroll
     for (int kk = 0; kk < KK / 2; ++kk) rope_rotate_halves(x[kk], x[kk + KK / 2], tab[2 * kk], tab[2 * kk + 1]);
@@ -159,7 +219,7 @@ __device__ __forceinline__ void rope_apply_row(const RopeDev& rope, const u32x4 
 
 template <int D>
 __device__ __forceinline__ void rotate_row_regs(const RopeDev& rope, int row, int g, u32x4 (&x)[D / 32]) {
-  u32x4 tab[D / 32];
+  u32x4 tab[kRopeTabRegs<D>];
   rope_fetch_row<D>(rope, row, g, tab);
   rope_apply_row<D>(rope, tab, x);
 }

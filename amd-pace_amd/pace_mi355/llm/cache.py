@@ -545,7 +545,7 @@ class PagedKVCache(KVCacheBase):
             if self.f32:
                 query, _ = rope(query, None)  # (the keys were rotated before their append)
                 qs = query.stride()
-            elif attention_mask is not None or rope_desc.rotary_dim != D or D % 64:
+            elif attention_mask is not None or rope_desc.rotary_dim != D:
                 # cases the attention launch does not fold in: rotate the queries (and a held-back append) first
                 self._flush()
                 query, _ = rope(query, None)

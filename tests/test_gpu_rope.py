@@ -252,10 +252,8 @@ def test_one_launch_step_rope_append_attention(device, D, neox, S):
         q_rot, k_rot = rope(qd, kd)
         kk2, vv2 = split.update_cache(k_rot, vd, 2)
         got2 = attn(q_rot, kk2, vv2)
-        if D % 64 == 0:
-            assert_bits_equal(got, got2, f"step {i}: fused launch vs separate launches")
-        else:  # no in-launch rotation for this head size: the first path appends before it attends, the second fuses the append
-            assert_attention_close(got2, want, f"step {i} separate launches")
+        # (head size 96 included: there the halves of a pair lie in lanes 32 apart, which exchange them in registers)
+        assert_bits_equal(got, got2, f"step {i}: fused launch vs separate launches")
         past += T
         kg, vg = fused.gather(n_rep=1)
         assert_bits_equal(kg, ref.key, f"pool K after step {i}")
