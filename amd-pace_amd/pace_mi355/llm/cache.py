@@ -277,8 +277,8 @@ class PagedKVCache(KVCacheBase):
         if v.shape != k.shape:
             raise RuntimeError("key_states and value_states differ in shape")
         if self.head_dim != self.model_dim:
-            if rope is not None:
-                raise NotImplementedError("rotary embedding with a zero-padded head size")
+            # (a rotary embedding then rotates the first rotary_dim <= model_dim dims of the padded rows, in a launch of
+            # its own: inside the attention launch it needs rotary_dim == the pool's head size)
             k, v = (torch.nn.functional.pad(t, (0, self.head_dim - self.model_dim)) for t in (k, v))
         if k.dtype != self.pool.dtype or v.dtype != self.pool.dtype:
             raise RuntimeError(f"the cache holds {self.pool.dtype}; got {k.dtype} / {v.dtype}")

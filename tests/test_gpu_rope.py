@@ -307,17 +307,33 @@ def test_longrope_rows_follow_the_reference_switch(device):
         assert_bits_equal(qo, rope_ref.rotate_longrope_form(q, cos, sin, 64), "longrope")
 
 
-def test_rope_with_a_zero_padded_head_size_is_refused(device):
-    """Head sizes the kernels are not built for are kept zero-padded by PagedKVCache; the rotation has no such
-    path and must say so instead of rotating padded rows."""
+@pytest.mark.parametrize("neox,rot", [(True, 80), (False, 80), (True, 64)])
+def test_rope_with_a_zero_padded_head_size(device, neox, rot):
+    """Head sizes the kernels are not built for (80: OPT-2.7B's) are kept zero-padded in slabs of the next built size;
+    the rotation then runs over the first rotary_dim dims of the padded rows in launches of its own (inside the
+    attention launch it takes rotary_dim == the pool's head size).  Pool contents bit-exact, attention within tolerance."""
     from pace_mi355.llm import PagedKVCache
+    from pace_mi355.ops import MultiHeadAttention
 
-    B, hkv, D, T = 2, 2, 80, 5
-    k, v = seeded_kv(1, B, hkv, T, D)
-    cache = PagedKVCache(64, num_kv_heads=hkv, n_rep=1)
-    mod = _module(64, rows=64)
-    rope = mod(k.to(device)[..., :64], torch.arange(T).repeat(B, 1).to(device))
-    with pytest.raises(NotImplementedError, match="zero-padded head size"):
-        cache.update_cache(k.to(device), v.to(device), 2, rope=rope)
-    pk, pv = cache.update_cache(k.to(device), v.to(device), 2)  # without rotation it is stored and read back as given
-    assert_bits_equal(pk.dense(), k, "K of head size 80")
+    B, hkv, n_rep, D = 2, 2, 2, 80
+    mod = _module(rot, rows=128)
+    cache = PagedKVCache(128, num_kv_heads=hkv, n_rep=n_rep)
+    ref = DynamicKVCacheRef(128)
+    attn = MultiHeadAttention()
+    past = 0
+    for i, T in enumerate([37, 1, 3, 1]):
+        k, v = seeded_kv(500 + i, B, hkv, T, D)
+        q = seeded_q(600 + i, B, hkv * n_rep, T, D)
+        pos = torch.arange(past, past + T).repeat(B, 1)
+        kd, vd, qd = k.to(device), v.to(device), q.to(device)
+        rope = mod(kd, pos.to(device)).with_style(neox)
+        want = _reference_step(q, k, v, mod, pos, ref, n_rep, neox)
+        kk, vv = cache.update_cache(kd, vd, 2, rope=rope)
+        assert cache.head_dim == 96 and cache.model_dim == 80
+        got = attn(qd, kk, vv)
+        assert got.shape == q.shape
+        assert_attention_close(got, want, f"step {i}")
+        past += T
+        kg, vg = cache.gather(n_rep=1)
+        assert_bits_equal(kg, ref.key, f"pool K after step {i}")
+        assert_bits_equal(vg, ref.value, f"pool V after step {i}")
