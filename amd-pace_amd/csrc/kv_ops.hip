@@ -213,6 +213,7 @@ struct GatherOut {
   int32_t zero_fill;          // dense: write zeros to rows in [len, out_len)
   int32_t batch;              // packed: sequences (cu_seqlens has batch + 1 entries)
   int32_t total_rows;         // packed: rows of the outputs
+  int32_t dense_rows;         // packed grid (one workgroup per block that exists), rows written in the dense layout
 };
 
 // Packed grid: which (sequence, head, logical block) workgroup `entry` stands for.
@@ -251,7 +252,8 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
   int64_t blk = table[(int64_t)b * table_stride + min(j, table_stride - 1)];
   const int t0 = j * PACE_KV_BLOCK_TOKENS;
   const bool live = t0 < len;  // uniform per workgroup
-  const int row_end = PACKED ? len : out.out_len;
+  const bool dense_rows = PACKED && out.dense_rows != 0;  // the dense layout from the packed grid
+  const int row_end = PACKED ? (dense_rows ? min(len, out.out_len) : len) : out.out_len;
   if (!live && (PACKED || !out.zero_fill || t0 >= row_end)) return;  // nothing to write
   blk = blk < 0 ? 0 : (blk >= pool.num_blocks ? pool.num_blocks - 1 : blk);  // never read outside the pool
   const uint16_t* ksrc = reinterpret_cast<const uint16_t*>(pool.k) + blk * pool.k_block_stride + h * pool.k_head_stride;
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
     }
   }
   __syncthreads();
-  const int64_t base = PACKED ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
+  const int64_t base = (PACKED && !dense_rows) ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int c = threadIdx.x + i * 256;
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(pace_kv_pool_t pool, con
     const int tok = c / CHUNKS, chunk = c % CHUNKS;
     const int t = t0 + tok;
     if (t >= row_end) continue;
-    if (PACKED && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
+    if (PACKED && !dense_rows && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
     u32x4 vv = {0u, 0u, 0u, 0u};
     if (t < len) {
 #pragma unroll
@@ -311,7 +313,8 @@ __global__ __launch_bounds__(256) void kv_gather_f32_kernel(pace_kv_pool_t pool,
   int64_t blk = table[(int64_t)b * table_stride + min(j, table_stride - 1)];
   const int t0 = j * PACE_KV_BLOCK_TOKENS;
   const bool live = t0 < len;  // uniform per workgroup
-  const int row_end = PACKED ? len : out.out_len;
+  const bool dense_rows = PACKED && out.dense_rows != 0;  // the dense layout from the packed grid
+  const int row_end = PACKED ? (dense_rows ? min(len, out.out_len) : len) : out.out_len;
   if (!live && (PACKED || !out.zero_fill || t0 >= row_end)) return;  // nothing to write
   blk = blk < 0 ? 0 : (blk >= pool.num_blocks ? pool.num_blocks - 1 : blk);  // never read outside the pool
   const int D = pool.head_dim, chunks = D / 4;
@@ -319,12 +322,12 @@ __global__ __launch_bounds__(256) void kv_gather_f32_kernel(pace_kv_pool_t pool,
   const float* vsrc = static_cast<const float*>(pool.v) + blk * pool.v_block_stride + h * pool.v_head_stride;
   float* ko = reinterpret_cast<float*>(out.k);
   float* vo = reinterpret_cast<float*>(out.v);
-  const int64_t base = PACKED ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
+  const int64_t base = (PACKED && !dense_rows) ? (int64_t)out.cu_seqlens[b] * out.stride_t : (int64_t)b * out.stride_b;
   for (int c = threadIdx.x; c < PACE_KV_BLOCK_TOKENS * chunks; c += 256) {
     const int tok = c / chunks, chunk = c % chunks;
     const int t = t0 + tok;
     if (t >= row_end) continue;
-    if (PACKED && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
+    if (PACKED && !dense_rows && out.cu_seqlens[b] + t >= out.total_rows) continue;  // never write past the outputs
     u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
     if (t < len) {
       kk = load16_stream(ksrc + c * 4), vv = load16_stream(vsrc + c * 4);
@@ -548,8 +551,22 @@ extern "C" int pace_kv_gather(const pace_kv_pool_t* pool, const int32_t* block_t
                               int64_t out_stride_b, int64_t out_stride_h, int32_t out_len, int32_t zero_fill, void* stream) {
   PACE_REQUIRE(pool != nullptr, "pace_kv_gather: pool is NULL");
   GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), nullptr, out_stride_b, out_stride_h,
-                   pool->head_dim, out_len, zero_fill ? 1 : 0, batch, 0};
+                   pool->head_dim, out_len, zero_fill ? 1 : 0, batch, 0, 0};
   return run_gather("pace_kv_gather", pool, block_table, table_stride, seq_lens, seq_len_bias, batch, n_rep, out_len, out, false,
+                    stream);
+}
+
+extern "C" int pace_kv_gather_live(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                                   const int32_t* seq_lens, int32_t seq_len_bias, const int32_t* cu_seqlens, int32_t batch,
+                                   int32_t n_rep, void* k_out, void* v_out, int64_t out_stride_b, int64_t out_stride_h,
+                                   int32_t out_len, int32_t total_tokens, void* stream) {
+  PACE_REQUIRE(pool != nullptr, "pace_kv_gather_live: pool is NULL");
+  if (batch > 0 && total_tokens > 0) PACE_REQUIRE(cu_seqlens != nullptr, "pace_kv_gather_live: cu_seqlens is NULL");
+  PACE_REQUIRE(out_len >= 0 && total_tokens >= 0, "pace_kv_gather_live: negative out_len (%d) or total_tokens (%d)", out_len, total_tokens);
+  if (out_len == 0) return PACE_KV_OK;
+  GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), cu_seqlens, out_stride_b, out_stride_h,
+                   pool->head_dim, out_len, 0, batch, total_tokens, 1};
+  return run_gather("pace_kv_gather_live", pool, block_table, table_stride, seq_lens, seq_len_bias, batch, n_rep, total_tokens, out, true,
                     stream);
 }
 
@@ -560,7 +577,7 @@ extern "C" int pace_kv_gather_packed(const pace_kv_pool_t* pool, const int32_t* 
   if (batch > 0 && total_tokens > 0) PACE_REQUIRE(cu_seqlens != nullptr, "pace_kv_gather_packed: cu_seqlens is NULL");
   PACE_REQUIRE(n_rep >= 1, "pace_kv_gather_packed: bad n_rep (%d)", n_rep);
   const int64_t row = (int64_t)pool->num_kv_heads * n_rep * pool->head_dim;  // one token, every output head
-  GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), cu_seqlens, 0, pool->head_dim, row, 0, 0, batch, total_tokens};
+  GatherOut out = {static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(v_out), cu_seqlens, 0, pool->head_dim, row, 0, 0, batch, total_tokens, 0};
   return run_gather("pace_kv_gather_packed", pool, block_table, table_stride, seq_lens, seq_len_bias, batch, n_rep, total_tokens,
                     out, true, stream);
 }

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "pace_kv_append_paged_at",
     "pace_kv_gather",
     "pace_kv_gather_packed",
+    "pace_kv_gather_live",
     "pace_kv_copy_blocks",
     "pace_rope_apply",
     "pace_rope_apply_f32",
@@ -190,6 +191,10 @@ def load() -> ctypes.CDLL:
     lib.pace_kv_gather_packed.restype = ctypes.c_int
     lib.pace_kv_gather_packed.argtypes = [
         P, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_void_p,
+    ]
+    lib.pace_kv_gather_live.restype = ctypes.c_int
+    lib.pace_kv_gather_live.argtypes = [
+        P, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p,
     ]
     lib.pace_kv_copy_blocks.restype = ctypes.c_int
     lib.pace_kv_copy_blocks.argtypes = [P, P, c_void_p, c_int32, c_void_p]

@@ -475,12 +475,26 @@ class PagedKVCache(KVCacheBase):
         if L:
             st = self.state
             table, (lens_dev, bias) = st.device_table(), st.device_lens(self.lens)
-            nat.check(
-                nat.load().pace_kv_gather(
-                    ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, self.batch, n_rep,
-                    k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, 1 if zero_fill else 0, nat.current_stream_ptr(),
+            total = int(self.lens.sum())
+            if not zero_fill and 0 < total < 1 << 31:
+                # nothing to write past the lengths: one workgroup per block that exists (in a ragged batch most of
+                # the [B, L] row range is padding)
+                cu = np.zeros(self.batch + 1, dtype=np.int64)
+                np.cumsum(self.lens, out=cu[1:])
+                cu_dev = torch.from_numpy(cu.astype(np.int32)).pin_memory().to(self.pool.device, non_blocking=True)
+                nat.check(
+                    nat.load().pace_kv_gather_live(
+                        ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, cu_dev.data_ptr(),
+                        self.batch, n_rep, k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, total, nat.current_stream_ptr(),
+                    )
                 )
-            )
+            elif zero_fill or total:
+                nat.check(
+                    nat.load().pace_kv_gather(
+                        ctypes.byref(self._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, self.batch, n_rep,
+                        k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, 1 if zero_fill else 0, nat.current_stream_ptr(),
+                    )
+                )
         if padded:
             k, v = k[..., : self.model_dim].contiguous(), v[..., : self.model_dim].contiguous()
         return k, v

@@ -345,7 +345,7 @@ def wl_ragged(torch, dev, args):
     forms = {}
     for form in ("packed", "dense", "dense_zero_fill"):
         fn = gather_call(torch, cache, form)
-        forms[form] = roofline(f"kv_gather_kernel<128,{'true' if form == 'packed' else 'false'}> ({form.replace('_', ' ')})", gather_b,
+        forms[form] = roofline(f"kv_gather_kernel<128,{'false' if form == 'dense_zero_fill' else 'true'}> ({form.replace('_', ' ')})", gather_b,
                                time_call(torch, fn, reps=5, warmup=1))
     check = {} if args.no_check else self_check(torch, step, spread_rows(lens1))
     return result_line(
@@ -378,11 +378,20 @@ def gather_call(torch, cache, form):
                                                 cu_dev.data_ptr(), B, 1, k.data_ptr(), v.data_ptr(), int(cu[-1]), nat.current_stream_ptr()))
         return fn
     k, v = (torch.empty(B, H, L, D, dtype=torch.bfloat16, device=dev) for _ in range(2))
-    zero = 1 if form == "dense_zero_fill" else 0
+    if form == "dense":  # rows past each length left alone: launched over the blocks that exist, like the packed form
+        cu = np.zeros(B + 1, dtype=np.int64)
+        np.cumsum(cache.lens, out=cu[1:])
+        cu_dev = torch.from_numpy(cu.astype(np.int32)).to(dev)
+
+        def fn(_keep=(cu_dev, k, v, table, lens_dev)):
+            nat.check(lib.pace_kv_gather_live(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias,
+                                              cu_dev.data_ptr(), B, 1, k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, int(cu[-1]),
+                                              nat.current_stream_ptr()))
+        return fn
 
     def fn(_keep=(k, v, table, lens_dev)):
         nat.check(lib.pace_kv_gather(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias, B, 1,
-                                     k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, zero, nat.current_stream_ptr()))
+                                     k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), L, 1, nat.current_stream_ptr()))
     return fn
 
 

@@ -158,6 +158,17 @@ int pace_kv_gather_packed(const pace_kv_pool_t* pool, const int32_t* block_table
                           void* stream);
 
 /*
+ * The dense form of pace_kv_gather without zero fill (rows past each length are left untouched), launched like the
+ * packed form: one workgroup per block that exists, found through cu_seqlens (device int32 [batch + 1], the running
+ * sum of the lengths, total_tokens = its last entry).  In a ragged batch most of a dense [out_len] row range lies
+ * past the lengths; this launch starts no workgroup for it.
+ */
+int pace_kv_gather_live(const pace_kv_pool_t* pool, const int32_t* block_table, int32_t table_stride,
+                        const int32_t* seq_lens, int32_t seq_len_bias, const int32_t* cu_seqlens, int32_t batch,
+                        int32_t n_rep, void* k_out, void* v_out, int64_t out_stride_b, int64_t out_stride_h,
+                        int32_t out_len, int32_t total_tokens, void* stream);
+
+/*
  * Copy whole blocks (compaction, beam copy-on-write; the reference's only cache
  * copy of this kind is index_select, pace/llm/cache.py:161-167).
  * pairs: device int32 [n_pairs][2] = (src block, dst block).  When src and dst
