@@ -149,6 +149,39 @@ def test_gather_without_zero_fill_leaves_padding_untouched(device):
         assert bool((o[0, :, 30:] == 3.0).all()) and bool((o[1, :, 5:] == 3.0).all()), "padding rows were written"
 
 
+@pytest.mark.parametrize("out_len", [40, 12])
+def test_gather_over_the_blocks_that_exist_writes_only_rows_that_exist(device, out_len):
+    """pace_kv_gather_live: the dense layout written from the grid of the packed form.  Rows below
+    min(len, out_len) bit-exact; padding rows, rows of an empty sequence and the memory behind the
+    outputs untouched -- also when out_len cuts a sequence short."""
+    import ctypes
+
+    from pace_mi355 import _native as nat
+
+    B, H, D, rep = 4, 2, 128, 2
+    lens = [30, 0, 5, 17]
+    cache = _paged(64)
+    k, v = seeded_kv(3, B, H, max(lens), D)
+    cache.append_ragged(k.to(device), v.to(device), lens)
+    st = cache.state
+    table, (lens_dev, bias) = st.device_table(), st.device_lens(cache.lens)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=device)
+    guard = 3 * D
+    flat = [torch.full((B * H * rep * out_len * D + guard,), 3.0, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    outs = [f[: B * H * rep * out_len * D].view(B, H * rep, out_len, D) for f in flat]
+    nat.check(nat.load().pace_kv_gather_live(ctypes.byref(cache._desc), table.data_ptr(), table.stride(0), lens_dev.data_ptr(), bias,
+                                             cu.data_ptr(), B, rep, outs[0].data_ptr(), outs[1].data_ptr(), outs[0].stride(0),
+                                             outs[0].stride(1), out_len, sum(lens), nat.current_stream_ptr()))
+    torch.cuda.synchronize()
+    for f, o, src in zip(flat, outs, (k, v)):
+        want = src.repeat_interleave(rep, dim=1)
+        for b, n in enumerate(lens):
+            m = min(n, out_len)
+            assert_bits_equal(o[b, :, :m], want[b, :, :m], f"rows of sequence {b}")
+            assert bool((o[b, :, m:] == 3.0).all()), f"rows past the end of sequence {b} were written"
+        assert bool((f[-guard:] == 3.0).all()), "memory behind the outputs was written"
+
+
 def test_beam_reorder(device):
     B, H, D = 4, 2, 64
     cache = _paged(128, num_blocks=80)
